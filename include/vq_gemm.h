@@ -1,0 +1,99 @@
+/*
+ * vq_gemm.h — C ABI of the MI355X (gfx950) vector-quantized GEMM library, libvqgemm.so.
+ *
+ * Every pointer is a device pointer (HIP, current device) unless stated otherwise; all
+ * matrices are dense row-major; `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  Calls only enqueue work; they do not synchronise.  Return value:
+ * 0 on success, a negative VQGEMM_E_* code for rejected arguments (nothing was launched),
+ * a positive hipError_t when the runtime refused the launch.
+ *
+ * Two data geometries are served.
+ *   Geometry B (K-axis vectors):  Y[M,N] = X[M,K] . W^T,
+ *       W[n, j*vec + t] = codebook[n / (N/n_codebooks)][codes[n, j]][t],
+ *       codes [N, K/vec] uint8 or uint16, codebook [n_codebooks, entries, vec] fp16.
+ *   Geometry A (the reference's native layout, bench.py:83-85 of the reference):
+ *       out[M, 2*Nc] = X[M,K] . W_dec,  W_dec[k, 2n + r] = codebook[n/4][w[k,n]][r],
+ *       w [K, Nc] uint8, codebook [Nc/4, 256, 2] fp16.
+ * Products accumulate in fp32 and are rounded once to fp16.
+ */
+#ifndef VQ_GEMM_H
+#define VQ_GEMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* argument errors */
+#define VQGEMM_OK 0
+#define VQGEMM_E_NULL (-1)      /* a required pointer is NULL */
+#define VQGEMM_E_SHAPE (-2)     /* negative size, K % vec != 0, N % n_codebooks != 0, ... */
+#define VQGEMM_E_CODEBITS (-3)  /* code_bits not 8/16, or entries > 2^code_bits */
+#define VQGEMM_E_VARIANT (-4)   /* unknown variant, or the variant cannot serve this shape */
+#define VQGEMM_E_ALIGN (-5)     /* a pointer is not aligned to its element size */
+
+/* kernel selection for the fused GEMM */
+#define VQGEMM_VARIANT_AUTO 0     /* pick by shape */
+#define VQGEMM_VARIANT_GENERIC 1  /* simple scalar kernel, any shape */
+#define VQGEMM_VARIANT_DECODE 2   /* M <= 16: K-sliced waves, 16x16x32 MFMA, LDS-resident codebook */
+#define VQGEMM_VARIANT_PREFILL 3  /* large M: 32x32x16 MFMA tiles, codewords gathered into operands */
+#define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */
+
+/*
+ * Fused VQ GEMM, geometry B.
+ * Replaces: torch::Tensor e2e_gemm(input, w, codebook) — reference bind.cpp:3,7 and the host
+ * wrappers strategy_2/bsz128/src.cu:255-316 (and the four sibling copies) — for the K-axis
+ * layout the measured configurations use.
+ * `workspace` is only read by VQGEMM_VARIANT_TWOPASS (N*K fp16 scratch); NULL otherwise.
+ */
+int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, void *y,
+                      int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                      int32_t n_codebooks, int32_t code_bits, int32_t variant,
+                      void *workspace, void *stream);
+
+/*
+ * Fused VQ GEMM, geometry A (reference-native tensors, same entry point of the reference:
+ * bind.cpp:3,7; indexing per strategy_2/bsz512/src.cu:163-176 and bench.py:46-56).
+ * out is [M, 2*Nc].  `workspace` as above (K*2*Nc fp16 for TWOPASS).
+ */
+int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *out,
+                      int64_t M, int64_t K, int64_t Nc, int32_t variant,
+                      void *workspace, void *stream);
+
+/*
+ * Stand-alone dequantisation to fp16 in HBM.
+ * Replaces: dequant_kernel + the intermediate B tensor of the two-pass strategy,
+ * reference strategy_1/src.cu:268-321,351.
+ * geometry B writes W[N,K]; geometry A writes W_dec[K, 2*Nc].
+ */
+int vqgemm_dequant_b(const void *codes, const void *codebook, void *w_out,
+                     int64_t N, int64_t K, int32_t vec, int32_t entries,
+                     int32_t n_codebooks, int32_t code_bits, void *stream);
+int vqgemm_dequant_a(const void *w, const void *codebook, void *w_out,
+                     int64_t K, int64_t Nc, void *stream);
+
+/*
+ * Plain fp16 GEMM o[M,N] = input[M,K] . w[K,N] (fp32 accumulate), the no-dequant control.
+ * Replaces: torch::Tensor gemm(input, w) — reference bind.cpp:4,8, strategy_1/src.cu:171-265.
+ */
+int vqgemm_gemm_f16(const void *x, const void *w, void *y, int64_t M, int64_t K, int64_t N,
+                    void *stream);
+
+/*
+ * Which kernel VQGEMM_VARIANT_AUTO resolves to for a geometry-B shape (host only, no GPU
+ * call): returns a VQGEMM_VARIANT_* value, or a negative error for an invalid shape.
+ */
+int vqgemm_select_variant_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                            int32_t n_codebooks, int32_t code_bits);
+
+/* Host string for a return code of this library (static storage). */
+const char *vqgemm_error_string(int code);
+
+/* Library version: major*10000 + minor*100 + patch. */
+int vqgemm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VQ_GEMM_H */

@@ -1,0 +1,134 @@
+"""CPU oracle for the vector-quantized GEMM path.  TEST INFRASTRUCTURE ONLY.
+
+This module is the checker, never the product: only tests, the smoke check and the
+bench's CPU-baseline leg may import it.  The shipped path is the HIP library; nothing
+in the package falls back to this code.
+
+It restates, in numpy, the mathematics of the reference's harness oracle
+(`bench.py:37-57`: advanced-index gather from the codebook, reshape, matmul) in the two
+data geometries the library serves:
+
+* geometry A — the reference's native layout (`bench.py:83-85`):
+  codes `w[K, Nc]` uint8, codebook `[Nc/4, 256, 2]` fp16,
+  `W_dec[k, n*2 + r] = codebook[n // 4, w[k, n], r]`, `out[M, 2*Nc] = X @ W_dec`.
+* geometry B — weights `W[N, K]` encoded along K with vector length `v`:
+  codes `[N, K/v]` uint8/uint16, codebook `[E, v]` or `[G, E, v]` (one codebook per
+  `N/G` consecutive output rows),
+  `W[n, j*v + t] = codebook[n // (N/G)][codes[n, j]][t]`, `Y[M, N] = X @ W.T`.
+
+The reference accumulates in fp16 (`strategy_1/src.cu:131`,
+`ref_gemm/cublas_gemm_fp16.cu:45`); the contract here is fp32 accumulation rounded once
+to fp16, so the GEMM functions accumulate in fp32 (and optionally fp64, which bounds the
+oracle's own rounding).
+
+Pinning status (no golden vectors exist in the reference; see tests/test_oracle.py):
+  dequant_a, dequant_b  — pinned bit-exactly: hand-written known-answer cases,
+                          brute-force triple loops, the C restatement, torch advanced
+                          indexing written the way `bench.py:46-55` writes it.
+  vq_gemm_a, vq_gemm_b, gemm — pinned: integer-valued known answers computed by hand,
+                          one-hot identities, fp64 cross-accumulation, the C restatement.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+CODEBOOKS_PER_GROUP_A = 4  # reference: one codebook per 4 code columns (bench.py:40)
+
+
+def _as_cb3(codebook: np.ndarray) -> np.ndarray:
+    cb = np.asarray(codebook)
+    if cb.ndim == 2:
+        cb = cb[None]
+    if cb.ndim != 3:
+        raise ValueError("codebook must be [E,v] or [G,E,v]")
+    return cb
+
+
+def dequant_b(codes: np.ndarray, codebook: np.ndarray) -> np.ndarray:
+    """Geometry B dequantisation: returns W[N, K] with the codebook's dtype.
+
+    W[n, j*v + t] = codebook[n // (N/G)][codes[n, j]][t]   (pure indexing, bit-exact).
+    """
+    codes = np.asarray(codes)
+    cb = _as_cb3(codebook)
+    G, E, v = cb.shape
+    N, J = codes.shape
+    if N % G != 0:
+        raise ValueError("N must be a multiple of the number of codebooks")
+    idx = codes.astype(np.int64)
+    if idx.size and (idx.min() < 0 or idx.max() >= E):
+        raise ValueError("code out of range")
+    g = (np.arange(N, dtype=np.int64) // (N // G))[:, None]        # [N,1]
+    w = cb[g, idx]                                                  # [N,J,v]
+    return np.ascontiguousarray(w.reshape(N, J * v))
+
+
+def dequant_a(w: np.ndarray, codebook: np.ndarray) -> np.ndarray:
+    """Geometry A dequantisation (`bench.py:37-55`): returns W_dec[K, Nc*ratio].
+
+    W_dec[k, n*ratio + r] = codebook[n // 4, w[k, n], r].
+    """
+    w = np.asarray(w)
+    cb = np.asarray(codebook)
+    if cb.ndim != 3:
+        raise ValueError("geometry A codebook must be [Nc/4, E, ratio]")
+    K, Nc = w.shape
+    if Nc % CODEBOOKS_PER_GROUP_A != 0 or cb.shape[0] * CODEBOOKS_PER_GROUP_A != Nc:
+        raise ValueError("geometry A needs codebook.shape[0]*4 == code columns")
+    idx = w.astype(np.int64)
+    if idx.size and idx.max() >= cb.shape[1]:
+        raise ValueError("code out of range")
+    row = (np.arange(Nc, dtype=np.int64) // CODEBOOKS_PER_GROUP_A)[None, :]  # [1,Nc]
+    dec = cb[np.broadcast_to(row, (K, Nc)), idx]                    # [K,Nc,ratio]
+    return np.ascontiguousarray(dec.reshape(K, Nc * cb.shape[2]))
+
+
+def _matmul(x: np.ndarray, wt: np.ndarray, acc) -> np.ndarray:
+    # x [M,K], wt [K,N]; accumulate in `acc`, round once to fp16.
+    return (x.astype(acc) @ wt.astype(acc)).astype(np.float16)
+
+
+def vq_gemm_b(x, codes, codebook, acc=np.float32) -> np.ndarray:
+    """Y[M,N] = X[M,K] @ dequant_b(codes, codebook).T, accumulated in `acc`, fp16 out."""
+    w = dequant_b(codes, codebook)
+    x = np.asarray(x)
+    if x.shape[1] != w.shape[1]:
+        raise ValueError("K mismatch")
+    return _matmul(x, w.T, acc)
+
+
+def vq_gemm_a(x, w, codebook, acc=np.float32) -> np.ndarray:
+    """out[M, 2*Nc] = X[M,K] @ dequant_a(w, codebook)  (`bench.py:55-56`)."""
+    dec = dequant_a(w, codebook)
+    x = np.asarray(x)
+    if x.shape[1] != dec.shape[0]:
+        raise ValueError("K mismatch")
+    return _matmul(x, dec, acc)
+
+
+def gemm(x, w, acc=np.float32) -> np.ndarray:
+    """Plain control GEMM `o[M,N] = input[M,K] @ w[K,N]` (`ref_gemm/cublas_gemm_fp16.cu:36-46`)."""
+    x = np.asarray(x)
+    w = np.asarray(w)
+    if x.shape[1] != w.shape[0]:
+        raise ValueError("K mismatch")
+    return _matmul(x, w, acc)
+
+
+def rel_err(y: np.ndarray, ref: np.ndarray, floor_frac: float = 1e-2):
+    """Error figures used by every GEMM parity check.
+
+    Returns (max |y-ref| / max(|ref|, tau), max|y-ref| / max|ref|) with
+    tau = floor_frac * rms(ref): outputs near zero would otherwise make the
+    per-element relative error unbounded whatever the accumulation precision.
+    """
+    y = np.asarray(y, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    if ref.size == 0:
+        return 0.0, 0.0
+    diff = np.abs(y - ref)
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    tau = max(floor_frac * rms, 1e-30)
+    e1 = float(np.max(diff / np.maximum(np.abs(ref), tau)))
+    e2 = float(np.max(diff) / max(float(np.max(np.abs(ref))), 1e-30))
+    return e1, e2

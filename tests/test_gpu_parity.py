@@ -1,0 +1,327 @@
+"""GPU parity tests: every kernel of libvqgemm.so, driven through the C ABI, against the CPU
+oracle on identical seeded inputs.
+
+Bars: dequantised weights bit-exact; GEMM outputs max |y-ref| / max(|ref|, tau) <= 2e-3 with
+tau = 1e-2 * rms(ref), against an fp64-accumulated oracle (the fp32 oracle itself sits
+within ~5e-4 of it; fp16 output rounding alone is <= 4.9e-4).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import vq_oracle as vo
+from vq_gemm_amd import cabi
+from vq_gemm_amd.problems import CONFIGS, GEOM_A, GEOM_B, ProblemSpec, make_problem
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+DEV = "cuda:0"
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _np(t):
+    return t.detach().cpu().numpy()
+
+
+def _check_gemm(y_gpu, x, codes, cb, geometry=GEOM_B, what=""):
+    if geometry == GEOM_B:
+        ref = vo.vq_gemm_b(_np(x), _np(codes), _np(cb), acc=np.float64)
+    else:
+        ref = vo.vq_gemm_a(_np(x), _np(codes), _np(cb), acc=np.float64)
+    e1, e2 = vo.rel_err(_np(y_gpu), ref)
+    _say(f"  {what}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+    assert e1 <= TOL, (what, e1, e2)
+    return e1
+
+
+SMALL_B = [
+    # name, M, K, N, vec, E, G, bits
+    ("tiny_v8", 1, 512, 16, 8, 256, 1, 8),
+    ("tiny_v4", 16, 1024, 64, 4, 256, 1, 8),
+    ("m7_n_ragged", 7, 1024, 50, 8, 256, 1, 8),
+    ("k_tail_v8", 3, 640, 32, 8, 256, 1, 8),          # K not a multiple of the 512 wave slice
+    ("u16_v4", 16, 512, 48, 4, 4096, 1, 16),
+    ("u16_v8", 5, 1024, 32, 8, 1000, 1, 16),
+    ("u8_v2", 4, 256, 32, 2, 256, 1, 8),
+    ("u16_v2", 2, 128, 16, 2, 300, 1, 16),
+    ("multi_cb16", 9, 512, 64, 8, 256, 4, 8),          # 16 rows per codebook
+    ("multi_cb128", 33, 512, 256, 8, 256, 2, 8),
+    ("m300_ragged", 300, 384, 200, 8, 256, 1, 8),       # prefill kernel with ragged M, N and a K tail
+    ("m64_v4", 64, 256, 96, 4, 256, 3, 8),
+    ("deep_k", 2, 9216, 32, 8, 256, 1, 8),              # more K than one workgroup's waves cover at once
+]
+
+
+def _spec(row):
+    name, M, K, N, v, E, G, bits = row
+    return ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+
+
+@pytest.mark.parametrize("row", SMALL_B, ids=[r[0] for r in SMALL_B])
+def test_dequant_b_bit_exact(row):
+    spec = _spec(row)
+    _say("dequant_b", spec)
+    _, codes, cb = make_problem(spec, seed=1, device=DEV)
+    w = cabi.dequant_b(codes, cb)
+    torch.cuda.synchronize()
+    want = vo.dequant_b(_np(codes), _np(cb))
+    assert np.array_equal(_np(w).view(np.uint16), want.view(np.uint16))
+    assert np.array_equal(want.view(np.uint16), c_oracle.dequant_b(_np(codes), _np(cb)).view(np.uint16))
+
+
+@pytest.mark.parametrize("row", SMALL_B, ids=[r[0] for r in SMALL_B])
+def test_e2e_gemm_b_all_variants(row):
+    spec = _spec(row)
+    x, codes, cb = make_problem(spec, seed=2, device=DEV)
+    auto = cabi.select_variant_b(spec.M, spec.K, spec.N, spec.vec, spec.entries, spec.n_codebooks, spec.code_bits)
+    _say("e2e_gemm_b", spec, "auto ->", cabi.VARIANT_NAMES[auto])
+    ran = []
+    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL,
+                    cabi.VARIANT_TWOPASS):
+        _say("  variant", cabi.VARIANT_NAMES[variant])
+        try:
+            y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
+        except cabi.VqGemmError as e:
+            assert e.code == -4, e          # "variant cannot serve this shape" is the only accepted refusal
+            assert variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL)
+            continue
+        torch.cuda.synchronize()
+        _check_gemm(y, x, codes, cb, what=f"{spec.name}/{cabi.VARIANT_NAMES[variant]}")
+        ran.append(variant)
+    assert cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran and cabi.VARIANT_TWOPASS in ran
+    if spec.M <= 16 and spec.vec in (2, 4, 8):
+        assert cabi.VARIANT_DECODE in ran
+
+
+@pytest.mark.parametrize("variant", [cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_GENERIC])
+@pytest.mark.parametrize("vec,bits,E", [(8, 8, 256), (4, 16, 4096), (4, 8, 256), (8, 16, 512)])
+def test_one_hot_activations_return_weight_columns_bit_exactly(variant, vec, bits, E):
+    """X = rows of the identity: Y[m,:] must equal W[:,m] exactly (1.0*w + zeros is exact), which
+    checks the gather, the MFMA operand layout and the K permutation through the real kernels."""
+    K, N, G = 1024, 96, 2
+    spec = ProblemSpec("onehot", GEOM_B, 16, K, N, vec, E, G, bits, codebook_3d=True)
+    _, codes, cb = make_problem(spec, seed=3, device=DEV)
+    w = vo.dequant_b(_np(codes), _np(cb))
+    for k0 in (0, 496, K - 16):
+        _say("one-hot", cabi.VARIANT_NAMES[variant], vec, bits, "k0", k0)
+        x = torch.zeros(16, K, dtype=torch.float16, device=DEV)
+        x[torch.arange(16), k0 + torch.arange(16)] = 1.0
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(_np(y).view(np.uint16), w[:, k0:k0 + 16].T.copy().view(np.uint16))
+
+
+def test_every_m_from_1_to_16_on_the_decode_kernel():
+    K, N = 1024, 80
+    for M in range(1, 17):
+        spec = ProblemSpec("m", GEOM_B, M, K, N, 8, 256, 1, 8)
+        x, codes, cb = make_problem(spec, seed=10 + M, device=DEV)
+        _say("decode M =", M)
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
+        torch.cuda.synchronize()
+        _check_gemm(y, x, codes, cb, what=f"M={M}")
+
+
+def test_properties_constant_codes_zero_codebook_scaling():
+    spec = ProblemSpec("prop", GEOM_B, 16, 1024, 128, 8, 256, 1, 8)
+    x, codes, cb = make_problem(spec, seed=4, device=DEV)
+    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL):
+        _say("properties", cabi.VARIANT_NAMES[variant])
+        const = torch.full_like(codes, 37)
+        y = cabi.e2e_gemm_b(x, const, cb, variant=variant)
+        assert torch.equal(y, y[:, :1].expand_as(y))            # all W rows identical
+        z = cabi.e2e_gemm_b(x, codes, torch.zeros_like(cb), variant=variant)
+        assert not z.any()
+        y1 = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
+        y4 = cabi.e2e_gemm_b(x * 4, codes, cb, variant=variant)
+        assert torch.equal(y4, (y1.float() * 4).half())          # power-of-two scaling is exact
+        # G identical codebooks == one codebook
+        cb4 = cb.unsqueeze(0).repeat(4, 1, 1).contiguous()
+        assert torch.equal(cabi.e2e_gemm_b(x, codes, cb4, variant=variant), y1)
+        # run-to-run determinism (the reference harness's own check, bench.py:118-132)
+        for _ in range(4):
+            assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=variant), y1)
+
+
+def test_empty_problems_and_rejections_on_device():
+    cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
+    x0 = torch.zeros(0, 64, dtype=torch.float16, device=DEV)
+    codes = torch.zeros(16, 8, dtype=torch.uint8, device=DEV)
+    assert cabi.e2e_gemm_b(x0, codes, cb).shape == (0, 16)
+    x = torch.randn(2, 64, device=DEV).half()
+    assert cabi.e2e_gemm_b(x, codes[:0], cb).shape == (2, 0)
+    with pytest.raises(cabi.VqGemmError) as ei:   # prefill kernel explicitly requested with a misaligned x
+        buf = torch.zeros(2 * 64 + 8, dtype=torch.float16, device=DEV)
+        xm = buf[1:1 + 128].view(2, 64)
+        cabi.e2e_gemm_b(xm, codes, cb, variant=cabi.VARIANT_PREFILL)
+    assert ei.value.code == -5
+    # ... while the automatic choice serves the same misaligned tensor with the generic kernel
+    xm.copy_(x)
+    y = cabi.e2e_gemm_b(xm, codes, cb)
+    torch.cuda.synchronize()
+    _check_gemm(y, xm, codes, cb, what="misaligned x")
+
+
+# ------------------------------------------------------------------ geometry A (reference-native tensors)
+@pytest.mark.parametrize("M,K,Nc", [(32, 256, 64), (5, 96, 8), (130, 512, 132)])
+def test_geometry_a(M, K, Nc):
+    spec = ProblemSpec("A", GEOM_A, M, K, 2 * Nc, 2, 256, Nc // 4, 8, codebook_std=1.0)
+    x, w, cb = make_problem(spec, seed=5, device=DEV)
+    _say("geometry A", M, K, Nc)
+    dec = cabi.dequant_a(w, cb)
+    torch.cuda.synchronize()
+    want = vo.dequant_a(_np(w), _np(cb))
+    assert np.array_equal(_np(dec).view(np.uint16), want.view(np.uint16))
+    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_TWOPASS):
+        y = cabi.e2e_gemm_a(x, w, cb, variant=variant)
+        torch.cuda.synchronize()
+        _check_gemm(y, x, w, cb, geometry=GEOM_A, what=f"A/{cabi.VARIANT_NAMES[variant]}")
+
+
+# ------------------------------------------------------------------ plain GEMM control and the hipBLASLt baseline
+@pytest.mark.parametrize("M,K,N", [(128, 128, 128), (33, 72, 50), (257, 1024, 384), (1, 64, 8)])
+def test_plain_gemm_and_hipblaslt_baseline(M, K, N):
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(M, K, generator=g).half().to(DEV)
+    w = (torch.randn(K, N, generator=g) * 0.05).half().to(DEV)
+    ref = vo.gemm(_np(x), _np(w), acc=np.float64)
+    _say("plain gemm", M, K, N)
+    y = cabi.gemm_f16(x, w)
+    torch.cuda.synchronize()
+    e1, _ = vo.rel_err(_np(y), ref)
+    assert e1 <= TOL, e1
+    _say("hipblaslt gemm", M, K, N)
+    yb = cabi.ref_gemm_f16(x, w)
+    ybt = cabi.ref_gemm_f16(x, w.t().contiguous(), w_is_nk=True)
+    torch.cuda.synchronize()
+    for t in (yb, ybt):
+        e1, _ = vo.rel_err(_np(t), ref)
+        assert e1 <= TOL, e1
+
+
+# ------------------------------------------------------------------ the measured configurations at full size
+def test_config_c1_full_against_golden_and_oracle():
+    import json, os
+    spec = CONFIGS["C1"]
+    x, codes, cb = make_problem(spec, seed=42, device=DEV)
+    _say("C1 full")
+    y = cabi.e2e_gemm_b(x, codes, cb)
+    w = cabi.dequant_b(codes, cb)
+    torch.cuda.synchronize()
+    _check_gemm(y, x, codes, cb, what="C1")
+    g = os.path.join(os.path.dirname(__file__), "golden")
+    data = np.load(os.path.join(g, "C1.npz"))
+    e1, _ = vo.rel_err(_np(y)[data["sample_rows"]][:, data["sample_cols"]], data["y_samples_f64"])
+    assert e1 <= TOL
+    assert np.array_equal(_np(w)[data["w_rows"]][:, data["w_cols"]].view(np.uint16), data["w_samples"].view(np.uint16))
+
+
+@pytest.mark.parametrize("name", ["C2", "C3"])
+def test_decode_configs_full_size(name):
+    spec = CONFIGS[name]
+    x, codes, cb = make_problem(spec, seed=42, device=DEV)
+    _say(name, "full", spec)
+    y = cabi.e2e_gemm_b(x, codes, cb)
+    w = cabi.dequant_b(codes, cb)
+    torch.cuda.synchronize()
+    want_w = vo.dequant_b(_np(codes), _np(cb))
+    assert np.array_equal(_np(w).view(np.uint16), want_w.view(np.uint16))       # bit-exact dequant at full size
+    ref = _np(x).astype(np.float64) @ want_w.astype(np.float64).T
+    e1, e2 = vo.rel_err(_np(y), ref)
+    _say(f"  {name}: rel_err={e1:.3e} {e2:.3e}")
+    assert e1 <= TOL
+    for _ in range(4):
+        assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)
+
+
+@pytest.mark.parametrize("name", ["C4", "C5"])
+def test_prefill_configs_full_size(name):
+    """Full-size prefill: bit-exact dequant, fp64 oracle on a sample of output rows, one-hot rows,
+    the two-pass route (dequant + plain GEMM) as a second on-device opinion, determinism."""
+    spec = CONFIGS[name]
+    x, codes, cb = make_problem(spec, seed=42, device=DEV)
+    _say(name, "full", spec)
+    # plant one-hot rows: those outputs must be bit-exact copies of weight columns
+    hot_rows = [0, spec.M // 2 + 1, spec.M - 1]
+    hot_k = [0, spec.K // 2 + 3, spec.K - 1]
+    for r, k in zip(hot_rows, hot_k):
+        x[r].zero_()
+        x[r, k] = 1.0
+    y = cabi.e2e_gemm_b(x, codes, cb)
+    torch.cuda.synchronize()
+    w = cabi.dequant_b(codes, cb)
+    torch.cuda.synchronize()
+    codes_np, cb_np = _np(codes), _np(cb)
+    rows = np.random.default_rng(0).choice(spec.N, size=4096 if name == "C4" else 2048, replace=False)
+    rows.sort()
+    # bit-exact dequant on a sample of W rows
+    g_of = rows // (spec.N // spec.n_codebooks)
+    w_np = _np(w[torch.from_numpy(rows).to(DEV)])
+    for g in np.unique(g_of):
+        sel = g_of == g
+        want = vo.dequant_b(codes_np[rows[sel]], cb_np[g])
+        assert np.array_equal(w_np[sel].view(np.uint16), want.view(np.uint16))
+    for r, k in zip(hot_rows, hot_k):
+        assert torch.equal(y[r], w[:, k]), (r, k)
+    # fp64 oracle on sampled X rows x sampled W rows
+    m_idx = np.sort(np.random.default_rng(1).choice(spec.M, size=48, replace=False))
+    ref = _np(x)[m_idx].astype(np.float64) @ w_np.astype(np.float64).T
+    got = _np(y[torch.from_numpy(m_idx).to(DEV)][:, torch.from_numpy(rows).to(DEV)])
+    e1, e2 = vo.rel_err(got, ref)
+    _say(f"  {name}: sampled rel_err={e1:.3e} {e2:.3e}")
+    assert e1 <= TOL
+    # the whole output against fp32 torch on the device (a library matmul on the dequantised weights)
+    ref_dev = (x.float() @ w.float().t())
+    err = ((y.float() - ref_dev).abs() / ref_dev.abs().clamp_min(1e-2 * ref_dev.pow(2).mean().sqrt())).max().item()
+    _say(f"  {name}: full-output rel_err vs device fp32 matmul={err:.3e}")
+    assert err <= TOL
+    del ref_dev
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)
+
+
+# ------------------------------------------------------------------ torch extension modules (the drop-in surface)
+def test_torch_extension_modules_serve_both_geometries():
+    from vq_gemm_amd import ops
+    spec = CONFIGS["C1"]
+    x, codes, cb = make_problem(spec, seed=42, device=DEV)
+    ref = vo.vq_gemm_b(_np(x), _np(codes), _np(cb), acc=np.float64)
+    for key in ("s1", "s2_128", "s2_512", "s3_naive", "s3_wasp"):
+        _say("module", key)
+        mod = ops.load_module(key)
+        y = mod.e2e_gemm(x, codes, cb)
+        torch.cuda.synchronize()
+        assert y.dtype == torch.float16 and y.shape == (spec.M, spec.N) and y.device == x.device
+        e1, _ = vo.rel_err(_np(y), ref)
+        assert e1 <= TOL, (key, e1)
+    # reference-native tensors, as bench.py:83-88 of the reference builds them
+    sa = ProblemSpec("A", GEOM_A, 128, 256, 256, 2, 256, 32, 8, codebook_std=1.0)
+    xa, wa, cba = make_problem(sa, seed=7, device=DEV)
+    refa = vo.vq_gemm_a(_np(xa), _np(wa), _np(cba), acc=np.float64)
+    for key in ("s1", "s2_128"):
+        ya = ops.load_module(key).e2e_gemm(xa, wa, cba)
+        torch.cuda.synchronize()
+        assert ya.shape == (128, 256)
+        e1, _ = vo.rel_err(_np(ya), refa)
+        assert e1 <= TOL, (key, e1)
+    # dequant + both gemm exports
+    mod = ops.load_module("s2_128")
+    assert np.array_equal(_np(mod.dequant(codes, cb)).view(np.uint16), vo.dequant_b(_np(codes), _np(cb)).view(np.uint16))
+    wd = mod.dequant(wa, cba)
+    assert np.array_equal(_np(wd).view(np.uint16), vo.dequant_a(_np(wa), _np(cba)).view(np.uint16))
+    for key in ("s2_128", "cublas_gemm"):
+        yg = ops.load_module(key).gemm(xa, wd)
+        torch.cuda.synchronize()
+        e1, _ = vo.rel_err(_np(yg), refa)
+        assert e1 <= TOL, (key, e1)
+    # non-contiguous / wrong-shape inputs
+    yt = mod.e2e_gemm(x.t().contiguous().t(), codes, cb)
+    assert torch.equal(yt, mod.e2e_gemm(x, codes, cb))
+    with pytest.raises(RuntimeError):
+        mod.e2e_gemm(x[:, :100], codes, cb)
+    with pytest.raises(RuntimeError):
+        mod.e2e_gemm(x.float(), codes, cb)

@@ -1,0 +1,178 @@
+"""ctypes view of the C ABI (include/vq_gemm.h, include/vq_gemm_ref.h).
+
+Used by the parity tests and the bench to drive libvqgemm.so directly with device pointers
+taken from torch tensors (torch is only the allocator here).  Loading fails loudly when the
+library has not been built; nothing falls back to a CPU implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+
+_LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+_INCLUDE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+
+VARIANT_AUTO, VARIANT_GENERIC, VARIANT_DECODE, VARIANT_PREFILL, VARIANT_TWOPASS = range(5)
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass"}
+
+_I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
+
+_SIGNATURES = {
+    "vqgemm_e2e_gemm_b": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
+    "vqgemm_e2e_gemm_a": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _P]),
+    "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
+    "vqgemm_dequant_a": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
+    "vqgemm_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _P]),
+    "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
+    "vqgemm_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "vqgemm_version": (ctypes.c_int, []),
+}
+_REF_SIGNATURES = {
+    "vqref_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _I32, _P]),
+    "vqref_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+}
+
+_lib = None
+_ref = None
+
+
+def declared_symbols(header: str):
+    """Function names declared in include/<header> (parsed from the header text)."""
+    text = open(os.path.join(_INCLUDE_DIR, header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vq(?:gemm|ref)_\w+)\s*\(", text)))
+
+
+def _load(name, sigs):
+    path = os.path.join(_LIB_DIR, name)
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it first (python compile_kernels.py build_ext --inplace); "
+                          "there is no CPU fallback")
+    lib = ctypes.CDLL(path)
+    for fn, (res, args) in sigs.items():
+        f = getattr(lib, fn)
+        f.restype = res
+        f.argtypes = args
+    return lib
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = _load("libvqgemm.so", _SIGNATURES)
+    return _lib
+
+
+def ref_lib():
+    global _ref
+    if _ref is None:
+        _ref = _load("libvqgemm_ref.so", _REF_SIGNATURES)
+    return _ref
+
+
+class VqGemmError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__(f"{what} failed with code {code}: {lib().vqgemm_error_string(code).decode()}")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _cb_dims(codebook):
+    if codebook.dim() == 2:
+        return 1, codebook.shape[0], codebook.shape[1]
+    return codebook.shape[0], codebook.shape[1], codebook.shape[2]
+
+
+def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=None):
+    """Geometry B fused GEMM through the C ABI.  Tensors must be contiguous device tensors."""
+    import torch
+    M, K = x.shape
+    N = codes.shape[0]
+    G, E, v = _cb_dims(codebook)
+    bits = 8 if codes.dtype == torch.uint8 else 16
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    if variant == VARIANT_TWOPASS and workspace is None:
+        workspace = torch.empty((N, K), dtype=torch.float16, device=x.device)
+    rc = lib().vqgemm_e2e_gemm_b(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(out), M, K, N, v, E, G, bits, variant,
+                                 _ptr(workspace), _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_e2e_gemm_b")
+    return out
+
+
+def e2e_gemm_a(x, w, codebook, variant=VARIANT_AUTO, out=None, workspace=None):
+    import torch
+    M, K = x.shape
+    Nc = w.shape[1]
+    if out is None:
+        out = torch.empty((M, 2 * Nc), dtype=torch.float16, device=x.device)
+    if variant == VARIANT_TWOPASS and workspace is None:
+        workspace = torch.empty((K, 2 * Nc), dtype=torch.float16, device=x.device)
+    rc = lib().vqgemm_e2e_gemm_a(_ptr(x), _ptr(w), _ptr(codebook), _ptr(out), M, K, Nc, variant, _ptr(workspace),
+                                 _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_e2e_gemm_a")
+    return out
+
+
+def dequant_b(codes, codebook, out=None):
+    import torch
+    N, J = codes.shape
+    G, E, v = _cb_dims(codebook)
+    bits = 8 if codes.dtype == torch.uint8 else 16
+    if out is None:
+        out = torch.empty((N, J * v), dtype=torch.float16, device=codes.device)
+    rc = lib().vqgemm_dequant_b(_ptr(codes), _ptr(codebook), _ptr(out), N, J * v, v, E, G, bits, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_dequant_b")
+    return out
+
+
+def dequant_a(w, codebook, out=None):
+    import torch
+    K, Nc = w.shape
+    if out is None:
+        out = torch.empty((K, 2 * Nc), dtype=torch.float16, device=w.device)
+    rc = lib().vqgemm_dequant_a(_ptr(w), _ptr(codebook), _ptr(out), K, Nc, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_dequant_a")
+    return out
+
+
+def gemm_f16(x, w, out=None):
+    import torch
+    M, K = x.shape
+    N = w.shape[1]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    rc = lib().vqgemm_gemm_f16(_ptr(x), _ptr(w), _ptr(out), M, K, N, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_gemm_f16")
+    return out
+
+
+def ref_gemm_f16(x, w, w_is_nk=False, out=None):
+    """hipBLASLt baseline: x[M,K] @ w[K,N], or x @ w[N,K].T when w_is_nk."""
+    import torch
+    M, K = x.shape
+    N = w.shape[0] if w_is_nk else w.shape[1]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    rc = ref_lib().vqref_gemm_f16(_ptr(x), _ptr(w), _ptr(out), M, K, N, 1 if w_is_nk else 0, _stream())
+    if rc != 0:
+        raise RuntimeError(f"vqref_gemm_f16 failed with code {rc}: {ref_lib().vqref_error_string(rc).decode()}")
+    return out
+
+
+def select_variant_b(M, K, N, vec, entries, n_codebooks, code_bits) -> int:
+    return lib().vqgemm_select_variant_b(M, K, N, vec, entries, n_codebooks, code_bits)

@@ -1,0 +1,212 @@
+// C ABI of libvqgemm.so: argument validation and kernel selection.  No torch types here;
+// the torch extension and the tests both call these entry points.
+#include "../../include/vq_gemm.h"
+#include "vq_common.h"
+
+#include <atomic>
+#include <limits.h>
+
+namespace vq {
+
+int device_cu_count()
+{
+    constexpr int kMaxDev = 64;
+    static std::atomic<int> cache[kMaxDev];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+    int v = cache[dev].load(std::memory_order_relaxed);
+    if (v > 0) return v;
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cache[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
+namespace {
+
+bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+int check_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits)
+{
+    if (M < 0 || K < 0 || N < 0 || M > INT_MAX / 2 || K > INT_MAX / 2 || N > INT_MAX / 2) return VQGEMM_E_SHAPE;
+    if (vec < 1 || vec > 4096 || entries < 1 || n_codebooks < 1) return VQGEMM_E_SHAPE;
+    if (code_bits != 8 && code_bits != 16) return VQGEMM_E_CODEBITS;
+    if ((int64_t)entries > ((int64_t)1 << code_bits)) return VQGEMM_E_CODEBITS;
+    if (K % vec != 0) return VQGEMM_E_SHAPE;
+    if (N % n_codebooks != 0) return VQGEMM_E_SHAPE;
+    return VQGEMM_OK;
+}
+
+ProblemB make_b(const void *x, const void *codes, const void *codebook, void *y, int64_t M, int64_t K, int64_t N,
+                int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits)
+{
+    ProblemB p;
+    p.x = static_cast<const half_t *>(x);
+    p.codes = codes;
+    p.cb = static_cast<const half_t *>(codebook);
+    p.y = static_cast<half_t *>(y);
+    p.M = (int)M; p.K = (int)K; p.N = (int)N;
+    p.vec = vec; p.entries = entries; p.n_codebooks = n_codebooks; p.code_bits = code_bits;
+    p.rows_per_cb = N > 0 ? (int)(N / n_codebooks) : 1;
+    if (p.rows_per_cb < 1) p.rows_per_cb = 1;
+    return p;
+}
+
+int select_b(const ProblemB &p, bool all_aligned16)
+{
+    if (p.K == 0 || !all_aligned16) return VQGEMM_VARIANT_GENERIC;
+    if (p.M <= 16 && decode_supports(p)) return VQGEMM_VARIANT_DECODE;
+    if (prefill_supports(p)) return VQGEMM_VARIANT_PREFILL;
+    return VQGEMM_VARIANT_GENERIC;
+}
+
+}  // namespace
+}  // namespace vq
+
+using namespace vq;
+
+extern "C" {
+
+int vqgemm_version(void) { return 100; }
+
+const char *vqgemm_error_string(int code)
+{
+    switch (code) {
+    case VQGEMM_OK: return "success";
+    case VQGEMM_E_NULL: return "a required pointer is NULL";
+    case VQGEMM_E_SHAPE: return "invalid shape (negative or too large size, K % vec != 0, N % n_codebooks != 0, ...)";
+    case VQGEMM_E_CODEBITS: return "code_bits must be 8 or 16 and entries <= 2^code_bits";
+    case VQGEMM_E_VARIANT: return "unknown kernel variant, or the variant cannot serve this shape";
+    case VQGEMM_E_ALIGN: return "pointer not aligned as the selected kernel requires";
+    default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown vqgemm error";
+}
+
+int vqgemm_select_variant_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks,
+                            int32_t code_bits)
+{
+    const int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    const ProblemB p = make_b(nullptr, nullptr, nullptr, nullptr, M, K, N, vec, entries, n_codebooks, code_bits);
+    return select_b(p, true);
+}
+
+int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, void *y, int64_t M, int64_t K,
+                      int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits,
+                      int32_t variant, void *workspace, void *stream)
+{
+    int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_TWOPASS) return VQGEMM_E_VARIANT;
+    if (M == 0 || N == 0) return VQGEMM_OK;
+    if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
+    const uintptr_t code_align = code_bits / 8;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(codebook, 2) || !aligned(codes, code_align)) return VQGEMM_E_ALIGN;
+    const bool a16 = aligned(x, 16) && aligned(y, 16) && aligned(codebook, 16) && aligned(codes, 16);
+    const ProblemB p = make_b(x, codes, codebook, y, M, K, N, vec, entries, n_codebooks, code_bits);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (variant == VQGEMM_VARIANT_AUTO) variant = select_b(p, a16);
+    hipError_t e = hipSuccess;
+    switch (variant) {
+    case VQGEMM_VARIANT_GENERIC:
+        e = launch_generic_b(p, s);
+        break;
+    case VQGEMM_VARIANT_DECODE:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !decode_supports(p)) return VQGEMM_E_VARIANT;
+        e = launch_decode_b(p, s);
+        break;
+    case VQGEMM_VARIANT_PREFILL:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !prefill_supports(p)) return VQGEMM_E_VARIANT;
+        e = launch_prefill_b(p, s);
+        break;
+    case VQGEMM_VARIANT_TWOPASS:
+        if (!workspace) return VQGEMM_E_NULL;
+        if (!aligned(workspace, 16)) return VQGEMM_E_ALIGN;
+        e = launch_dequant_b(p, static_cast<half_t *>(workspace), s);
+        if (e == hipSuccess)
+            e = launch_gemm_nt(p.x, static_cast<const half_t *>(workspace), p.y, p.M, p.K, p.N, s);
+        break;
+    default:
+        return VQGEMM_E_VARIANT;
+    }
+    return static_cast<int>(e);
+}
+
+int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *out, int64_t M, int64_t K,
+                      int64_t Nc, int32_t variant, void *workspace, void *stream)
+{
+    if (M < 0 || K < 0 || Nc < 0 || M > INT_MAX / 2 || K > INT_MAX / 2 || Nc > INT_MAX / 4) return VQGEMM_E_SHAPE;
+    if (Nc % 4 != 0) return VQGEMM_E_SHAPE;
+    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_TWOPASS) return VQGEMM_E_VARIANT;
+    if (M == 0 || Nc == 0) return VQGEMM_OK;
+    if (!out || !codebook || (K > 0 && (!x || !w))) return VQGEMM_E_NULL;
+    if (!aligned(x, 2) || !aligned(out, 4) || !aligned(codebook, 4)) return VQGEMM_E_ALIGN;
+    ProblemA p;
+    p.x = static_cast<const half_t *>(x);
+    p.w = static_cast<const uint8_t *>(w);
+    p.cb = static_cast<const half_t *>(codebook);
+    p.y = static_cast<half_t *>(out);
+    p.M = (int)M; p.K = (int)K; p.Nc = (int)Nc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipSuccess;
+    switch (variant) {
+    case VQGEMM_VARIANT_AUTO:
+    case VQGEMM_VARIANT_GENERIC:
+        e = launch_generic_a(p, s);
+        break;
+    case VQGEMM_VARIANT_TWOPASS:
+        if (!workspace) return VQGEMM_E_NULL;
+        if (!aligned(workspace, 16)) return VQGEMM_E_ALIGN;
+        e = launch_dequant_a(p, static_cast<half_t *>(workspace), s);
+        if (e == hipSuccess)
+            e = launch_gemm_nn(p.x, static_cast<const half_t *>(workspace), p.y, p.M, p.K, 2 * p.Nc, s);
+        break;
+    default:
+        return VQGEMM_E_VARIANT;  // the decode/prefill tilings are geometry-B kernels
+    }
+    return static_cast<int>(e);
+}
+
+int vqgemm_dequant_b(const void *codes, const void *codebook, void *w_out, int64_t N, int64_t K, int32_t vec,
+                     int32_t entries, int32_t n_codebooks, int32_t code_bits, void *stream)
+{
+    const int rc = check_b(0, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (N == 0 || K == 0) return VQGEMM_OK;
+    if (!codes || !codebook || !w_out) return VQGEMM_E_NULL;
+    if (!aligned(w_out, 2) || !aligned(codebook, 2) || !aligned(codes, code_bits / 8)) return VQGEMM_E_ALIGN;
+    const ProblemB p = make_b(nullptr, codes, codebook, nullptr, 0, K, N, vec, entries, n_codebooks, code_bits);
+    return static_cast<int>(launch_dequant_b(p, static_cast<half_t *>(w_out), static_cast<hipStream_t>(stream)));
+}
+
+int vqgemm_dequant_a(const void *w, const void *codebook, void *w_out, int64_t K, int64_t Nc, void *stream)
+{
+    if (K < 0 || Nc < 0 || K > INT_MAX / 2 || Nc > INT_MAX / 4 || Nc % 4 != 0) return VQGEMM_E_SHAPE;
+    if (K == 0 || Nc == 0) return VQGEMM_OK;
+    if (!w || !codebook || !w_out) return VQGEMM_E_NULL;
+    if (!aligned(w_out, 4) || !aligned(codebook, 4)) return VQGEMM_E_ALIGN;
+    ProblemA p;
+    p.x = nullptr;
+    p.w = static_cast<const uint8_t *>(w);
+    p.cb = static_cast<const half_t *>(codebook);
+    p.y = nullptr;
+    p.M = 0; p.K = (int)K; p.Nc = (int)Nc;
+    return static_cast<int>(launch_dequant_a(p, static_cast<half_t *>(w_out), static_cast<hipStream_t>(stream)));
+}
+
+int vqgemm_gemm_f16(const void *x, const void *w, void *y, int64_t M, int64_t K, int64_t N, void *stream)
+{
+    if (M < 0 || K < 0 || N < 0 || M > INT_MAX / 2 || K > INT_MAX / 2 || N > INT_MAX / 2) return VQGEMM_E_SHAPE;
+    if (M == 0 || N == 0) return VQGEMM_OK;
+    if (!y || (K > 0 && (!x || !w))) return VQGEMM_E_NULL;
+    if (!aligned(x, 2) || !aligned(w, 2) || !aligned(y, 2)) return VQGEMM_E_ALIGN;
+    return static_cast<int>(launch_gemm_nn(static_cast<const half_t *>(x), static_cast<const half_t *>(w),
+                                           static_cast<half_t *>(y), (int)M, (int)K, (int)N,
+                                           static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

@@ -1,0 +1,74 @@
+// Shared device helpers and launcher declarations for the gfx950 VQ-GEMM kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vq {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// Problem description shared by the geometry-B kernels.
+struct ProblemB {
+    const half_t *x;      // [M,K]
+    const void *codes;    // [N, K/vec] u8 or u16
+    const half_t *cb;     // [G, E, vec]
+    half_t *y;            // [M,N]
+    int M, K, N;
+    int vec, entries, n_codebooks, code_bits;
+    int rows_per_cb;      // N / G
+};
+
+struct ProblemA {
+    const half_t *x;      // [M,K]
+    const uint8_t *w;     // [K,Nc]
+    const half_t *cb;     // [Nc/4, 256, 2]
+    half_t *y;            // [M, 2*Nc]
+    int M, K, Nc;
+};
+
+__device__ __forceinline__ uint32_t lane_id() { return threadIdx.x & (kWave - 1); }
+
+// 16-byte global load / store helpers (addresses must be 16-byte aligned).
+__device__ __forceinline__ uint4_t ld_global_16(const void *p) { return *reinterpret_cast<const uint4_t *>(p); }
+__device__ __forceinline__ void st_global_16(void *p, uint4_t v) { *reinterpret_cast<uint4_t *>(p) = v; }
+
+template <typename T>
+__device__ __forceinline__ half8_t as_half8(T v)
+{
+    static_assert(sizeof(T) == 16, "16-byte value expected");
+    union { T t; half8_t h; } u;
+    u.t = v;
+    return u.h;
+}
+
+// ---- launchers (defined one per .hip file) -------------------------------------------
+hipError_t launch_dequant_b(const ProblemB &p, half_t *w_out, hipStream_t s);
+hipError_t launch_dequant_a(const ProblemA &p, half_t *w_out, hipStream_t s);
+
+hipError_t launch_generic_b(const ProblemB &p, hipStream_t s);
+hipError_t launch_generic_a(const ProblemA &p, hipStream_t s);
+
+bool decode_supports(const ProblemB &p);
+hipError_t launch_decode_b(const ProblemB &p, hipStream_t s);
+
+bool prefill_supports(const ProblemB &p);
+hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s);
+
+// o[M,N] = x[M,K] . w[K,N]
+hipError_t launch_gemm_nn(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);
+// y[M,N] = x[M,K] . w[N,K]^T
+hipError_t launch_gemm_nt(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);
+
+int device_cu_count();
+
+}  // namespace vq

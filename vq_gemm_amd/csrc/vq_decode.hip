@@ -1,0 +1,254 @@
+// Decode kernel (M <= 16): Y[M,N] = X[M,K] . W^T with W given as codes + codebook.
+//
+// The kernel is bound by the HBM stream of the code matrix (N*K/vec code bytes), so the
+// design goal is one pass over the codes with every other operand resident on the CU:
+//
+//   * A workgroup owns tiles of 16 output columns (16 rows of W).  Each of its waves owns a
+//     512-wide slice of K and keeps the matching slice of X in registers, already in MFMA
+//     operand order, for the whole kernel: X is read from memory once per workgroup and never
+//     passes through the LDS.
+//   * The codebook (entries*vec*2 bytes) is resident in the LDS.  A lane streams 16 bytes of
+//     codes of one W row, gathers the codewords and uses them *directly* as the 8-half A
+//     operand of v_mfma_f32_16x16x32_f16: with vec = 8 one ds_read_b128 is one operand.
+//     The order in which a lane walks K is irrelevant to a dot product, so it is chosen so
+//     that each lane's codes are contiguous in memory; X is loaded in the same order.
+//   * Per tile a wave issues 16 MFMAs (its K slice), the partial 16x16 fp32 results of the
+//     waves are summed through 1 KB LDS slots, and one wave converts and stores the tile.
+//
+// M < 16 pads the X operand with zeros (the matrix core is idle anyway: the kernel is
+// bandwidth bound by a wide margin); fp32 accumulation throughout, one rounding to fp16.
+#include "vq_common.h"
+
+namespace vq {
+
+namespace {
+
+constexpr int kSliceK = 512;   // K handled by one wave
+constexpr int kSteps = 16;     // MFMA steps per slice (32 k each)
+constexpr int kTileN = 16;
+constexpr int kMaxWaves = 16;
+
+template <int VEC, typename CodeT>
+struct DecodeCfg {
+    static constexpr int CPL = 16 / (int)sizeof(CodeT);  // codes in one 16-byte lane load
+    static constexpr int CPO = 8 / VEC;                  // codes per 8-half MFMA operand
+    static constexpr int SPL = CPL / CPO;                // MFMA steps fed by one lane load
+    static constexpr int K_LANE = CPL * VEC;             // k covered by one lane load
+    static constexpr int K_WAVE = 4 * K_LANE;            // k covered by one wave load (4 k-groups)
+    static constexpr int LPT = kSliceK / K_WAVE;         // lane loads per slice
+    static_assert(CPO >= 1 && SPL >= 1 && LPT >= 1 && LPT * SPL == kSteps, "unsupported code layout");
+};
+
+template <typename CodeT, int CPL>
+__device__ __forceinline__ uint32_t extract_code(const uint4_t &cw, int c)
+{
+    if constexpr (sizeof(CodeT) == 1)
+        return (cw[c >> 2] >> (8 * (c & 3))) & 0xffu;
+    else
+        return (cw[c >> 1] >> (16 * (c & 1))) & 0xffffu;
+}
+
+// Gather the 8-half operand made of CPO consecutive codewords starting at code c0.
+template <int VEC, typename CodeT>
+__device__ __forceinline__ half8_t gather_operand(const uint8_t *cb_lds, const uint4_t &cw, int c0)
+{
+    typedef DecodeCfg<VEC, CodeT> C;
+    if constexpr (VEC == 8) {
+        const uint32_t code = extract_code<CodeT, C::CPL>(cw, c0);
+        return *reinterpret_cast<const half8_t *>(cb_lds + code * 16u);
+    } else if constexpr (VEC == 4) {
+        const uint32_t a = extract_code<CodeT, C::CPL>(cw, c0);
+        const uint32_t b = extract_code<CodeT, C::CPL>(cw, c0 + 1);
+        const half4_t lo = *reinterpret_cast<const half4_t *>(cb_lds + a * 8u);
+        const half4_t hi = *reinterpret_cast<const half4_t *>(cb_lds + b * 8u);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    } else {
+        static_assert(VEC == 2, "vector length must be 2, 4 or 8");
+        half2_t q[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t c = extract_code<CodeT, C::CPL>(cw, c0 + i);
+            q[i] = *reinterpret_cast<const half2_t *>(cb_lds + c * 4u);
+        }
+        const half4_t lo = __builtin_shufflevector(q[0], q[1], 0, 1, 2, 3);
+        const half4_t hi = __builtin_shufflevector(q[2], q[3], 0, 1, 2, 3);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+}
+
+template <int VEC, typename CodeT>
+__global__ __launch_bounds__(1024) void decode_kernel(const half_t *__restrict__ x,
+                                                      const CodeT *__restrict__ codes,
+                                                      const half_t *__restrict__ cb,
+                                                      half_t *__restrict__ y, int M, int K, int N,
+                                                      int entries, int rows_per_cb, int tiles_per_wg,
+                                                      int n_tiles, int n_chunks)
+{
+    typedef DecodeCfg<VEC, CodeT> C;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int n_waves = blockDim.x >> 6;
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int r16 = lane & 15;  // W row within the tile (A operand) / X row m (B operand)
+    const int kq = lane >> 4;   // k-group of the lane, 0..3
+    const int J = K / VEC;
+    const int cb_bytes = entries * VEC * 2;
+    uint8_t *cb_lds = smem;
+    float4_t *red = reinterpret_cast<float4_t *>(smem + ((cb_bytes + 15) & ~15));
+
+    const int tile_begin = blockIdx.x * tiles_per_wg;
+    const int tile_end = min(tile_begin + tiles_per_wg, n_tiles);
+    if (tile_begin >= tile_end) return;
+
+    // k of MFMA step s for this lane inside a slice that starts at k0.
+    auto step_k = [&](int k0, int s) { return k0 + (s / C::SPL) * C::K_WAVE + kq * C::K_LANE + (s % C::SPL) * 8; };
+
+    half8_t xr[kSteps];
+    auto load_x = [&](int k0) {
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            const int k = step_k(k0, s);
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (r16 < M && k < K) v = ld_global_16(x + (int64_t)r16 * K + k);
+            xr[s] = as_half8(v);
+        }
+    };
+    auto load_codes = [&](int tile, int k0, uint4_t (&cw)[C::LPT]) {
+        const int row = min(tile * kTileN + r16, N - 1);
+#pragma unroll
+        for (int t = 0; t < C::LPT; t++) {
+            const int k = k0 + t * C::K_WAVE + kq * C::K_LANE;
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (k < K) v = ld_global_16(codes + (int64_t)row * J + k / VEC);
+            cw[t] = v;
+        }
+    };
+
+    const int chunk_k = n_waves * kSliceK;
+    uint4_t cw_next[C::LPT];
+    load_codes(tile_begin, wave * kSliceK, cw_next);
+    if (n_chunks == 1) load_x(wave * kSliceK);
+
+    int cur_cb = -1;
+    int parity = 0;
+    for (int tile = tile_begin; tile < tile_end; tile++) {
+        const int g = (tile * kTileN) / rows_per_cb;
+        if (g != cur_cb) {
+            // (Re)load the codebook of this row block into the LDS.
+            if (cur_cb >= 0) __syncthreads();
+            const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g * entries * VEC);
+            for (int i = threadIdx.x; i < cb_bytes / 16; i += blockDim.x)
+                reinterpret_cast<uint4_t *>(cb_lds)[i] = src[i];
+            __syncthreads();
+            cur_cb = g;
+        }
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        for (int chunk = 0; chunk < n_chunks; chunk++) {
+            const int k0 = chunk * chunk_k + wave * kSliceK;
+            uint4_t cw[C::LPT];
+#pragma unroll
+            for (int t = 0; t < C::LPT; t++) cw[t] = cw_next[t];
+            // Prefetch the next (tile, chunk) codes while this one is consumed.
+            {
+                int ntile = tile, nchunk = chunk + 1;
+                if (nchunk == n_chunks) { nchunk = 0; ntile = tile + 1; }
+                if (ntile < tile_end) load_codes(ntile, nchunk * chunk_k + wave * kSliceK, cw_next);
+            }
+            if (n_chunks > 1) load_x(k0);
+#pragma unroll
+            for (int s = 0; s < kSteps; s++) {
+                const half8_t a = gather_operand<VEC, CodeT>(cb_lds, cw[s / C::SPL], (s % C::SPL) * C::CPO);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xr[s], acc, 0, 0, 0);
+            }
+        }
+        // Sum the K slices of the waves: slot (parity, wave, lane).
+        red[(parity * n_waves + wave) * 64 + lane] = acc;
+        __syncthreads();
+        if (wave == (tile % n_waves)) {
+            float4_t sum = red[(parity * n_waves) * 64 + lane];
+            for (int w = 1; w < n_waves; w++) {
+                const float4_t v = red[(parity * n_waves + w) * 64 + lane];
+                sum += v;
+            }
+            // D[i][j]: j = lane % 16 is the X row m, i = 4*(lane/16) + r is the W row.
+            const int m = r16;
+            const int n = tile * kTileN + 4 * kq;
+            if (m < M) {
+                half_t *dst = y + (int64_t)m * N + n;
+                if ((N & 3) == 0 && n + 3 < N) {
+                    half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                    *reinterpret_cast<half4_t *>(dst) = h;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (n + r < N) dst[r] = (half_t)sum[r];
+                }
+            }
+        }
+        parity ^= 1;
+    }
+}
+
+template <int VEC, typename CodeT>
+hipError_t launch_decode_typed(const ProblemB &p, hipStream_t s)
+{
+    const int slices = (p.K + kSliceK - 1) / kSliceK;
+    const int n_waves = slices < kMaxWaves ? slices : kMaxWaves;
+    const int n_chunks = (slices + n_waves - 1) / n_waves;
+    const int n_tiles = (p.N + kTileN - 1) / kTileN;
+    const int target = device_cu_count() * 2;
+    int tiles_per_wg = (n_tiles + target - 1) / target;
+    if (tiles_per_wg < 1) tiles_per_wg = 1;
+    const int grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+    const int cb_bytes = p.entries * VEC * 2;
+    const size_t smem = (size_t)((cb_bytes + 15) & ~15) + (size_t)2 * n_waves * 64 * sizeof(float4_t);
+    auto kern = decode_kernel<VEC, CodeT>;
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
+                       p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb, tiles_per_wg, n_tiles, n_chunks);
+    return hipGetLastError();
+}
+
+template <int VEC, typename CodeT>
+bool decode_cfg_supports(const ProblemB &p)
+{
+    typedef DecodeCfg<VEC, CodeT> C;
+    return p.K % C::K_LANE == 0;  // whole 16-byte code loads, 16-byte aligned code rows
+}
+
+constexpr size_t kDecodeLdsBudget = 144 * 1024;  // codebook + reduction slots must fit the 160 KB LDS
+
+}  // namespace
+
+bool decode_supports(const ProblemB &p)
+{
+    if (p.M < 1 || p.M > 16 || p.N < 1 || p.K < 1) return false;
+    if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
+    if (p.n_codebooks > 1 && p.rows_per_cb % kTileN != 0) return false;
+    if ((size_t)p.entries * p.vec * 2 + 2 * kMaxWaves * 1024 > kDecodeLdsBudget) return false;
+    if (p.K % 8 != 0) return false;
+    if (((size_t)p.entries * p.vec * 2) % 16 != 0) return false;
+    const bool u8 = p.code_bits == 8;
+    switch (p.vec) {
+    case 8: return u8 ? decode_cfg_supports<8, uint8_t>(p) : decode_cfg_supports<8, uint16_t>(p);
+    case 4: return u8 ? decode_cfg_supports<4, uint8_t>(p) : decode_cfg_supports<4, uint16_t>(p);
+    default: return u8 ? decode_cfg_supports<2, uint8_t>(p) : decode_cfg_supports<2, uint16_t>(p);
+    }
+}
+
+hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
+{
+    if (!decode_supports(p)) return hipErrorInvalidValue;
+    const bool u8 = p.code_bits == 8;
+    switch (p.vec) {
+    case 8: return u8 ? launch_decode_typed<8, uint8_t>(p, s) : launch_decode_typed<8, uint16_t>(p, s);
+    case 4: return u8 ? launch_decode_typed<4, uint8_t>(p, s) : launch_decode_typed<4, uint16_t>(p, s);
+    default: return u8 ? launch_decode_typed<2, uint8_t>(p, s) : launch_decode_typed<2, uint16_t>(p, s);
+    }
+}
+
+}  // namespace vq

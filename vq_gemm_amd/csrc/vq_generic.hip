@@ -1,0 +1,82 @@
+// Shape-agnostic fused VQ-GEMM kernels: one output element per thread, scalar loads,
+// sequential fp32 accumulation.  They serve every shape the tiled kernels reject (odd K,
+// unusual vector lengths, codebooks too large for the LDS) and act as an independent
+// on-device statement of the math in the tests.  Not tuned.
+#include "vq_common.h"
+
+namespace vq {
+
+template <typename CodeT>
+__global__ __launch_bounds__(256) void generic_b_kernel(const half_t *__restrict__ x,
+                                                        const CodeT *__restrict__ codes,
+                                                        const half_t *__restrict__ cb,
+                                                        half_t *__restrict__ y, int M, int K, int N,
+                                                        int vec, int entries, int rows_per_cb)
+{
+    // blockDim = (64, 4): x index -> n (coalesced y stores), y index -> m.
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    const int J = K / vec;
+    const half_t *book = cb + (int64_t)(n / rows_per_cb) * entries * vec;
+    const CodeT *crow = codes + (int64_t)n * J;
+    for (int m = blockIdx.y * blockDim.y + threadIdx.y; m < M; m += gridDim.y * blockDim.y) {
+        const half_t *xrow = x + (int64_t)m * K;
+        float acc = 0.0f;
+        for (int j = 0; j < J; j++) {
+            uint32_t c = crow[j];
+            c = c < (uint32_t)entries ? c : (uint32_t)entries - 1;  // memory safety only
+            const half_t *cw = book + (int64_t)c * vec;
+            for (int t = 0; t < vec; t++) acc += (float)xrow[j * vec + t] * (float)cw[t];
+        }
+        y[(int64_t)m * N + n] = (half_t)acc;
+    }
+}
+
+hipError_t launch_generic_b(const ProblemB &p, hipStream_t s)
+{
+    if (p.M == 0 || p.N == 0) return hipSuccess;
+    dim3 block(64, 4);
+    dim3 grid((p.N + 63) / 64, (unsigned)(((p.M + 3) / 4) < 32768 ? (p.M + 3) / 4 : 32768));
+    if (p.code_bits == 8)
+        hipLaunchKernelGGL((generic_b_kernel<uint8_t>), grid, block, 0, s, p.x, static_cast<const uint8_t *>(p.codes),
+                           p.cb, p.y, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
+    else
+        hipLaunchKernelGGL((generic_b_kernel<uint16_t>), grid, block, 0, s, p.x, static_cast<const uint16_t *>(p.codes),
+                           p.cb, p.y, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
+    return hipGetLastError();
+}
+
+// Geometry A: out[m, 2n + r] = sum_k x[m,k] * cb[n/4][w[k,n]][r].  One thread per code
+// column computes both outputs of the codeword.
+__global__ __launch_bounds__(256) void generic_a_kernel(const half_t *__restrict__ x,
+                                                        const uint8_t *__restrict__ w,
+                                                        const half_t *__restrict__ cb,
+                                                        half_t *__restrict__ y, int M, int K, int Nc)
+{
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= Nc) return;
+    const half_t *book = cb + (int64_t)(n >> 2) * 256 * 2;
+    for (int m = blockIdx.y * blockDim.y + threadIdx.y; m < M; m += gridDim.y * blockDim.y) {
+        const half_t *xrow = x + (int64_t)m * K;
+        float a0 = 0.0f, a1 = 0.0f;
+        for (int k = 0; k < K; k++) {
+            const uint32_t c = w[(int64_t)k * Nc + n];
+            const float xv = (float)xrow[k];
+            a0 += xv * (float)book[c * 2];
+            a1 += xv * (float)book[c * 2 + 1];
+        }
+        y[(int64_t)m * (2 * Nc) + 2 * n] = (half_t)a0;
+        y[(int64_t)m * (2 * Nc) + 2 * n + 1] = (half_t)a1;
+    }
+}
+
+hipError_t launch_generic_a(const ProblemA &p, hipStream_t s)
+{
+    if (p.M == 0 || p.Nc == 0) return hipSuccess;
+    dim3 block(64, 4);
+    dim3 grid((p.Nc + 63) / 64, (unsigned)(((p.M + 3) / 4) < 32768 ? (p.M + 3) / 4 : 32768));
+    hipLaunchKernelGGL(generic_a_kernel, grid, block, 0, s, p.x, p.w, p.cb, p.y, p.M, p.K, p.Nc);
+    return hipGetLastError();
+}
+
+}  // namespace vq
