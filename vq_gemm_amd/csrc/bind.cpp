@@ -10,7 +10,7 @@
 // mirroring the reference's one-extension-per-strategy scheme (compile_kernels.py:55-68).
 #include <torch/extension.h>
 #include <c10/hip/HIPStream.h>
-#include <c10/hip/HIPGuard.h>
+#include <c10/core/DeviceGuard.h>
 
 #include "../../include/vq_gemm.h"
 #include "../../include/vq_gemm_ref.h"
@@ -107,7 +107,7 @@ torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codeb
     TORCH_CHECK(w.device() == input.device() && codebook.device() == input.device(),
                 "input, w and codebook must be on the same device");
     const Geometry g = classify(input, w, codebook);
-    c10::hip::HIPGuard guard(input.device());
+    c10::DeviceGuard guard(input.device());
     torch::Tensor x = canon(input), c = canon(w), cb = canon(codebook);
     torch::Tensor out = torch::empty({g.M, g.N}, input.options());
     torch::Tensor ws;
@@ -139,7 +139,7 @@ torch::Tensor gemm(torch::Tensor input, torch::Tensor w)
     TORCH_CHECK(input.scalar_type() == torch::kFloat16 && w.scalar_type() == torch::kFloat16, "gemm expects float16");
     TORCH_CHECK(input.size(1) == w.size(0), "gemm: input is [M,", input.size(1), "] but w is [", w.size(0), ",N]");
     TORCH_CHECK(w.device() == input.device(), "input and w must be on the same device");
-    c10::hip::HIPGuard guard(input.device());
+    c10::DeviceGuard guard(input.device());
     torch::Tensor x = canon(input), ww = canon(w);
     torch::Tensor out = torch::empty({input.size(0), w.size(1)}, input.options());
     check_rc(vqgemm_gemm_f16(x.data_ptr(), ww.data_ptr(), out.data_ptr(), input.size(0), input.size(1), w.size(1),
@@ -161,7 +161,7 @@ torch::Tensor dequant(torch::Tensor w, torch::Tensor codebook)
     const int64_t v = codebook.size(-1), E = codebook.size(-2);
     const int64_t G = codebook.dim() == 3 ? codebook.size(0) : 1;
     const bool is_a = w.scalar_type() == torch::kUInt8 && codebook.dim() == 3 && v == 2 && E == 256 && G * 4 == w.size(1);
-    c10::hip::HIPGuard guard(w.device());
+    c10::DeviceGuard guard(w.device());
     torch::Tensor c = canon(w), cb = canon(codebook);
     auto opts = codebook.options();
     if (is_a) {
@@ -188,7 +188,7 @@ torch::Tensor gemm(torch::Tensor input, torch::Tensor w)
     TORCH_CHECK(input.scalar_type() == torch::kFloat16 && w.scalar_type() == torch::kFloat16, "gemm expects float16");
     TORCH_CHECK(input.size(1) == w.size(0), "gemm: input is [M,", input.size(1), "] but w is [", w.size(0), ",N]");
     TORCH_CHECK(w.device() == input.device(), "input and w must be on the same device");
-    c10::hip::HIPGuard guard(input.device());
+    c10::DeviceGuard guard(input.device());
     torch::Tensor x = canon(input), ww = canon(w);
     torch::Tensor out = torch::empty({input.size(0), w.size(1)}, input.options());
     check_rc(vqref_gemm_f16(x.data_ptr(), ww.data_ptr(), out.data_ptr(), input.size(0), input.size(1), w.size(1),
