@@ -8,16 +8,27 @@
 //     operand (vec = 8: one ds_read_b128 == one operand).  The order in which K is walked is
 //     free, so it is chosen to make a lane's codes contiguous: one 16-byte global load per
 //     lane feeds CPL/CPO MFMA steps.
-//   * X tiles (256 rows x 64 k) are staged global -> registers -> LDS, double buffered, with
-//     the 16-byte chunks of a row XOR-swizzled so that operand reads are conflict free; the
-//     loads for stage i+2 are in flight while stage i is multiplied.
-//   * fp32 accumulation; one rounding to fp16 in the epilogue.
+//   * X tiles (256 rows x 64 k) go global -> LDS directly (global_load_lds_dwordx4, no register
+//     staging) through four buffers (three when the codebooks are large), issued three stages
+//     ahead of their use so that an HBM miss is covered by two stages of MFMA work.
+//     The LDS has 64 banks of 4 bytes: two 128-byte tile rows form one 256-byte bank row and
+//     the sixteen 16-byte chunks of a bank row are XOR-swizzled with the bank-row index, which
+//     makes the operand reads (32 consecutive rows x one chunk per half wave) conflict free.
+//     A direct load fills 64 consecutive slots per wave, so each lane fetches whatever chunk
+//     the swizzle assigns to its slot.
+//   * The MFMA operands of step s+1 are fetched from the LDS while step s is multiplied, also
+//     across stage boundaries: the barrier that publishes stage i+2 sits a whole stage ahead
+//     of its first read.
+//   * fp32 accumulation; one rounding to fp16 in the epilogue, which transposes through the
+//     LDS so that Y is written in 256-byte row segments.
 //
 // K order.  A lane of the 32x32x16 MFMA holds 8 consecutive k of one row; lanes 0-31 hold
 // k-group 0 and lanes 32-63 k-group 1.  A "super stage" is the K range fed by one 16-byte
 // code load per lane: lane group g covers the contiguous range
 // [S*2*K_LANE + g*K_LANE, +K_LANE).  LDS stage t of the super stage holds, for both groups,
 // the 32 k starting at offset t*32 of the group's range: two 64-byte pieces per X row.
+// K must be a multiple of K_LANE; when it is not a multiple of 2*K_LANE the last super stage
+// has no data for group 1 and the TAIL instantiation zeroes that group's W operand.
 #include "vq_common.h"
 
 namespace vq {
@@ -73,10 +84,50 @@ __device__ __forceinline__ half8_t gather8(const uint8_t *book, const uint4_t &c
     }
 }
 
-// Physical 16-byte slot of logical chunk cc (0..7) of X-tile row `row`.
-__device__ __forceinline__ int x_slot(int row, int cc) { return row * 8 + (cc ^ (row & 7)); }
+// Byte offset inside a stage buffer of logical 16-byte chunk cc (0..7) of X-tile row `row`.
+__device__ __forceinline__ int x_offset(int row, int cc)
+{
+    const int bank_row = row >> 1;
+    const int pos = (((row & 1) << 3) | cc) ^ (bank_row & 15);
+    return (bank_row * 16 + pos) * 16;
+}
 
-template <int VEC, typename CodeT>
+// s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
+// compiler knows nothing about this transfer, so every consumer sits behind an explicit
+// wait_vmcnt + barrier.  `lds_base` must be wave-uniform.
+__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(sbase)
+                 : "memory");
+}
+
+// 16-byte global load into registers outside the compiler's vmcnt bookkeeping (so that its own
+// waits never drain the LDS-bound loads in flight).  The result must not be touched before a
+// wait_vmcnt that covers it; pin_loaded() ties that wait to the registers.
+__device__ __forceinline__ uint4_t load_16_untracked(const void *p)
+{
+    uint4_t v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int NB_>
+__device__ __forceinline__ void pin_loaded(uint4_t (&r)[NB_])
+{
+#pragma unroll
+    for (int i = 0; i < NB_; i++) asm volatile("" : "+v"(r[i]));
+}
+
+template <int VEC, typename CodeT, bool TAIL, int NS>
 __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__restrict__ x,
                                                               const CodeT *__restrict__ codes,
                                                               const half_t *__restrict__ cb,
@@ -85,91 +136,80 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                                                               int tiles_n, int cb_lds_count)
 {
     typedef PrefillCfg<VEC, CodeT> C;
+    static_assert(NS == 3 || NS == 4, "three or four X stages");
+    constexpr int D = NS - 1;                 // X loads run D stages ahead of the MFMAs
+    constexpr int kInFlight = (D - 2) * kChunksPerThread;  // loads allowed to stay in flight at a stage end
     extern __shared__ __align__(16) uint8_t smem[];
-    uint8_t *xbuf = smem;                       // 2 stages
-    uint8_t *cb_lds = smem + 2 * kStageBytes;   // cb_lds_count codebooks
+    constexpr int kCbBase = NS * kStageBytes;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, kg = lane >> 5;
     const int J = K / VEC;
     const int cb_bytes = entries * VEC * 2;
 
-    // Tile mapping.  Consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD
-    // a contiguous band of tile columns so that its L2 sees one set of code rows and the X
-    // rows are re-read by neighbours at about the same time.
+    // Tile mapping.  Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
+    // Re-number them so that an XCD works on consecutive tiles of the (row band major) tile
+    // order: its workgroups then share a few 256-row bands of X, the large operand.
     int wg = blockIdx.x;
     const int n_wg = tiles_m * tiles_n;
-    {
-        const int xcd = wg & 7, idx = wg >> 3;
-        const int per_xcd = (n_wg + 7) >> 3;
-        const int lin = xcd * per_xcd + idx;
-        wg = (lin < n_wg && (n_wg & 7) == 0) ? lin : wg;
-    }
-    const int tm = wg % tiles_m, tn = wg / tiles_m;
+    if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+    const int tm = wg / tiles_n, tn = wg % tiles_n;
     const int m0 = tm * BM, n0 = tn * BN;
+    const int n_super = (K + C::K_SUPER - 1) / C::K_SUPER;
+    const int n_stage = n_super * C::STAGES;
 
-    // ---- codebooks of this tile's rows -> LDS ------------------------------------------
+    // ---- per-lane W rows, codebook bases and code streams ---------------------------------
     const int g_first = n0 / rows_per_cb;
-    {
-        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g_first * entries * VEC);
-        const int n16 = cb_lds_count * cb_bytes / 16;
-        const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
-        for (int i = tid; i < n16; i += kThreads)
-            if (i < g_total_16) reinterpret_cast<uint4_t *>(cb_lds)[i] = src[i];
-    }
-
-    // Per-lane W rows and codebook bases for the NB column blocks of this wave.
     uint32_t book[NB];  // byte offset of the lane's codebook inside smem
     const CodeT *code_row[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
         const int n = min(n0 + wn * WN + nb * 32 + l32, N - 1);
-        book[nb] = 2 * kStageBytes + (n / rows_per_cb - g_first) * cb_bytes;
+        book[nb] = kCbBase + (n / rows_per_cb - g_first) * cb_bytes;
         code_row[nb] = codes + (int64_t)n * J;
     }
+    auto issue_codes = [&](int super, uint4_t (&dst)[NB]) {
+        super = min(super, n_super - 1);  // past the end: harmless re-reads instead of branches
+        int k = super * C::K_SUPER + kg * C::K_LANE;
+        if (TAIL && k >= K) k = 0;  // k-group 1 of a partial last super stage: any valid codes (operand is zeroed)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) dst[nb] = load_16_untracked(code_row[nb] + k / VEC);
+    };
 
-    // ---- X staging: thread -> (row, chunk) of each stage ---------------------------------
-    // chunk id q = i*256 + tid; row = q/8, cc = q%8 (k-group cc/4, step cc%4).
-    const half_t *x_src[kChunksPerThread];
-    int x_dst[kChunksPerThread];
-    int x_koff[kChunksPerThread];
+    // ---- X staging: global -> LDS directly ------------------------------------------------
+    // Load i of wave w fills the 64 consecutive 16-byte slots [(4i+w)*64, +64) of a stage buffer;
+    // the lane looks up which (row, chunk) lives in its slot under the swizzle and reads that.
+    uint32_t x_voff[kChunksPerThread];
 #pragma unroll
     for (int i = 0; i < kChunksPerThread; i++) {
-        const int q = i * kThreads + tid;
-        const int row = q >> 3, cc = q & 7;
-        const int gm = min(m0 + row, M - 1);
-        x_koff[i] = (cc >> 2) * C::K_LANE + (cc & 3) * 8;
-        x_src[i] = x + (int64_t)gm * K + x_koff[i];
-        x_dst[i] = x_slot(row, cc) * 16;
+        const int slot = (4 * i + wave) * 64 + lane;
+        const int bank_row = slot >> 4;
+        const int v = (slot & 15) ^ (bank_row & 15);
+        const int row = 2 * bank_row + (v >> 3), cc = v & 7;
+        const int gm = min(m0 + row, M - 1) - m0;
+        const int koff = (cc >> 2) * C::K_LANE + (cc & 3) * 8;
+        x_voff[i] = (uint32_t)(((int64_t)gm * K + koff) * 2);
     }
-    const int n_super = (K + C::K_SUPER - 1) / C::K_SUPER;
-    const int n_stage = n_super * C::STAGES;
-
-    uint4_t xreg[kChunksPerThread];
-    auto issue_x = [&](int stage) {
-        const int kbase = (stage / C::STAGES) * C::K_SUPER + (stage % C::STAGES) * 32;
+    const half_t *x_tile = x + (int64_t)m0 * K;
+    auto issue_x = [&](int stage, int buf) {
+        stage = min(stage, n_stage - 1);
+        const int super = stage / C::STAGES;
+        int kbase = super * C::K_SUPER + (stage % C::STAGES) * 32;
+        const half_t *sbase = x_tile + kbase;
+        if (TAIL && super == n_super - 1) {
+            // k-group 1 of the partial last super stage lies past K: read k-group 0's bytes again.
 #pragma unroll
-        for (int i = 0; i < kChunksPerThread; i++) {
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (stage < n_stage && kbase + x_koff[i] < K) v = ld_global_16(x_src[i] + kbase);
-            xreg[i] = v;
-        }
-    };
-    auto commit_x = [&](int buf) {
+            for (int i = 0; i < kChunksPerThread; i++) {
+                const int slot = (4 * i + wave) * 64 + lane;
+                const int hi = (((slot & 15) ^ ((slot >> 4) & 15)) >> 2) & 1;
+                load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, x_voff[i] - (hi ? C::K_LANE * 2 : 0), sbase);
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < kChunksPerThread; i++)
-            *reinterpret_cast<uint4_t *>(xbuf + buf * kStageBytes + x_dst[i]) = xreg[i];
-    };
-    uint4_t cw[NB], cw_next[NB];
-    auto issue_codes = [&](int super, uint4_t (&dst)[NB]) {
-        const int k = super * C::K_SUPER + kg * C::K_LANE;
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (super < n_super && k < K) v = ld_global_16(code_row[nb] + k / VEC);
-            dst[nb] = v;
+            for (int i = 0; i < kChunksPerThread; i++)
+                load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, x_voff[i], sbase);
         }
     };
 
@@ -181,70 +221,146 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[nb][mb][r] = 0.f;
 
-    // ---- prologue ------------------------------------------------------------------------
-    issue_codes(0, cw_next);
-    issue_x(0);
-    commit_x(0);
-    issue_x(1);
+    // Operand read offsets inside a stage buffer: row = wm*128 + mb*32 + l32, chunk = kg*4 + s.
+    int x_rd[MB][4];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) x_rd[mb][s] = x_offset(wm * WM + mb * 32 + l32, kg * 4 + s);
+
+    half8_t wop[2][NB], xop[2][MB];
+    auto fetch_operands = [&](int set, int buf, const uint4_t (&c)[NB], int t, int s, bool last_super) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            half8_t w = gather8<VEC, CodeT>(smem + book[nb], c[nb], (t * 4 + s) * C::CPO);
+            if (TAIL && last_super && kg == 1) w = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            wop[set][nb] = w;
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+            xop[set][mb] = *reinterpret_cast<const half8_t *>(smem + buf * kStageBytes + x_rd[mb][s]);
+    };
+
+    // ---- prologue --------------------------------------------------------------------------
+    uint4_t cw[NB], cw1[NB], cw2[NB];  // codes of super stage S, S+1, S+2
+    issue_codes(0, cw);
+    issue_codes(1, cw1);
+    issue_codes(2, cw2);
+#pragma unroll
+    for (int d = 0; d < D; d++) issue_x(d, d);
+    {
+        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g_first * entries * VEC);
+        const int n16 = cb_lds_count * cb_bytes / 16;
+        const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
+        for (int i = tid; i < n16; i += kThreads)
+            if (i < g_total_16) reinterpret_cast<uint4_t *>(smem + kCbBase)[i] = src[i];
+    }
+    wait_vmcnt<0>();
+    pin_loaded(cw);
+    pin_loaded(cw1);
+    pin_loaded(cw2);
     __syncthreads();
 
-    // Operand read offsets inside a stage buffer: row = wm*128 + mb*32 + l32, chunk = kg*4 + s.
-    int x_rd[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) x_rd[mb] = wm * WM + mb * 32 + l32;
+    int buf = 0;  // buffer of the current stage; stage+j lives in (buf + j) % NS
+    fetch_operands(0, buf, cw, 0, 0, n_super == 1);
 
     for (int super = 0; super < n_super; super++) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) cw[nb] = cw_next[nb];
-        issue_codes(super + 1, cw_next);
+        const bool last_super = super == n_super - 1;
+        const bool next_last = super + 1 == n_super - 1;
 #pragma unroll
         for (int t = 0; t < C::STAGES; t++) {
             const int stage = super * C::STAGES + t;
-            const int buf = stage & 1;
-            // Stage+1 data is in registers: park it in the other buffer (all waves finished
-            // reading that buffer at the barrier that ended the previous iteration), then
-            // start the loads of stage+2.
-            commit_x(buf ^ 1);
-            issue_x(stage + 2);
-            const uint8_t *xs = xbuf + buf * kStageBytes;
+            const int buf_next = buf + 1 == NS ? 0 : buf + 1;
+            // Stage+D goes into the buffer that was read during stage-1 (every wave has passed the
+            // barrier that ended it).
+            issue_x(stage + D, buf == 0 ? NS - 1 : buf - 1);
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                half8_t wop[NB], xop[MB];
-#pragma unroll
-                for (int nb = 0; nb < NB; nb++)
-                    wop[nb] = gather8<VEC, CodeT>(smem + book[nb], cw[nb], (t * 4 + s) * C::CPO);
-#pragma unroll
-                for (int mb = 0; mb < MB; mb++)
-                    xop[mb] = *reinterpret_cast<const half8_t *>(xs + x_slot(x_rd[mb], kg * 4 + s) * 16);
+                const int cur = s & 1;
+                if (s < 3)
+                    fetch_operands(cur ^ 1, buf, cw, t, s + 1, last_super);
+                else if (t + 1 < C::STAGES)
+                    fetch_operands(cur ^ 1, buf_next, cw, t + 1, 0, last_super);
+                else
+                    fetch_operands(cur ^ 1, buf_next, cw1, 0, 0, next_last);
+                // Keep the fetches of the next step ahead of this step's MFMAs: left alone, the
+                // scheduler sinks each load to just before its first use and the LDS latency
+                // lands on the matrix pipe.
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++)
 #pragma unroll
                     for (int mb = 0; mb < MB; mb++)
-                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wop[nb], xop[mb], acc[nb][mb], 0, 0, 0);
+                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wop[cur][nb], xop[cur][mb], acc[nb][mb], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            // Publish stage+2: its loads (issued D-2 stages ago) must have landed in every wave.
+            wait_vmcnt<kInFlight>();
+            pin_loaded(cw2);
             __syncthreads();
+            buf = buf_next;
         }
-    }
-
-    // ---- epilogue: D[i][j], i = W row = 8*(r/4) + 4*kg + r%4, j = X row = l32 --------------
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        const int m = m0 + wm * WM + mb * 32 + l32;
-        if (m >= M) continue;
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
+            cw[nb] = cw1[nb];
+            cw1[nb] = cw2[nb];
+        }
+        issue_codes(super + 3, cw2);
+    }
+    // Drain the clamped loads still in flight before the stage buffers are reused.
+    wait_vmcnt<0>();
+    pin_loaded(cw2);
+    __syncthreads();
+
+    // ---- epilogue: D[i][j], i = W row = 8*(r/4) + 4*kg + r%4, j = X row = l32 --------------
+    if ((N & 7) == 0) {
+        // Through the LDS: each wave transposes its 128x128 fp16 block, 64 rows at a time, in a
+        // private region (row pitch 272 bytes) and stores 256-byte row segments.
+        constexpr int kPitch = 272;
+        uint8_t *stage_out = smem + wave * (64 * kPitch);
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int n = n0 + wn * WN + nb * 32 + 8 * q + 4 * kg;
-                half_t *dst = y + (int64_t)m * N + n;
-                if ((N & 3) == 0 && n + 3 < N) {
-                    half4_t h = {(half_t)acc[nb][mb][4 * q], (half_t)acc[nb][mb][4 * q + 1],
-                                 (half_t)acc[nb][mb][4 * q + 2], (half_t)acc[nb][mb][4 * q + 3]};
-                    *reinterpret_cast<half4_t *>(dst) = h;
-                } else {
+        for (int h = 0; h < 2; h++) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if (n + r < N) dst[r] = (half_t)acc[nb][mb][4 * q + r];
+            for (int mbh = 0; mbh < 2; mbh++) {
+                const int mb = 2 * h + mbh;
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        half4_t hv = {(half_t)acc[nb][mb][4 * q], (half_t)acc[nb][mb][4 * q + 1],
+                                      (half_t)acc[nb][mb][4 * q + 2], (half_t)acc[nb][mb][4 * q + 3]};
+                        *reinterpret_cast<half4_t *>(stage_out + (mbh * 32 + l32) * kPitch + (nb * 32 + 8 * q + 4 * kg) * 2) = hv;
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int row = i * 4 + (lane >> 4), c = lane & 15;
+                const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
+                const int m = m0 + wm * WM + h * 64 + row;
+                const int n = n0 + wn * WN + c * 8;
+                if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) {
+            const int m = m0 + wm * WM + mb * 32 + l32;
+            if (m >= M) continue;
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int n = n0 + wn * WN + nb * 32 + 8 * q + 4 * kg;
+                    half_t *dst = y + (int64_t)m * N + n;
+                    if ((N & 3) == 0 && n + 3 < N) {
+                        half4_t h = {(half_t)acc[nb][mb][4 * q], (half_t)acc[nb][mb][4 * q + 1],
+                                     (half_t)acc[nb][mb][4 * q + 2], (half_t)acc[nb][mb][4 * q + 3]};
+                        *reinterpret_cast<half4_t *>(dst) = h;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (n + r < N) dst[r] = (half_t)acc[nb][mb][4 * q + r];
+                    }
                 }
             }
         }
@@ -264,13 +380,25 @@ int codebooks_per_tile(const ProblemB &p)
     return n < p.n_codebooks ? n : p.n_codebooks;
 }
 
+size_t lds_bytes(const ProblemB &p, int n_stages)
+{
+    return (size_t)n_stages * kStageBytes + (size_t)codebooks_per_tile(p) * p.entries * p.vec * 2;
+}
+
+// Four X stages when the codebooks leave room for them, else three.
+int pick_stages(const ProblemB &p) { return lds_bytes(p, 4) <= kLdsLimit ? 4 : 3; }
+
 template <int VEC, typename CodeT>
 hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s)
 {
+    typedef PrefillCfg<VEC, CodeT> C;
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     const int n_cb = codebooks_per_tile(p);
-    const size_t smem = (size_t)2 * kStageBytes + (size_t)n_cb * p.entries * VEC * 2;
-    auto kern = prefill_kernel<VEC, CodeT>;
+    const int ns = pick_stages(p);
+    const size_t smem = lds_bytes(p, ns);
+    const bool tail = (p.K % C::K_SUPER) != 0;
+    auto kern = ns == 4 ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
+                        : (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>);
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
@@ -293,7 +421,7 @@ bool prefill_supports(const ProblemB &p)
     if (p.M < 1 || p.N < 1 || p.K < 1) return false;
     if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
     if (((size_t)p.entries * p.vec * 2) % 16 != 0) return false;
-    if ((size_t)2 * kStageBytes + (size_t)codebooks_per_tile(p) * p.entries * p.vec * 2 > kLdsLimit) return false;
+    if (lds_bytes(p, 3) > kLdsLimit) return false;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
     case 8: return u8 ? prefill_cfg_supports<8, uint8_t>(p) : prefill_cfg_supports<8, uint16_t>(p);
