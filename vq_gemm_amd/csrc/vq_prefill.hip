@@ -193,24 +193,20 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         x_voff[i] = (uint32_t)(((int64_t)gm * K + koff) * 2);
     }
     const half_t *x_tile = x + (int64_t)m0 * K;
-    auto issue_x = [&](int stage, int buf) {
-        stage = min(stage, n_stage - 1);
+    // Load i (0..7) of a stage: one 16-byte chunk per lane, 1 KB per wave.
+    auto issue_x_one = [&](int stage, int buf, int i) {
+        stage = min(stage, n_stage - 1);  // past the end: harmless re-reads instead of branches
         const int super = stage / C::STAGES;
-        int kbase = super * C::K_SUPER + (stage % C::STAGES) * 32;
-        const half_t *sbase = x_tile + kbase;
+        const half_t *sbase = x_tile + super * C::K_SUPER + (stage % C::STAGES) * 32;
+        uint32_t voff = x_voff[i];
         if (TAIL && super == n_super - 1) {
-            // k-group 1 of the partial last super stage lies past K: read k-group 0's bytes again.
-#pragma unroll
-            for (int i = 0; i < kChunksPerThread; i++) {
-                const int slot = (4 * i + wave) * 64 + lane;
-                const int hi = (((slot & 15) ^ ((slot >> 4) & 15)) >> 2) & 1;
-                load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, x_voff[i] - (hi ? C::K_LANE * 2 : 0), sbase);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kChunksPerThread; i++)
-                load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, x_voff[i], sbase);
+            // k-group 1 of the partial last super stage lies past K: read k-group 0's bytes again
+            // (that group's W operand is zeroed).
+            const int slot = (4 * i + wave) * 64 + lane;
+            const int hi = (((slot & 15) ^ ((slot >> 4) & 15)) >> 2) & 1;
+            voff -= hi ? C::K_LANE * 2 : 0;
         }
+        load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, voff, sbase);
     };
 
     float16_t acc[NB][MB];
@@ -247,7 +243,9 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     issue_codes(1, cw1);
     issue_codes(2, cw2);
 #pragma unroll
-    for (int d = 0; d < D; d++) issue_x(d, d);
+    for (int d = 0; d < D; d++)
+#pragma unroll
+        for (int i = 0; i < kChunksPerThread; i++) issue_x_one(d, d, i);
     {
         const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g_first * entries * VEC);
         const int n16 = cb_lds_count * cb_bytes / 16;
@@ -272,26 +270,42 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
             const int stage = super * C::STAGES + t;
             const int buf_next = buf + 1 == NS ? 0 : buf + 1;
             // Stage+D goes into the buffer that was read during stage-1 (every wave has passed the
-            // barrier that ended it).
-            issue_x(stage + D, buf == 0 ? NS - 1 : buf - 1);
+            // barrier that ended it); its eight loads are spread over the four steps.
+            const int buf_load = buf == 0 ? NS - 1 : buf - 1;
 #pragma unroll
             for (int s = 0; s < 4; s++) {
                 const int cur = s & 1;
+                // Fetch the operands of the next step and multiply this step's.  A wave issues in
+                // order and an MFMA holds the matrix pipe for 32 cycles, so the LDS reads and their
+                // address arithmetic are dealt out between the MFMAs instead of ahead of them.
                 if (s < 3)
                     fetch_operands(cur ^ 1, buf, cw, t, s + 1, last_super);
                 else if (t + 1 < C::STAGES)
                     fetch_operands(cur ^ 1, buf_next, cw, t + 1, 0, last_super);
                 else
                     fetch_operands(cur ^ 1, buf_next, cw1, 0, 0, next_last);
-                // Keep the fetches of the next step ahead of this step's MFMAs: left alone, the
-                // scheduler sinks each load to just before its first use and the LDS latency
-                // lands on the matrix pipe.
+                auto mfma = [&](int j) {
+                    const int nb = j / MB, mb = j % MB;
+                    acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wop[cur][nb], xop[cur][mb], acc[nb][mb], 0, 0, 0);
+                };
+#pragma unroll
+                for (int j = 0; j < 8; j++) mfma(j);
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // a few VALU (gather addresses)
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                issue_x_one(stage + D, buf_load, 2 * s);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++)
+                for (int j = 8; j < 12; j++) mfma(j);
+                __builtin_amdgcn_sched_barrier(0);
+                issue_x_one(stage + D, buf_load, 2 * s + 1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int mb = 0; mb < MB; mb++)
-                        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wop[cur][nb], xop[cur][mb], acc[nb][mb], 0, 0, 0);
+                for (int j = 12; j < 16; j++) mfma(j);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // Publish stage+2: its loads (issued D-2 stages ago) must have landed in every wave.
