@@ -1,0 +1,222 @@
+"""Benchmark of the VQ-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only-main]
+
+One "step" is one fused VQ-GEMM launch over one weight matrix.  The headline workload is the
+decode GEMV (M=1, K=4096, N=4096, 8-vectors, uint8 codes, one 256x8 codebook).  So that the
+2 MB of codes really stream from HBM, the steps rotate over a pool of distinct code matrices
+larger than the L2 and the 256 MB Infinity Cache; the launches are captured in HIP graphs so that
+host launch overhead does not pace a microsecond-scale kernel, and timed with HIP events recorded
+on the stream the kernels run on.  Inputs are resident in HBM before the timed region.
+
+Printed: ONE JSON line (rank 0).  `value` is the decode configuration's effective bandwidth:
+the bytes an uncompressed fp16 GEMV would have had to stream (fp16 weights + X + Y) per
+second.  `roofline` prices the same kernel against HBM peak on its *algorithmic* bytes (codes
++ codebook + X + Y).  Next to it: the hipBLASLt fp16 GEMM on the dequantised weights timed by
+the same loop, the other measured configurations, and the reference math on the host CPU
+(torch gather + fp32 matmul, all cores) on a bounded sample.
+
+Counterpart of the reference harness bench.py:62-171 (same operator call, the accuracy and
+determinism reports), with timing moved out of the kernel wrappers into the harness.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+FP16_MFMA_PEAK_TFLOPS = 2500.0
+POOL_BYTES = 640 << 20  # distinct code matrices rotated through by the bandwidth-bound configs
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the single-GPU VQ-GEMM path; this build has no multi-GPU leg "
+              "(the path shards along N without any exchange). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from vq_gemm_amd import cabi
+    from vq_gemm_amd.problems import CONFIGS, make_problem
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    cabi.lib()      # fail loudly if the HIP library is missing
+    cabi.ref_lib()
+
+    def barrier():
+        torch.cuda.synchronize()
+
+    def time_launches(launch, n_bufs, steps, warmup, chunk=500):
+        """Average seconds per launch of `launch(i)` (i rotates over n_bufs), HIP graphs + events."""
+        stream = torch.cuda.Stream()   # default priority
+        with torch.cuda.stream(stream):
+            for i in range(max(warmup, 1)):
+                launch(i % n_bufs)
+            stream.synchronize()
+            graphs = []
+            done = 0
+            while done < steps:
+                c = min(chunk, steps - done)
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for i in range(c):
+                        launch((done + i) % n_bufs)
+                graphs.append(g)
+                done += c
+            graphs[0].replay()          # first replay uploads the graph: keep it out of the timing
+            stream.synchronize()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            barrier()
+            e0.record(stream)
+            for g in graphs:
+                g.replay()
+            e1.record(stream)
+            e1.synchronize()
+            barrier()
+            return e0.elapsed_time(e1) * 1e-3 / steps
+
+    def bench_config(name, steps, warmup, cold_pool):
+        spec = CONFIGS[name]
+        x, codes, cb = make_problem(spec, seed=42, device=dev)
+        n_bufs = max(1, min(512, POOL_BYTES // max(spec.code_bytes, 1))) if cold_pool else 1
+        pool = [codes]
+        gen = torch.Generator(device=dev).manual_seed(1234)
+        for _ in range(n_bufs - 1):
+            c = torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev, dtype=torch.int32)
+            pool.append(c.to(spec.code_dtype))
+        y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
+        t_cold = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[i], cb, out=y), n_bufs, steps, warmup)
+        t_warm = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[0], cb, out=y), 1, steps, warmup) if cold_pool else t_cold
+        # hipBLASLt fp16 on the dequantised weights (a pool of them for the cold protocol)
+        n_wbufs = max(1, min(n_bufs, POOL_BYTES * 2 // spec.dense_weight_bytes)) if cold_pool else 1
+        wpool = [cabi.dequant_b(pool[i], cb) for i in range(n_wbufs)]
+        t_blas = time_launches(lambda i: cabi.ref_gemm_f16(x, wpool[i], w_is_nk=True, out=y), n_wbufs, steps, warmup)
+        res = {
+            "M": spec.M, "K": spec.K, "N": spec.N, "vec": spec.vec, "code_bits": spec.code_bits,
+            "entries": spec.entries, "n_codebooks": spec.n_codebooks,
+            "variant": cabi.VARIANT_NAMES[cabi.select_variant_b(spec.M, spec.K, spec.N, spec.vec, spec.entries,
+                                                                 spec.n_codebooks, spec.code_bits)],
+            "us": t_cold * 1e6, "us_warm_cache": t_warm * 1e6,
+            "tflops": spec.flops / t_cold / 1e12,
+            "tflops_2p40": spec.flops / t_cold / 1024 ** 4,   # the reference's own divisor (strategy_1/src.cu:396)
+            "algorithmic_gbps": spec.algorithmic_bytes / t_cold / 1e9,
+            "effective_gbps": (spec.dense_weight_bytes + 2 * spec.M * (spec.K + spec.N)) / t_cold / 1e9,
+            "hbm_roofline_frac": spec.algorithmic_bytes / t_cold / 1e9 / HBM_PEAK_GBPS,
+            "mfma_roofline_frac": spec.flops / t_cold / 1e12 / FP16_MFMA_PEAK_TFLOPS,
+            "hipblaslt_us": t_blas * 1e6, "hipblaslt_tflops": spec.flops / t_blas / 1e12,
+            "speedup_vs_hipblaslt": t_blas / t_cold,
+            "code_buffers_rotated": n_bufs, "steps": steps,
+        }
+        # run-to-run determinism, as the reference harness reports it (bench.py:118-132)
+        y0 = cabi.e2e_gemm_b(x, codes, cb).clone()
+        res["deterministic_5_runs"] = all(torch.equal(cabi.e2e_gemm_b(x, codes, cb), y0) for _ in range(4))
+        del pool, wpool
+        torch.cuda.empty_cache()
+        return res, (x, codes, cb, y0)
+
+    # ---- headline: decode GEMV ---------------------------------------------------------------
+    main_name = "C2"
+    main_res, (x, codes, cb, y_gpu) = bench_config(main_name, args.steps, args.warmup, cold_pool=True)
+    spec = CONFIGS[main_name]
+
+    others = {}
+    if not args.only_main:
+        others["C3"], _ = bench_config("C3", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        others["C1"], _ = bench_config("C1", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=False)
+        others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
+        others["C5"], _ = bench_config("C5", 10, 3, cold_pool=False)
+
+    # ---- CPU baseline: the reference math (gather + fp32 matmul) on the host cores -------------
+    cpu = None
+    if not args.skip_cpu:
+        import numpy as np
+
+        from oracle import torch_baseline
+        from oracle import vq_oracle as vo
+
+        xc, cc, cbc = x.cpu(), codes.cpu(), cb.cpu()
+        budget_s, reps, t_total = 12.0, 0, 0.0   # about 12 s of CPU work
+        best = float("inf")
+        y_cpu = None
+        while t_total < budget_s and reps < 5000:
+            t0 = time.perf_counter()
+            y_cpu = torch_baseline.vq_gemm_b(xc, cc, cbc)
+            dt = time.perf_counter() - t0
+            best = min(best, dt)
+            t_total += dt
+            reps += 1
+        mean = t_total / reps
+        e1, e2 = vo.rel_err(y_gpu.cpu().numpy(), y_cpu.numpy().astype(np.float64))
+        cpu = {
+            "value": (spec.dense_weight_bytes + 2 * spec.M * (spec.K + spec.N)) / mean / 1e9, "unit": "GB/s",
+            "cores": torch.get_num_threads(), "host_cpu_count": os.cpu_count(), "kind": "port",
+            "sample": f"{reps} full {main_name} GEMVs (dequant gather + fp32 matmul, torch CPU), {t_total:.1f} s; mean per step",
+            "ms_per_step": mean * 1e3, "best_ms_per_step": best * 1e3,
+            "gpu_vs_cpu_max_rel_err": e1, "gpu_vs_cpu_max_err_over_max": e2,
+        }
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "decode_c2_hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    t = main_res["us"] * 1e-6
+    out = {
+        "metric": "vq_gemm_decode_effective_bandwidth",
+        "value": main_res["effective_gbps"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "C2 decode GEMV: M=1 K=4096 N=4096, vec 8, uint8 codes [4096,512], one fp16 codebook [256,8]; "
+                               f"cold HBM (rotating {main_res['code_buffers_rotated']} code matrices), fp32 accumulate",
+                   "kernel": main_res["variant"]},
+        "roofline": {"bound": "hbm", "achieved": spec.algorithmic_bytes / t / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": spec.algorithmic_bytes / t / 1e9 / HBM_PEAK_GBPS, "traffic": traffic,
+                     "algorithmic_bytes_per_launch": spec.algorithmic_bytes,
+                     "kernel_us": main_res["us"], "kernel_us_warm_cache": main_res["us_warm_cache"]},
+        "cpu_baseline": cpu,
+        "tflops": main_res["tflops"],
+        "hipblaslt": {"us": main_res["hipblaslt_us"], "tflops": main_res["hipblaslt_tflops"],
+                      "speedup_vs_hipblaslt": main_res["speedup_vs_hipblaslt"]},
+        "deterministic_5_runs": main_res["deterministic_5_runs"],
+        "other_configs": others,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

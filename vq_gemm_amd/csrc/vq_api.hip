@@ -5,6 +5,9 @@
 
 #include <atomic>
 #include <limits.h>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace vq {
 
@@ -20,6 +23,22 @@ int device_cu_count()
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
     cache[dev].store(cus, std::memory_order_relaxed);
     return cus;
+}
+
+hipError_t ensure_dynamic_lds(const void *kernel, size_t bytes)
+{
+    if (bytes <= 48 * 1024) return hipSuccess;  // within the default limit
+    static std::mutex mu;
+    static std::map<std::pair<int, const void *>, size_t> granted;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mu);
+    size_t &g = granted[{dev, kernel}];
+    if (bytes <= g) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) g = bytes;
+    return e;
 }
 
 namespace {

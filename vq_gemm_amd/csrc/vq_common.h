@@ -71,4 +71,8 @@ hipError_t launch_gemm_nt(const half_t *x, const half_t *w, half_t *y, int M, in
 
 int device_cu_count();
 
+// Raises a kernel's dynamic-LDS limit when `bytes` needs it; remembers what was granted per
+// (device, kernel) so that steady-state launches make no attribute call.
+hipError_t ensure_dynamic_lds(const void *kernel, size_t bytes);
+
 }  // namespace vq

@@ -203,11 +203,8 @@ hipError_t launch_decode_typed(const ProblemB &p, hipStream_t s)
     const int cb_bytes = p.entries * VEC * 2;
     const size_t smem = (size_t)((cb_bytes + 15) & ~15) + (size_t)2 * n_waves * 64 * sizeof(float4_t);
     auto kern = decode_kernel<VEC, CodeT>;
-    if (smem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return e;
-    }
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
                        p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb, tiles_per_wg, n_tiles, n_chunks);
     return hipGetLastError();

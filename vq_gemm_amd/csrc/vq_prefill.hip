@@ -413,8 +413,7 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s)
     const bool tail = (p.K % C::K_SUPER) != 0;
     auto kern = ns == 4 ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
                         : (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>);
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
                        static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb,
