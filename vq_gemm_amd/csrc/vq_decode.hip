@@ -36,6 +36,7 @@ struct DecodeCfg {
     static constexpr int K_LANE = CPL * VEC;             // k covered by one lane load
     static constexpr int K_WAVE = 4 * K_LANE;            // k covered by one wave load (4 k-groups)
     static constexpr int LPT = kSliceK / K_WAVE;         // lane loads per slice
+    static constexpr int PF = LPT <= 2 ? 4 : (LPT <= 4 ? 3 : 2);  // (tile, chunk) code loads kept in flight
     static_assert(CPO >= 1 && SPL >= 1 && LPT >= 1 && LPT * SPL == kSteps, "unsupported code layout");
 };
 
@@ -76,18 +77,40 @@ __device__ __forceinline__ half8_t gather_operand(const uint8_t *cb_lds, const u
     }
 }
 
-template <int VEC, typename CodeT>
-__global__ __launch_bounds__(1024) void decode_kernel(const half_t *__restrict__ x,
+constexpr int kStagePitch = 1024 + 16;  // bytes per staged X row slice; the pad spreads rows over the banks
+
+// s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");  // keep the compiler from moving LDS reads above the wait
+}
+
+// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].
+// `lds_base` must be wave-uniform; completion is only visible through vmcnt.
+__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(sbase)
+                 : "memory");
+}
+
+// stage_off >= 0: the X slices are staged through the LDS at that offset (n_chunks == 1 only);
+// `aliased` says that the staging area overlaps the codebook, which is then loaded afterwards.
+template <int VEC, typename CodeT, int MAX_THREADS>
+__global__ __launch_bounds__(MAX_THREADS) void decode_kernel(const half_t *__restrict__ x,
                                                       const CodeT *__restrict__ codes,
                                                       const half_t *__restrict__ cb,
                                                       half_t *__restrict__ y, int M, int K, int N,
-                                                      int entries, int rows_per_cb, int tiles_per_wg,
-                                                      int n_tiles, int n_chunks)
+                                                      int entries, int rows_per_cb, int n_tiles,
+                                                      int n_chunks, int stage_off, int aliased)
 {
     typedef DecodeCfg<VEC, CodeT> C;
     extern __shared__ __align__(16) uint8_t smem[];
     const int n_waves = blockDim.x >> 6;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int r16 = lane & 15;  // W row within the tile (A operand) / X row m (B operand)
     const int kq = lane >> 4;   // k-group of the lane, 0..3
@@ -96,8 +119,9 @@ __global__ __launch_bounds__(1024) void decode_kernel(const half_t *__restrict__
     uint8_t *cb_lds = smem;
     float4_t *red = reinterpret_cast<float4_t *>(smem + ((cb_bytes + 15) & ~15));
 
-    const int tile_begin = blockIdx.x * tiles_per_wg;
-    const int tile_end = min(tile_begin + tiles_per_wg, n_tiles);
+    // Balanced contiguous split of the tiles over the workgroups.
+    const int tile_begin = (int)(((int64_t)blockIdx.x * n_tiles) / gridDim.x);
+    const int tile_end = (int)(((int64_t)(blockIdx.x + 1) * n_tiles) / gridDim.x);
     if (tile_begin >= tile_end) return;
 
     // k of MFMA step s for this lane inside a slice that starts at k0.
@@ -123,71 +147,144 @@ __global__ __launch_bounds__(1024) void decode_kernel(const half_t *__restrict__
             cw[t] = v;
         }
     };
+    auto load_codebook = [&](int g) {
+        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g * entries * VEC);
+        for (int i = threadIdx.x; i < cb_bytes / 16; i += blockDim.x) reinterpret_cast<uint4_t *>(cb_lds)[i] = src[i];
+    };
 
     const int chunk_k = n_waves * kSliceK;
-    uint4_t cw_next[C::LPT];
-    load_codes(tile_begin, wave * kSliceK, cw_next);
-    if (n_chunks == 1) load_x(wave * kSliceK);
+    // The unit of work is a (tile, chunk) pair; the codes of the next PF units are always in
+    // flight, so a workgroup with only a few tiles pays the memory latency once, not per tile.
+    const int q_begin = tile_begin * n_chunks, q_end = tile_end * n_chunks;
+    // The 1024-thread build has half the registers per lane: shallower prefetch, no codebook registers.
+    constexpr int PF = MAX_THREADS > 512 ? (C::LPT <= 2 ? 2 : 1) : C::PF;
+    uint4_t cwq[PF][C::LPT];
+    auto load_unit = [&](int q, uint4_t (&cw)[C::LPT]) {
+        const int tile = q / n_chunks, chunk = q - tile * n_chunks;
+        load_codes(tile, chunk * chunk_k + wave * kSliceK, cw);
+    };
+#pragma unroll
+    for (int u = 0; u < PF; u++)
+        if (q_begin + u < q_end) load_unit(q_begin + u, cwq[u]);
+
+    // Small codebooks are fetched into registers up front so that their latency overlaps the
+    // X staging even when the staging area and the codebook share LDS space.
+    const int cb_chunks = cb_bytes / 16;
+    const bool cb_in_regs = MAX_THREADS <= 512 && cb_chunks <= 4 * (int)blockDim.x;
+    uint4_t cb_regs[4];
+    auto fetch_codebook = [&](int g) {
+        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g * entries * VEC);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = threadIdx.x + j * blockDim.x;
+            cb_regs[j] = i < cb_chunks ? src[i] : uint4_t{0u, 0u, 0u, 0u};
+        }
+    };
+    auto store_codebook = [&]() {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < cb_chunks) reinterpret_cast<uint4_t *>(cb_lds)[i] = cb_regs[j];
+        }
+    };
 
     int cur_cb = -1;
-    int parity = 0;
-    for (int tile = tile_begin; tile < tile_end; tile++) {
-        const int g = (tile * kTileN) / rows_per_cb;
-        if (g != cur_cb) {
-            // (Re)load the codebook of this row block into the LDS.
-            if (cur_cb >= 0) __syncthreads();
-            const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g * entries * VEC);
-            for (int i = threadIdx.x; i < cb_bytes / 16; i += blockDim.x)
-                reinterpret_cast<uint4_t *>(cb_lds)[i] = src[i];
-            __syncthreads();
-            cur_cb = g;
+    if (stage_off >= 0) {
+        // X -> registers through the LDS.  A lane needs 16-byte pieces scattered over its row
+        // slice; fetched directly, every load instruction touches dozens of cache lines and
+        // uses 16 bytes of each.  Instead the wave copies each row slice (1 KB, contiguous) into
+        // a private LDS window and the lanes pick their pieces from there.
+        const int k0 = wave * kSliceK;
+        const uint32_t win = stage_off + wave * M * kStagePitch;
+        const int kl = k0 + 8 * lane;
+        for (int i = 0; i < M; i++)
+            load_to_lds_16(win + i * kStagePitch, (uint32_t)((i * K + (kl < K ? kl : 0)) * 2), x);
+        const int g = (tile_begin * kTileN) / rows_per_cb;
+        if (cb_in_regs) fetch_codebook(g);
+        else if (!aliased) load_codebook(g);
+        wait_vmcnt<0>();
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            const int k = step_k(k0, s);
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (r16 < M && k < K) v = *reinterpret_cast<const uint4_t *>(smem + win + r16 * kStagePitch + (k - k0) * 2);
+            xr[s] = as_half8(v);
         }
-        float4_t acc = {0.f, 0.f, 0.f, 0.f};
-        for (int chunk = 0; chunk < n_chunks; chunk++) {
-            const int k0 = chunk * chunk_k + wave * kSliceK;
+        if (aliased) __syncthreads();  // every wave has picked up its X before the codebook overwrites it
+        if (cb_in_regs) store_codebook();
+        else if (aliased) load_codebook(g);
+        __syncthreads();
+        cur_cb = g;
+    } else if (n_chunks == 1) {
+        load_x(wave * kSliceK);
+    }
+
+    int parity = 0;
+    // Four accumulators: consecutive MFMAs do not wait on each other's result.
+    float4_t acc[4];
+#pragma unroll
+    for (int a = 0; a < 4; a++) acc[a] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int qb = q_begin; qb < q_end; qb += PF) {
+#pragma unroll
+        for (int u = 0; u < PF; u++) {
+            const int q = qb + u;
+            if (q >= q_end) break;
+            const int tile = q / n_chunks, chunk = q - tile * n_chunks;
+            const int g = (tile * kTileN) / rows_per_cb;
+            if (g != cur_cb) {
+                // (Re)load the codebook of this row block into the LDS.
+                if (cur_cb >= 0) __syncthreads();
+                load_codebook(g);
+                __syncthreads();
+                cur_cb = g;
+            }
             uint4_t cw[C::LPT];
 #pragma unroll
-            for (int t = 0; t < C::LPT; t++) cw[t] = cw_next[t];
-            // Prefetch the next (tile, chunk) codes while this one is consumed.
-            {
-                int ntile = tile, nchunk = chunk + 1;
-                if (nchunk == n_chunks) { nchunk = 0; ntile = tile + 1; }
-                if (ntile < tile_end) load_codes(ntile, nchunk * chunk_k + wave * kSliceK, cw_next);
-            }
-            if (n_chunks > 1) load_x(k0);
+            for (int t = 0; t < C::LPT; t++) cw[t] = cwq[u][t];
+            if (q + PF < q_end) load_unit(q + PF, cwq[u]);
+            if (n_chunks > 1) load_x(chunk * chunk_k + wave * kSliceK);
 #pragma unroll
             for (int s = 0; s < kSteps; s++) {
                 const half8_t a = gather_operand<VEC, CodeT>(cb_lds, cw[s / C::SPL], (s % C::SPL) * C::CPO);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xr[s], acc, 0, 0, 0);
+                acc[s & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xr[s], acc[s & 3], 0, 0, 0);
             }
-        }
-        // Sum the K slices of the waves: slot (parity, wave, lane).
-        red[(parity * n_waves + wave) * 64 + lane] = acc;
-        __syncthreads();
-        if (wave == (tile % n_waves)) {
-            float4_t sum = red[(parity * n_waves) * 64 + lane];
-            for (int w = 1; w < n_waves; w++) {
-                const float4_t v = red[(parity * n_waves + w) * 64 + lane];
-                sum += v;
-            }
-            // D[i][j]: j = lane % 16 is the X row m, i = 4*(lane/16) + r is the W row.
-            const int m = r16;
-            const int n = tile * kTileN + 4 * kq;
-            if (m < M) {
-                half_t *dst = y + (int64_t)m * N + n;
-                if ((N & 3) == 0 && n + 3 < N) {
-                    half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
-                    *reinterpret_cast<half4_t *>(dst) = h;
-                } else {
+            if (chunk != n_chunks - 1) continue;
+
+            const float4_t part = (acc[0] + acc[1]) + (acc[2] + acc[3]);
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if (n + r < N) dst[r] = (half_t)sum[r];
+            for (int a = 0; a < 4; a++) acc[a] = float4_t{0.f, 0.f, 0.f, 0.f};
+            // Sum the K slices of the waves: slot (parity, wave, lane).
+            red[(parity * n_waves + wave) * 64 + lane] = part;
+            __syncthreads();
+            if (wave == (tile % n_waves)) {
+                float4_t sum = red[(parity * n_waves) * 64 + lane];
+                for (int w = 1; w < n_waves; w++) {
+                    const float4_t v = red[(parity * n_waves + w) * 64 + lane];
+                    sum += v;
+                }
+                // D[i][j]: j = lane % 16 is the X row m, i = 4*(lane/16) + r is the W row.
+                const int m = r16;
+                const int n = tile * kTileN + 4 * kq;
+                if (m < M) {
+                    half_t *dst = y + (int64_t)m * N + n;
+                    if ((N & 3) == 0 && n + 3 < N) {
+                        half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                        *reinterpret_cast<half4_t *>(dst) = h;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (n + r < N) dst[r] = (half_t)sum[r];
+                    }
                 }
             }
+            parity ^= 1;
         }
-        parity ^= 1;
     }
 }
+
+constexpr size_t kDecodeLdsLimit = 160 * 1024;
+constexpr size_t kStageMinBytes = 32 * 1024;
+constexpr size_t kDisjointBudget = 64 * 1024;  // keep at least two workgroups per CU when staging beside the codebook
 
 template <int VEC, typename CodeT>
 hipError_t launch_decode_typed(const ProblemB &p, hipStream_t s)
@@ -196,17 +293,36 @@ hipError_t launch_decode_typed(const ProblemB &p, hipStream_t s)
     const int n_waves = slices < kMaxWaves ? slices : kMaxWaves;
     const int n_chunks = (slices + n_waves - 1) / n_waves;
     const int n_tiles = (p.N + kTileN - 1) / kTileN;
-    const int target = device_cu_count() * 2;
-    int tiles_per_wg = (n_tiles + target - 1) / target;
-    if (tiles_per_wg < 1) tiles_per_wg = 1;
-    const int grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     const int cb_bytes = p.entries * VEC * 2;
-    const size_t smem = (size_t)((cb_bytes + 15) & ~15) + (size_t)2 * n_waves * 64 * sizeof(float4_t);
-    auto kern = decode_kernel<VEC, CodeT>;
+    const size_t base = (size_t)((cb_bytes + 15) & ~15) + (size_t)2 * n_waves * 64 * sizeof(float4_t);
+    const size_t stage = (size_t)n_waves * p.M * kStagePitch;
+    size_t smem = base;
+    int stage_off = -1, aliased = 0;
+    // Staging pays off when X is large enough for its scattered fetch to load the L1/L2 path;
+    // a small X is read directly (one LDS round trip less on the critical path).
+    if (n_chunks == 1 && (size_t)p.M * p.K * 2 > kStageMinBytes) {
+        if (base + stage <= kDisjointBudget) {
+            stage_off = (int)base;
+            smem = base + stage;
+        } else if (stage <= kDecodeLdsLimit) {
+            stage_off = 0;
+            aliased = 1;
+            smem = stage > base ? stage : base;
+        }
+    }
+    // One workgroup per tile range; as many workgroups as can be resident at once.
+    int per_cu = (int)(kDecodeLdsLimit / smem);
+    const int by_waves = 16 / n_waves > 0 ? 16 / n_waves : 1;
+    if (per_cu > by_waves) per_cu = by_waves;
+    if (per_cu < 1) per_cu = 1;
+    const int target = device_cu_count() * per_cu;
+    const int grid = n_tiles < target ? n_tiles : target;
+    // Up to 8 waves: compiled for 512 threads, which doubles the register budget per lane.
+    auto kern = n_waves <= 8 ? decode_kernel<VEC, CodeT, 512> : decode_kernel<VEC, CodeT, 1024>;
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
-                       p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb, tiles_per_wg, n_tiles, n_chunks);
+                       p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb, n_tiles, n_chunks, stage_off, aliased);
     return hipGetLastError();
 }
 
