@@ -34,6 +34,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 FP16_MFMA_PEAK_TFLOPS = 2500.0
 POOL_BYTES = 640 << 20  # distinct code matrices rotated through by the bandwidth-bound configs
+# HBM bytes one cold decode launch moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# 256 MiB copy (summary under profiles/): 1158 KiB x 2.0 read + 8 KiB written.
+MEASURED_C2_HBM_BYTES_PER_LAUNCH = 2_379_776
 
 
 def parse_args():
@@ -43,6 +46,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
+    ap.add_argument("--probe", metavar="CONFIG", default=None,
+                    help="profiling aid: launch CONFIG (C1..C5) --steps times, cold-HBM rotation for the decode "
+                         "configs, followed by one 256 MiB device copy as a counter yardstick; prints no JSON")
     return ap.parse_args()
 
 
@@ -68,6 +74,26 @@ def main():
 
     def barrier():
         torch.cuda.synchronize()
+
+    if args.probe:
+        spec = CONFIGS[args.probe]
+        x, codes, cb = make_problem(spec, seed=42, device=dev)
+        n_bufs = max(1, min(512, POOL_BYTES // spec.code_bytes)) if spec.M <= 16 else 1
+        gen = torch.Generator(device=dev).manual_seed(1234)
+        pool = [codes] + [torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev,
+                                        dtype=torch.int32).to(spec.code_dtype) for _ in range(n_bufs - 1)]
+        y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        barrier()
+        for i in range(args.steps):
+            cabi.e2e_gemm_b(x, pool[i % n_bufs], cb, out=y)
+        barrier()
+        dst.copy_(src)   # yardstick: reads 256 MiB, writes 256 MiB
+        barrier()
+        print(f"probe {args.probe}: {args.steps} launches over {n_bufs} code matrices, then one 256 MiB copy",
+              file=sys.stderr)
+        return
 
     def time_launches(launch, n_bufs, steps, warmup, chunk=500):
         """Average seconds per launch of `launch(i)` (i rotates over n_bufs), HIP graphs + events."""
@@ -179,13 +205,7 @@ def main():
             "gpu_vs_cpu_max_rel_err": e1, "gpu_vs_cpu_max_err_over_max": e2,
         }
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "decode_c2_hbm_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-        except Exception:
-            traffic = None
+    traffic = MEASURED_C2_HBM_BYTES_PER_LAUNCH
 
     t = main_res["us"] * 1e-6
     out = {
