@@ -51,6 +51,9 @@ SMALL_B = [
     ("u16_v2", 2, 128, 16, 2, 300, 1, 16),
     ("multi_cb16", 9, 512, 64, 8, 256, 4, 8),          # 16 rows per codebook
     ("multi_cb128", 33, 512, 256, 8, 256, 2, 8),
+    ("m17", 17, 512, 48, 8, 256, 1, 8),                  # decode kernel in 16-row slabs
+    ("m64_slabs", 64, 1024, 80, 4, 4096, 1, 16),
+    ("m65_prefill", 65, 256, 64, 8, 256, 1, 8),
     ("m300_ragged", 300, 384, 200, 8, 256, 1, 8),       # prefill kernel with ragged M, N and a K tail
     ("m64_v4", 64, 256, 96, 4, 256, 3, 8),
     ("deep_k", 2, 9216, 32, 8, 256, 1, 8),              # more K than one workgroup's waves cover at once
@@ -94,7 +97,7 @@ def test_e2e_gemm_b_all_variants(row):
         _check_gemm(y, x, codes, cb, what=f"{spec.name}/{cabi.VARIANT_NAMES[variant]}")
         ran.append(variant)
     assert cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran and cabi.VARIANT_TWOPASS in ran
-    if spec.M <= 16 and spec.vec in (2, 4, 8):
+    if spec.M <= 64 and spec.vec in (2, 4, 8):
         assert cabi.VARIANT_DECODE in ran
 
 

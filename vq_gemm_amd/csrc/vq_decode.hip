@@ -27,6 +27,7 @@ constexpr int kSliceK = 512;   // K handled by one wave
 constexpr int kSteps = 16;     // MFMA steps per slice (32 k each)
 constexpr int kTileN = 16;
 constexpr int kMaxWaves = 16;
+constexpr int kDecodeMaxM = 64;  // taller activations are served in 16-row slabs up to this height
 
 template <int VEC, typename CodeT>
 struct DecodeCfg {
@@ -339,7 +340,7 @@ constexpr size_t kDecodeLdsBudget = 144 * 1024;  // codebook + reduction slots m
 
 bool decode_supports(const ProblemB &p)
 {
-    if (p.M < 1 || p.M > 16 || p.N < 1 || p.K < 1) return false;
+    if (p.M < 1 || p.M > kDecodeMaxM || p.N < 1 || p.K < 1) return false;
     if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
     if (p.n_codebooks > 1 && p.rows_per_cb % kTileN != 0) return false;
     if ((size_t)p.entries * p.vec * 2 + 2 * kMaxWaves * 1024 > kDecodeLdsBudget) return false;
@@ -357,11 +358,23 @@ hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
-    switch (p.vec) {
-    case 8: return u8 ? launch_decode_typed<8, uint8_t>(p, s) : launch_decode_typed<8, uint16_t>(p, s);
-    case 4: return u8 ? launch_decode_typed<4, uint8_t>(p, s) : launch_decode_typed<4, uint16_t>(p, s);
-    default: return u8 ? launch_decode_typed<2, uint8_t>(p, s) : launch_decode_typed<2, uint16_t>(p, s);
+    // The kernel multiplies 16 rows of X at a time; taller X (up to kDecodeMaxM rows) goes in
+    // 16-row slabs, one launch each: still far better than a 256-row MFMA tile that is mostly
+    // padding and fills only N/256 compute units.
+    for (int m0 = 0; m0 < p.M; m0 += 16) {
+        ProblemB q = p;
+        q.x = p.x + (int64_t)m0 * p.K;
+        q.y = p.y + (int64_t)m0 * p.N;
+        q.M = p.M - m0 < 16 ? p.M - m0 : 16;
+        hipError_t e;
+        switch (p.vec) {
+        case 8: e = u8 ? launch_decode_typed<8, uint8_t>(q, s) : launch_decode_typed<8, uint16_t>(q, s); break;
+        case 4: e = u8 ? launch_decode_typed<4, uint8_t>(q, s) : launch_decode_typed<4, uint16_t>(q, s); break;
+        default: e = u8 ? launch_decode_typed<2, uint8_t>(q, s) : launch_decode_typed<2, uint16_t>(q, s); break;
+        }
+        if (e != hipSuccess) return e;
     }
+    return hipSuccess;
 }
 
 }  // namespace vq
