@@ -55,7 +55,8 @@ int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, vo
 /*
  * Fused VQ GEMM, geometry A (reference-native tensors, same entry point of the reference:
  * bind.cpp:3,7; indexing per strategy_2/bsz512/src.cu:163-176 and bench.py:46-56).
- * out is [M, 2*Nc].  `workspace` as above (K*2*Nc fp16 for TWOPASS).
+ * out is [M, 2*Nc].  `workspace` (K*2*Nc fp16) is required by TWOPASS; VQGEMM_VARIANT_AUTO takes the
+ * two-pass route when it is given and the scalar kernel when it is NULL.
  */
 int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *out,
                       int64_t M, int64_t K, int64_t Nc, int32_t variant,

@@ -137,7 +137,7 @@ def build_ext(keys=None, force: bool = True, jobs: int = 6):
                f"-DTORCH_EXTENSION_NAME={name}", "-DTORCH_API_INCLUDE_EXTENSION_H", f"-DVQ_VARIANT={variant}"]
         if is_ref:
             cmd.append("-DVQ_REF_MODULE=1")
-        cmd += incs + [src, "-o", out, f"-L{LIB_DIR}", "-lvqgemm_ref" if is_ref else "-lvqgemm",
+        cmd += incs + [src, "-o", out, f"-L{LIB_DIR}"] + (["-lvqgemm_ref"] if is_ref else ["-lvqgemm", "-lvqgemm_ref"]) + [
                        f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
                        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
         _run(cmd)

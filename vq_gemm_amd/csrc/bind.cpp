@@ -112,17 +112,27 @@ torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codeb
     torch::Tensor out = torch::empty({g.M, g.N}, input.options());
     torch::Tensor ws;
     void *ws_ptr = nullptr;
-    if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS) {
-        ws = torch::empty({g.is_a ? g.K : g.N, g.is_a ? g.N : g.K}, input.options());
+    if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS && !g.is_a) {
+        ws = torch::empty({g.N, g.K}, input.options());
         ws_ptr = ws.data_ptr();
     }
     int rc;
     if (g.is_a) {
-        // The decode/prefill tilings are K-axis kernels; reference-native tensors take the
-        // library's own choice unless the module is the two-pass one.
-        const int variant = VQ_VARIANT == VQGEMM_VARIANT_TWOPASS ? VQGEMM_VARIANT_TWOPASS : VQGEMM_VARIANT_AUTO;
-        rc = vqgemm_e2e_gemm_a(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.Nc, variant,
-                               ws_ptr, cur_stream(input));
+        // Reference-native tensors: the tiled fused kernels are K-axis kernels, so this layout is
+        // served as the reference's two-pass strategy does it (strategy_1/src.cu:323-399): the
+        // bit-exact dequant kernel writes W_dec[K, 2*Nc], then a plain GEMM multiplies.  The
+        // second pass is a library GEMM (hipBLASLt, fp32 accumulate) except in the s1 module,
+        // which keeps this library's own MFMA GEMM as the reference's s1 keeps its own.
+        torch::Tensor dec = torch::empty({g.K, g.N}, input.options());
+        rc = vqgemm_dequant_a(c.data_ptr(), cb.data_ptr(), dec.data_ptr(), g.K, g.Nc, cur_stream(input));
+        check_rc(rc, "e2e_gemm (dequant pass)");
+        if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS) {
+            rc = vqgemm_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, cur_stream(input));
+        } else {
+            const int rrc = vqref_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, 0, cur_stream(input));
+            TORCH_CHECK(rrc == 0, "e2e_gemm (GEMM pass) failed: ", vqref_error_string(rrc), " (code ", rrc, ")");
+            rc = 0;
+        }
     } else {
         rc = vqgemm_e2e_gemm_b(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.N, g.vec,
                                g.entries, g.n_codebooks, g.code_bits, VQ_VARIANT, ws_ptr, cur_stream(input));

@@ -172,8 +172,10 @@ int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *
     p.M = (int)M; p.K = (int)K; p.Nc = (int)Nc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipSuccess;
+    // No tiled fused kernel for this layout yet: with scratch the two-pass route (bit-exact dequant,
+    // then the MFMA GEMM) is the fast one, without it only the scalar kernel remains.
+    if (variant == VQGEMM_VARIANT_AUTO) variant = workspace ? VQGEMM_VARIANT_TWOPASS : VQGEMM_VARIANT_GENERIC;
     switch (variant) {
-    case VQGEMM_VARIANT_AUTO:
     case VQGEMM_VARIANT_GENERIC:
         e = launch_generic_a(p, s);
         break;
