@@ -119,6 +119,46 @@ def test_one_hot_activations_return_weight_columns_bit_exactly(variant, vec, bit
         assert np.array_equal(_np(y).view(np.uint16), w[:, k0:k0 + 16].T.copy().view(np.uint16))
 
 
+# Shapes that give a workgroup of the batched decode kernel several tiles (full batches, short
+# last batches, replicated and plain codebooks, every batch size), sized for a 256-CU device.
+BATCHED_B = [
+    # name, M, K, N, vec, E, bits
+    ("u8v8_m1_7_tiles", 1, 4096, 28672, 8, 256, 8),
+    ("u8v8_m16_9_tiles", 16, 4096, 36864, 8, 256, 8),
+    ("u8v8_m5_k1024", 5, 1024, 40960, 8, 256, 8),
+    ("u8v8_m3_e100", 3, 4096, 8192, 8, 100, 8),
+    ("u16v8_m3_k2048", 3, 2048, 20480, 8, 300, 16),
+    ("u8v4_m2", 2, 4096, 16384, 4, 256, 8),
+    ("u8v2_m16_k512", 16, 512, 16384, 2, 256, 8),
+    ("u16v4_m9_e4096", 9, 4096, 12288, 4, 4096, 16),
+]
+
+
+@pytest.mark.parametrize("row", BATCHED_B, ids=[r[0] for r in BATCHED_B])
+def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
+    name, M, K, N, v, E, bits = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, 1, bits)
+    x, codes, cb = make_problem(spec, seed=21, device=DEV)
+    _say("batched decode", spec)
+    assert cabi.select_variant_b(M, K, N, v, E, 1, bits) == cabi.VARIANT_DECODE
+    y = cabi.e2e_gemm_b(x, codes, cb)
+    torch.cuda.synchronize()
+    w = vo.dequant_b(_np(codes), _np(cb))
+    xf = _np(x).astype(np.float64)
+    ref = np.concatenate([xf @ w[r:r + 4096].astype(np.float64).T for r in range(0, N, 4096)], axis=1)
+    e1, e2 = vo.rel_err(_np(y), ref)
+    _say(f"  {name}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+    assert e1 <= TOL
+    # a permuted one-hot X reads W out bit for bit through the same kernel
+    eye = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+    cols = [(37 * m + 11) % K for m in range(M)]
+    for m, c in enumerate(cols):
+        eye[m, c] = 1.0
+    yw = cabi.e2e_gemm_b(eye, codes, cb)
+    assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)
+
+
 def test_every_m_from_1_to_16_on_the_decode_kernel():
     K, N = 1024, 80
     for M in range(1, 17):
@@ -143,9 +183,15 @@ def test_properties_constant_codes_zero_codebook_scaling():
         y1 = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
         y4 = cabi.e2e_gemm_b(x * 4, codes, cb, variant=variant)
         assert torch.equal(y4, (y1.float() * 4).half())          # power-of-two scaling is exact
-        # G identical codebooks == one codebook
+        # G identical codebooks == one codebook: the same W exactly (a permuted one-hot X reads it
+        # out bit for bit), the same product up to the order of the fp32 sums (the kernels for one
+        # and for several codebooks split K differently)
         cb4 = cb.unsqueeze(0).repeat(4, 1, 1).contiguous()
-        assert torch.equal(cabi.e2e_gemm_b(x, codes, cb4, variant=variant), y1)
+        eye = torch.eye(16, 1024, dtype=torch.float16, device=DEV).roll(5, dims=1)
+        assert torch.equal(cabi.e2e_gemm_b(eye, codes, cb4, variant=variant),
+                           cabi.e2e_gemm_b(eye, codes, cb, variant=variant))
+        y1g = cabi.e2e_gemm_b(x, codes, cb4, variant=variant)
+        assert vo.rel_err(_np(y1g), _np(y1).astype(np.float64))[0] <= 2e-3
         # run-to-run determinism (the reference harness's own check, bench.py:118-132)
         for _ in range(4):
             assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=variant), y1)

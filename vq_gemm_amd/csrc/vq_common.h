@@ -60,6 +60,9 @@ hipError_t launch_generic_a(const ProblemA &p, hipStream_t s);
 
 bool decode_supports(const ProblemB &p);
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s);
+// the general kernel behind launch_decode_b: one slab of at most 16 rows of X
+bool decode_general_supports(const ProblemB &p);
+hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);
 
 bool prefill_supports(const ProblemB &p);
 hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s);

@@ -1,88 +1,198 @@
-// Decode kernel (M <= 16): Y[M,N] = X[M,K] . W^T with W given as codes + codebook.
+// Decode path (at most 64 rows of X, 16 per launch): Y[M,N] = X[M,K] . W^T with W given as
+// codes + codebook.  This file holds the batched kernel, which takes the common shapes (one
+// codebook, K a multiple of 256 up to 4096, N a multiple of 16), and the dispatch; every other
+// shape goes to the general kernel of vq_decode_general.hip.
 //
-// The kernel is bound by the HBM stream of the code matrix (N*K/vec code bytes), so the
-// design goal is one pass over the codes with every other operand resident on the CU:
+// The path is bound by the HBM stream of the code matrix (N*K/vec code bytes), so the design
+// goal is one pass over the codes with every other operand resident on the CU:
 //
-//   * A workgroup owns tiles of 16 output columns (16 rows of W).  Each of its waves owns a
-//     512-wide slice of K and keeps the matching slice of X in registers, already in MFMA
-//     operand order, for the whole kernel: X is read from memory once per workgroup and never
-//     passes through the LDS.
-//   * The codebook (entries*vec*2 bytes) is resident in the LDS.  A lane streams 16 bytes of
-//     codes of one W row, gathers the codewords and uses them *directly* as the 8-half A
-//     operand of v_mfma_f32_16x16x32_f16: with vec = 8 one ds_read_b128 is one operand.
-//     The order in which a lane walks K is irrelevant to a dot product, so it is chosen so
-//     that each lane's codes are contiguous in memory; X is loaded in the same order.
-//   * Per tile a wave issues 16 MFMAs (its K slice), the partial 16x16 fp32 results of the
-//     waves are summed through 1 KB LDS slots, and one wave converts and stores the tile.
+//   * A workgroup owns tiles of 16 output columns (16 rows of W).  Wave w owns K slice w (256 k)
+//     and keeps the matching slice of X in registers, already in MFMA operand order, for the
+//     whole kernel; K = 4096 makes 16 waves, four per SIMD at 128 registers each.
+//   * The codebook (entries*vec*2 bytes) is resident in the LDS.  A lane streams the codes of
+//     one W row, gathers the codewords and uses them *directly* as the 8-half A operand of
+//     v_mfma_f32_16x16x32_f16: with vec = 8 one ds_read_b128 is one operand.  The order in which
+//     a lane walks K is irrelevant to a dot product, so it is chosen so that each lane's codes
+//     are contiguous in memory; X is loaded in the same order.
+//   * Per tile a wave issues 8 MFMAs (its K slice); the partial 16x16 fp32 results of the waves
+//     are summed through the LDS and one wave converts and stores them.
 //
 // M < 16 pads the X operand with zeros (the matrix core is idle anyway: the kernel is
 // bandwidth bound by a wide margin); fp32 accumulation throughout, one rounding to fp16.
 #include "vq_common.h"
+
+#include <type_traits>
 
 namespace vq {
 
 namespace {
 
 constexpr int kTileN = 16;
-constexpr int kMaxWaves = 8;   // 512 threads: leaves 256 registers per lane
+constexpr int kSliceK = 256;     // K owned by one wave
+constexpr int kSteps = 8;        // MFMA steps (32 k each) per slice
+constexpr int kMaxWaves = 16;    // 1024 threads, 128 registers per lane
 constexpr int kDecodeMaxM = 64;  // taller activations are served in 16-row slabs up to this height
+constexpr int kStageK = 512;     // X is staged in pieces of 512 k of one row (1 KB, one wave instruction)
+constexpr int kStagePitch = kStageK * 2 + 16;  // LDS bytes per staged piece; the pad spreads rows over the banks
 
-// STEPS = MFMA steps (32 k each) of the K slice one wave owns: 16 (512 k) up to K = 4096,
-// 32 (1024 k, X slice of 128 registers) beyond, so that K = 8192 still needs one pass.
-template <int VEC, typename CodeT, int STEPS = 16>
+template <int VEC, typename CodeT>
 struct DecodeCfg {
-    static constexpr int kSliceK = 32 * STEPS;
-    static constexpr int kSteps = STEPS;
-    static constexpr int CPL = 16 / (int)sizeof(CodeT);  // codes in one 16-byte lane load
+    // bytes of codes a lane loads at a time: 16, or 8 where 16 would span more than the slice
+    static constexpr int LB = 16 / (int)sizeof(CodeT) * VEC * 4 > kSliceK ? 8 : 16;
+    static constexpr int CPL = LB / (int)sizeof(CodeT);  // codes in one lane load
     static constexpr int CPO = 8 / VEC;                  // codes per 8-half MFMA operand
     static constexpr int SPL = CPL / CPO;                // MFMA steps fed by one lane load
     static constexpr int K_LANE = CPL * VEC;             // k covered by one lane load
     static constexpr int K_WAVE = 4 * K_LANE;            // k covered by one wave load (4 k-groups)
     static constexpr int LPT = kSliceK / K_WAVE;         // lane loads per slice
-    // (tile, chunk) code loads kept in flight, as many as the registers allow
-    static constexpr int PF = STEPS <= 16 ? (LPT <= 4 ? 4 : 2) : (LPT <= 2 ? 2 : 1);
+    static constexpr int WPL = LB / 4;                   // 32-bit words per lane load
+    // tiles a wave works through between two cross-wave reductions
+    static constexpr int TB = LPT * WPL <= 2 ? 4 : (LPT <= 2 ? 2 : 1);
     static_assert(CPO >= 1 && SPL >= 1 && LPT >= 1 && LPT * SPL == kSteps, "unsupported code layout");
 };
 
-template <typename CodeT, int CPL>
-__device__ __forceinline__ uint32_t extract_code(const uint4_t &cw, int c)
+// The codes one lane holds for one slice: LPT loads of WPL words.
+//
+// The loads are inline assembly that the compiler does not wait for (see the gathers below for
+// the technique): its own bookkeeping drains every load in flight once a store is pending too,
+// because the counter cannot tell loads from stores, and the tile loop would pay a full memory
+// latency per tile.  Loads complete in order among themselves, so the oldest unit in flight has
+// landed once at most `younger loads` operations are outstanding, whatever stores are pending.
+template <int VEC, typename CodeT>
+struct LaneCodes {
+    typedef DecodeCfg<VEC, CodeT> C;
+    typedef uint32_t words_t __attribute__((ext_vector_type(C::WPL)));
+    words_t w[C::LPT];
+
+    // Load t of the slice, from a wave-uniform base plus a 32-bit lane offset and an immediate: the address
+    // of the next tile costs the scalar unit two additions and the vector unit nothing.
+    template <int IMM>
+    __device__ __forceinline__ void load_async_s(int t, uint32_t voff, const void *sbase)
+    {
+        if constexpr (C::WPL == 4)
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(w[t]) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+        else
+            asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=v"(w[t]) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+    }
+    __device__ __forceinline__ void pin()
+    {
+#pragma unroll
+        for (int t = 0; t < C::LPT; t++) asm volatile("" : "+v"(w[t]));
+    }
+};
+
+// ---- hand-issued LDS gathers ------------------------------------------------------------
+// Left to the compiler, only two gathers are in flight ahead of the MFMAs that use them and
+// every step waits for the LDS latency.  The gathers are therefore issued as inline assembly,
+// which the compiler neither reorders nor waits for; the code below waits for them itself
+// (lgkmcnt counts LDS instructions, which complete in order) and ties each wait to the
+// registers with an empty asm (`pin`) so that no use can be moved above it.  A gathered
+// operand is consumed in the straight-line code that issued it: nothing in flight is ever
+// live across a branch, where the compiler might copy or spill a register still being written.
+__device__ __forceinline__ void lds_read_async(uint4_t &dst, uint32_t addr)
 {
-    if constexpr (sizeof(CodeT) == 1)
-        return (cw[c >> 2] >> (8 * (c & 3))) & 0xffu;
-    else
-        return (cw[c >> 1] >> (16 * (c & 1))) & 0xffffu;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(dst) : "v"(addr) : "memory");
+}
+__device__ __forceinline__ void lds_read_async(uint2_t &dst, uint32_t addr)
+{
+    asm volatile("ds_read_b64 %0, %1" : "=v"(dst) : "v"(addr) : "memory");
+}
+__device__ __forceinline__ void lds_read_async(uint32_t &dst, uint32_t addr)
+{
+    asm volatile("ds_read_b32 %0, %1" : "=v"(dst) : "v"(addr) : "memory");
 }
 
-// Gather the 8-half operand made of CPO consecutive codewords starting at code c0.
-// STRIDE is the byte distance between codebook entries in the LDS: the entry size for a plain
-// codebook, 256 for the bank-replicated one (see decode_kernel).
-template <int VEC, typename CodeT, int STRIDE>
-__device__ __forceinline__ half8_t gather_operand(const uint8_t *cb_lds, const uint4_t &cw, int c0)
+// s_waitcnt for the LDS counter only (gfx9 encoding: lgkmcnt = simm16[11:8], at most 15).
+template <int N>
+__device__ __forceinline__ void wait_lgkmcnt()
 {
-    typedef DecodeCfg<VEC, CodeT> C;
-    if constexpr (VEC == 8) {
-        const uint32_t code = extract_code<CodeT, C::CPL>(cw, c0);
-        return *reinterpret_cast<const half8_t *>(cb_lds + code * (uint32_t)STRIDE);
-    } else if constexpr (VEC == 4) {
-        const uint32_t a = extract_code<CodeT, C::CPL>(cw, c0);
-        const uint32_t b = extract_code<CodeT, C::CPL>(cw, c0 + 1);
-        const half4_t lo = *reinterpret_cast<const half4_t *>(cb_lds + a * (uint32_t)STRIDE);
-        const half4_t hi = *reinterpret_cast<const half4_t *>(cb_lds + b * (uint32_t)STRIDE);
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    } else {
-        static_assert(VEC == 2, "vector length must be 2, 4 or 8");
-        half2_t q[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t c = extract_code<CodeT, C::CPL>(cw, c0 + i);
-            q[i] = *reinterpret_cast<const half2_t *>(cb_lds + c * (uint32_t)STRIDE);
-        }
-        const half4_t lo = __builtin_shufflevector(q[0], q[1], 0, 1, 2, 3);
-        const half4_t hi = __builtin_shufflevector(q[2], q[3], 0, 1, 2, 3);
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    static_assert(N >= 0 && N <= 15, "lgkmcnt has four bits");
+    __builtin_amdgcn_s_waitcnt(0xc07f | (N << 8));
+}
+
+// The same for a count that is only constant after unrolling (values above 15 wait for 15).
+__device__ __forceinline__ void wait_lgkmcnt_upto(int n)
+{
+    switch (n < 15 ? n : 15) {
+    case 0: wait_lgkmcnt<0>(); break;
+    case 1: wait_lgkmcnt<1>(); break;
+    case 2: wait_lgkmcnt<2>(); break;
+    case 3: wait_lgkmcnt<3>(); break;
+    case 4: wait_lgkmcnt<4>(); break;
+    case 5: wait_lgkmcnt<5>(); break;
+    case 6: wait_lgkmcnt<6>(); break;
+    case 7: wait_lgkmcnt<7>(); break;
+    case 8: wait_lgkmcnt<8>(); break;
+    case 9: wait_lgkmcnt<9>(); break;
+    case 10: wait_lgkmcnt<10>(); break;
+    case 11: wait_lgkmcnt<11>(); break;
+    case 12: wait_lgkmcnt<12>(); break;
+    case 13: wait_lgkmcnt<13>(); break;
+    case 14: wait_lgkmcnt<14>(); break;
+    default: wait_lgkmcnt<15>(); break;
     }
 }
 
+// One 8-half MFMA operand as the pieces it is gathered in: one codeword per piece.
+template <int VEC> struct OperandPiece;
+template <> struct OperandPiece<8> { typedef uint4_t type; };
+template <> struct OperandPiece<4> { typedef uint2_t type; };
+template <> struct OperandPiece<2> { typedef uint32_t type; };
+
+template <int VEC>
+struct Operand {
+    static constexpr int kPieces = 8 / VEC;
+    typename OperandPiece<VEC>::type p[kPieces];
+
+    __device__ __forceinline__ void pin()
+    {
+#pragma unroll
+        for (int i = 0; i < kPieces; i++) asm volatile("" : "+v"(p[i]));
+    }
+    __device__ __forceinline__ half8_t value() const
+    {
+        uint4_t v;
+        if constexpr (VEC == 8) {
+            v = p[0];
+        } else if constexpr (VEC == 4) {
+            v = uint4_t{p[0][0], p[0][1], p[1][0], p[1][1]};
+        } else {
+            v = uint4_t{p[0], p[1], p[2], p[3]};
+        }
+        return as_half8(v);
+    }
+};
+
+// LDS byte address of codeword number c of a lane's 16 bytes of codes.
+//   plain table:      code * entry_bytes (the table starts at LDS address 0)
+//   replicated table: code * 256 + base, base < 256 being the lane's copy: one byte permute
+//                     puts the code into byte 1 and the base into byte 0 of the address.
+template <int VEC, typename CodeT, bool REPL>
+__device__ __forceinline__ uint32_t codeword_addr(const LaneCodes<VEC, CodeT> &cw, int c, uint32_t base)
+{
+    typedef DecodeCfg<VEC, CodeT> C;
+    constexpr bool u8 = sizeof(CodeT) == 1;
+    const int t = c / C::CPL, ci = c % C::CPL;  // lane load, code within it
+    const uint32_t word = u8 ? cw.w[t][ci >> 2] : cw.w[t][ci >> 1];
+    const int byte = u8 ? (ci & 3) : 2 * (ci & 1);
+    if constexpr (REPL) {
+        // selector bytes: 0 = byte 0 of `base`, 4 + b = byte b of `word`, 0x0c = zero
+        return __builtin_amdgcn_perm(word, base, 0x0c0c0000u | ((4u + byte) << 8));
+    } else {
+        const uint32_t code = u8 ? ((word >> (8 * byte)) & 0xffu) : ((word >> (8 * byte)) & 0xffffu);
+        return code * (uint32_t)(VEC * 2);
+    }
+}
+
+// Issue the gathers of the operand of MFMA step s: codewords s*CPO .. s*CPO + CPO-1 of the slice.
+template <int VEC, typename CodeT, bool REPL>
+__device__ __forceinline__ void gather_issue(Operand<VEC> &o, const LaneCodes<VEC, CodeT> &cw, int s, uint32_t base)
+{
+    typedef DecodeCfg<VEC, CodeT> C;
+#pragma unroll
+    for (int i = 0; i < Operand<VEC>::kPieces; i++)
+        lds_read_async(o.p[i], codeword_addr<VEC, CodeT, REPL>(cw, s * C::CPO + i, base));
+}
 
 // s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
 template <int N>
@@ -102,337 +212,318 @@ __device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff,
                  : "memory");
 }
 
-// stage_off >= 0: the X slices are staged through the LDS at that offset (n_chunks == 1 only);
-// `aliased` says that the staging area overlaps the codebook, which is then loaded afterwards.
-//
-// REPL: bank-replicated codebook.  A gather at uniformly random entries loses more than half of
-// the LDS bandwidth to bank conflicts, and at 16 LDS bytes read per code byte streamed the LDS is
-// what bounds a long u8/v8 GEMV.  With at most 256 entries the codebook is laid out as one
-// 256-byte bank row per entry holding 256/entry_bytes copies of it; lane l reads copy
-// l % copies, so the lanes served together never share a bank whatever the codes are.
-template <int VEC, typename CodeT, int STEPS, bool REPL>
-__global__ __launch_bounds__(512) void decode_kernel(const half_t *__restrict__ x,
-                                                      const CodeT *__restrict__ codes,
-                                                      const half_t *__restrict__ cb,
-                                                      half_t *__restrict__ y, int M, int K, int N,
-                                                      int entries, int rows_per_cb, int tiles_q,
-                                                      int tiles_r, int n_chunks, int stage_off,
-                                                      int aliased)
+// ---- batched kernel -----------------------------------------------------------------------
+// The common case (one codebook, K a multiple of 256 and at most 4096, N a multiple of 16) gets
+// a loop that is lean in instructions: a CU issues one vector and one scalar instruction per
+// cycle in total, whatever the number of waves, and a loop that spends a hundred instructions
+// per wave and tile on control flow, addresses and the reduction is bound by exactly that.
+//   * A wave works through TB consecutive tiles (its K slice of each) before the waves meet, so
+//     barriers, waits and loop control are paid once per TB tiles (TB = 1 for workgroups with
+//     fewer tiles than a full batch).
+//   * Code loads take a scalar base per tile and one lane offset computed before the loop.
+//   * The MFMA chain of a tile starts from a zero constant: no accumulator is cleared or summed.
+//   * The partial results go to the LDS packed as [slot][wave], slot = (tile, k-group, X row)
+//     over the rows of X that exist only; a reducing wave takes 64 slots per pass, every lane
+//     summing the 16-byte entries of its slot, so a pass covers 16/M tiles.
+// `recip_m` = ceil(65536 / M), for the division of a slot number by M.
+constexpr int kSlotPitch = 16 * kMaxWaves + 16;  // LDS bytes per slot; the pad spreads the slots over the banks
+
+template <int VEC, typename CodeT, bool REPL, int TB>
+__global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
+                                                               const CodeT *__restrict__ codes,
+                                                               const half_t *__restrict__ cb,
+                                                               half_t *__restrict__ y, int M, int K, int N,
+                                                               int entries, int tiles_q, int tiles_r,
+                                                               int stage_off, int aliased, int recip_m)
 {
-    typedef DecodeCfg<VEC, CodeT, STEPS> C;
-    constexpr int kSliceK = C::kSliceK;
-    constexpr int kSteps = C::kSteps;
-    constexpr int kStagePitch = kSliceK * 2 + 16;  // bytes per staged X row slice; the pad spreads rows over the banks
+    typedef DecodeCfg<VEC, CodeT> C;
+    typedef LaneCodes<VEC, CodeT> Codes;
+    constexpr int kPieces = Operand<VEC>::kPieces;
+    constexpr int kEntryBytes = VEC * 2;
     extern __shared__ __align__(16) uint8_t smem[];
-    const int n_waves = blockDim.x >> 6;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = blockDim.x >> 6;  // = K / 256: wave w owns K slice w
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int r16 = lane & 15;  // W row within the tile (A operand) / X row m (B operand)
     const int kq = lane >> 4;   // k-group of the lane, 0..3
     const int J = K / VEC;
-    const int cb_bytes = entries * VEC * 2;
-    constexpr int kEntryBytes = VEC * 2;
-    constexpr int kStride = REPL ? 256 : kEntryBytes;
-    const int cb_lds_bytes = REPL ? entries * 256 : ((cb_bytes + 15) & ~15);
-    uint8_t *cb_lds = smem;
-    // Lane's copy of the entries in the replicated layout (0 in the plain one).
-    const uint8_t *cb_gather = smem + (REPL ? (lane % (256 / kEntryBytes)) * kEntryBytes : 0);
-    float4_t *red = reinterpret_cast<float4_t *>(smem + cb_lds_bytes);
+    const int cb_slots = REPL ? entries * 16 : entries * kEntryBytes / 16;  // 16-byte slots of the LDS table
+    uint4_t *cb_lds = reinterpret_cast<uint4_t *>(smem);
+    const uint32_t gather_base = REPL ? (lane % (256 / kEntryBytes)) * kEntryBytes : 0;
+    const uint32_t red_base = cb_slots * 16;
 
-    // Balanced contiguous split of the tiles over the workgroups: tiles_q each, one more for the
-    // first tiles_r (quotient and remainder of tiles / workgroups, computed by the host).
     const int wg = blockIdx.x;
     const int tile_begin = wg * tiles_q + min(wg, tiles_r);
     const int tile_end = tile_begin + tiles_q + (wg < tiles_r ? 1 : 0);
     if (tile_begin >= tile_end) return;
+    const int n_units = (tile_end - tile_begin + TB - 1) / TB;
 
-    // k of MFMA step s for this lane inside a slice that starts at k0.
-    auto step_k = [&](int k0, int s) { return k0 + (s / C::SPL) * C::K_WAVE + kq * C::K_LANE + (s % C::SPL) * 8; };
-
-    half8_t xr[kSteps];
-    auto load_x = [&](int k0) {
+    // Codes: lane offset inside a tile, scalar base per tile.  The last unit may hold fewer than
+    // TB tiles.
+    const uint32_t voff = (uint32_t)((r16 * J + (w * kSliceK + kq * C::K_LANE) / VEC) * (int)sizeof(CodeT));
+    const int64_t tile_bytes = (int64_t)kTileN * J * (int)sizeof(CodeT);
+    auto load_unit = [&](int q, Codes (&cw)[TB]) {
 #pragma unroll
-        for (int s = 0; s < kSteps; s++) {
-            const int k = step_k(k0, s);
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (r16 < M && k < K) v = ld_global_16(x + (int64_t)r16 * K + k);
-            xr[s] = as_half8(v);
+        for (int j = 0; j < TB; j++) {
+            const int tile = tile_begin + q * TB + j;
+            if (tile >= tile_end) break;
+            const uint8_t *sbase = reinterpret_cast<const uint8_t *>(codes) + tile * tile_bytes;
+            if constexpr (C::LPT >= 1) cw[j].template load_async_s<0>(0, voff, sbase);
+            if constexpr (C::LPT >= 2) cw[j].template load_async_s<4 * C::LB>(1, voff, sbase);
+            if constexpr (C::LPT >= 3) cw[j].template load_async_s<8 * C::LB>(2, voff, sbase);
+            if constexpr (C::LPT >= 4) cw[j].template load_async_s<12 * C::LB>(3, voff, sbase);
+            static_assert(C::LPT <= 4, "at most four lane loads per slice");
         }
     };
-    auto load_codes = [&](int tile, int k0, uint4_t (&cw)[C::LPT]) {
-        const int row = min(tile * kTileN + r16, N - 1);
-#pragma unroll
-        for (int t = 0; t < C::LPT; t++) {
-            const int k = k0 + t * C::K_WAVE + kq * C::K_LANE;
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (k < K) v = ld_global_16(codes + (int64_t)row * J + k / VEC);
-            cw[t] = v;
-        }
-    };
-    auto load_codebook = [&](int g) {
+    // Two units of codes are in flight: ring slot q % 2 holds unit q.
+    Codes cwq[2][TB];
+    load_unit(0, cwq[0]);
+    if (n_units > 1) load_unit(1, cwq[1]);
+
+    // Codebook: global -> registers -> LDS, fetched now, stored once the LDS is free.
+    constexpr int kCbRegs = 4;
+    const bool cb_in_regs = cb_slots <= kCbRegs * (int)blockDim.x;
+    uint4_t cb_regs[kCbRegs];
+    auto read_slot = [&](int i) {
         if constexpr (REPL) {
-            // 16-byte slot i of the table belongs to entry i / 16; it holds 16 / entry_bytes copies.
-            // All loads are issued before the first write so that their latencies overlap.
             typedef uint32_t entry_t __attribute__((ext_vector_type(kEntryBytes / 4)));
-            const entry_t *src = reinterpret_cast<const entry_t *>(cb + (int64_t)g * entries * VEC);
-            constexpr int kMaxIter = 4;  // loads in flight per thread and round
-            for (int base = 0; base < entries * 16; base += kMaxIter * (int)blockDim.x) {
-                entry_t e[kMaxIter];
+            const entry_t e = reinterpret_cast<const entry_t *>(cb)[i >> 4];
+            uint4_t v;
 #pragma unroll
-                for (int j = 0; j < kMaxIter; j++) {
-                    const int i = base + j * (int)blockDim.x + (int)threadIdx.x;
-                    e[j] = src[(i < entries * 16 ? i : 0) >> 4];
-                }
-#pragma unroll
-                for (int j = 0; j < kMaxIter; j++) {
-                    const int i = base + j * (int)blockDim.x + (int)threadIdx.x;
-                    uint4_t v;
-#pragma unroll
-                    for (int d = 0; d < 4; d++) v[d] = e[j][d % (kEntryBytes / 4)];
-                    if (i < entries * 16) reinterpret_cast<uint4_t *>(cb_lds)[i] = v;
-                }
-            }
+            for (int d = 0; d < 4; d++) v[d] = e[d % (kEntryBytes / 4)];
+            return v;
         } else {
-            const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g * entries * VEC);
-            for (int i = threadIdx.x; i < cb_bytes / 16; i += blockDim.x) reinterpret_cast<uint4_t *>(cb_lds)[i] = src[i];
-        }
-    };
-
-    const int chunk_k = n_waves * kSliceK;
-    // The unit of work is a (tile, chunk) pair; the codes of the next PF units are always in
-    // flight, so a workgroup with only a few tiles pays the memory latency once, not per tile.
-    const int q_begin = tile_begin * n_chunks, q_end = tile_end * n_chunks;
-    constexpr int PF = C::PF;
-    uint4_t cwq[PF][C::LPT];
-    auto load_unit = [&](int q, uint4_t (&cw)[C::LPT]) {
-        const int tile = n_chunks == 1 ? q : q / n_chunks, chunk = q - tile * n_chunks;
-        load_codes(tile, chunk * chunk_k + wave * kSliceK, cw);
-    };
-#pragma unroll
-    for (int u = 0; u < PF; u++)
-        if (q_begin + u < q_end) load_unit(q_begin + u, cwq[u]);
-
-    // Small codebooks are fetched into registers up front so that their latency overlaps the
-    // X staging even when the staging area and the codebook share LDS space.
-    const int cb_chunks = cb_bytes / 16;
-    const bool cb_in_regs = !REPL && cb_chunks <= 4 * (int)blockDim.x;
-    uint4_t cb_regs[4];
-    auto fetch_codebook = [&](int g) {
-        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g * entries * VEC);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int i = threadIdx.x + j * blockDim.x;
-            cb_regs[j] = i < cb_chunks ? src[i] : uint4_t{0u, 0u, 0u, 0u};
+            return reinterpret_cast<const uint4_t *>(cb)[i];
         }
     };
     auto store_codebook = [&]() {
+        if (cb_in_regs) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int i = threadIdx.x + j * blockDim.x;
-            if (i < cb_chunks) reinterpret_cast<uint4_t *>(cb_lds)[i] = cb_regs[j];
+            for (int j = 0; j < kCbRegs; j++) {
+                const int i = threadIdx.x + j * blockDim.x;
+                if (i < cb_slots) cb_lds[i] = cb_regs[j];
+            }
+        } else {
+            for (int i = threadIdx.x; i < cb_slots; i += blockDim.x) cb_lds[i] = read_slot(i);
         }
     };
-
-    // Everything the first tile waits for is requested before anything is waited for: codes
-    // (above), codebook, X.
-    int cur_cb = -1;
-    const int g0 = rows_per_cb >= N ? 0 : (tile_begin * kTileN) / rows_per_cb;
-    if (stage_off < 0 && cb_in_regs) fetch_codebook(g0);
-    if (stage_off >= 0) {
-        // X -> registers through the LDS.  A lane needs 16-byte pieces scattered over its row
-        // slice; fetched directly, every load instruction touches dozens of cache lines and
-        // uses 16 bytes of each.  Instead the wave copies each row slice (1 KB, contiguous) into
-        // a private LDS window and the lanes pick their pieces from there.
-        const int k0 = wave * kSliceK;
-        const uint32_t win = stage_off + wave * M * kStagePitch;
-        for (int i = 0; i < M; i++)
+    if (cb_in_regs) {
+        // (whole waves past the end of the table issue no load: every vector memory instruction
+        // of the prologue queues behind the others of the CU)
 #pragma unroll
-            for (int h = 0; h < kSliceK / 512; h++) {
-                const int kl = k0 + h * 512 + 8 * lane;
-                load_to_lds_16(win + i * kStagePitch + h * 1024, (uint32_t)((i * K + (kl < K ? kl : 0)) * 2), x);
-            }
-        const int g = g0;
-        if (cb_in_regs) fetch_codebook(g);
-        else if (!aliased) load_codebook(g);
-        wait_vmcnt<0>();
-#pragma unroll
-        for (int s = 0; s < kSteps; s++) {
-            const int k = step_k(k0, s);
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (r16 < M && k < K) v = *reinterpret_cast<const uint4_t *>(smem + win + r16 * kStagePitch + (k - k0) * 2);
-            xr[s] = as_half8(v);
-        }
-        if (aliased) __syncthreads();  // every wave has picked up its X before the codebook overwrites it
-        if (cb_in_regs) store_codebook();
-        else if (aliased) load_codebook(g);
-        __syncthreads();
-        cur_cb = g;
-    } else {
-        if (n_chunks == 1) load_x(wave * kSliceK);
-        if (cb_in_regs) {
-            store_codebook();
-            __syncthreads();
-            cur_cb = g0;
+        for (int j = 0; j < kCbRegs; j++) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if ((i & ~63) < cb_slots) cb_regs[j] = read_slot(i < cb_slots ? i : 0);
         }
     }
 
-    int parity = 0;
-    // Four accumulators: consecutive MFMAs do not wait on each other's result.
-    float4_t acc[4];
+    // X slice of the wave -> registers, in MFMA operand order; rows past M are zero.
+    const int k0 = w * kSliceK;
+    auto step_k = [&](int s) { return (s / C::SPL) * C::K_WAVE + kq * C::K_LANE + (s % C::SPL) * 8; };
+    half8_t xr[kSteps];
+    {
+        // Through the LDS in pieces of 512 k of one row (1 KB, contiguous): a few whole-wave
+        // copies per workgroup instead of eight mostly idle loads per wave.  Every vector memory
+        // instruction of the prologue queues behind the others of the CU, so their number is
+        // what the first tile waits for.
+        const int n_blocks = K / kStageK + (K % kStageK ? 1 : 0);
+        for (int pc = w; pc < n_blocks * M; pc += n_waves) {
+            const int b = pc / M, i = pc - b * M;
+            const int kl = b * kStageK + 8 * lane;
+            load_to_lds_16(stage_off + pc * kStagePitch, (uint32_t)((i * K + (kl < K ? kl : 0)) * 2), x);
+        }
+        const uint32_t win = stage_off + ((k0 / kStageK) * M + r16) * kStagePitch + (k0 % kStageK) * 2;
+        if (!aliased) store_codebook();
+        wait_vmcnt<0>();
+        __syncthreads();  // pieces staged by the other waves
 #pragma unroll
-    for (int a = 0; a < 4; a++) acc[a] = float4_t{0.f, 0.f, 0.f, 0.f};
-    for (int qb = q_begin; qb < q_end; qb += PF) {
-#pragma unroll
-        for (int u = 0; u < PF; u++) {
-            const int q = qb + u;
-            if (q >= q_end) break;
-            const int tile = n_chunks == 1 ? q : q / n_chunks, chunk = q - tile * n_chunks;
-            const int g = rows_per_cb >= N ? 0 : (tile * kTileN) / rows_per_cb;
-            if (g != cur_cb) {
-                // (Re)load the codebook of this row block into the LDS.
-                if (cur_cb >= 0) __syncthreads();
-                load_codebook(g);
-                __syncthreads();
-                cur_cb = g;
-            }
-            uint4_t cw[C::LPT];
-#pragma unroll
-            for (int t = 0; t < C::LPT; t++) cw[t] = cwq[u][t];
-            if (q + PF < q_end) load_unit(q + PF, cwq[u]);
-            if (n_chunks > 1) load_x(chunk * chunk_k + wave * kSliceK);
-#pragma unroll
-            for (int s = 0; s < kSteps; s++) {
-                const half8_t a = gather_operand<VEC, CodeT, kStride>(cb_gather, cw[s / C::SPL], (s % C::SPL) * C::CPO);
-                acc[s & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xr[s], acc[s & 3], 0, 0, 0);
-                // Bound how far the scheduler hoists gathers ahead of their MFMAs (register pressure).
-                if (STEPS > 16 && (s & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-            }
-            if (chunk != n_chunks - 1) continue;
-
-            const float4_t p = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-#pragma unroll
-            for (int a = 0; a < 4; a++) acc[a] = float4_t{0.f, 0.f, 0.f, 0.f};
-            // Sum the K slices of the waves through LDS slots (parity, wave, lane); the waves take
-            // turns at adding up and storing a tile.
-            red[(parity * n_waves + wave) * 64 + lane] = p;
+        for (int s = 0; s < kSteps; s++) {
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (r16 < M) v = *reinterpret_cast<const uint4_t *>(smem + win + step_k(s) * 2);
+            xr[s] = as_half8(v);
+        }
+        if (aliased) {
+            __syncthreads();  // every wave has picked up its X before the codebook overwrites it
+            store_codebook();
             __syncthreads();
-            if (wave == (tile % n_waves)) {
-                float4_t sum = red[(parity * n_waves) * 64 + lane];
-                for (int w = 1; w < n_waves; w++) {
-                    const float4_t v = red[(parity * n_waves + w) * 64 + lane];
-                    sum += v;
-                }
-                // D[i][j]: j = lane % 16 is the X row m, i = 4*(lane/16) + r is the W row.
-                const int m = r16;
-                const int n = tile * kTileN + 4 * kq;
-                if (m < M) {
-                    half_t *dst = y + (int64_t)m * N + n;
-                    if ((N & 3) == 0 && n + 3 < N) {
-                        half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
-                        *reinterpret_cast<half4_t *>(dst) = h;
-                    } else {
+        }
+    }
+
+    // Partial results: slot (j, kq, m) = (j*4 + kq)*M + m for tile j of the unit; this lane writes
+    // entry w of the slots (j, kq, r16).
+    const uint32_t wr_addr = red_base + (uint32_t)(kq * M + r16) * kSlotPitch + w * 16;
+    const uint32_t wr_stride = (uint32_t)(4 * M) * kSlotPitch;
+    const int n_slots = TB * 4 * M;
+    const int n_passes = (n_slots + 63) >> 6;
+    int turn = 0;  // the wave that takes the next reduction pass
+
+    auto process_unit = [&](int q, Codes (&cur)[TB]) {
+        // This unit's codes have landed when only the loads of the next unit are out (a short last
+        // unit has fewer of them: then everything is awaited).
+        const int nt = min(TB, tile_end - (tile_begin + q * TB));  // tiles of this unit
+        if (tile_begin + (q + 2) * TB <= tile_end) wait_vmcnt<TB * C::LPT>();
+        else wait_vmcnt<0>();
 #pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            if (n + r < N) dst[r] = (half_t)sum[r];
+        for (int j = 0; j < TB; j++) cur[j].pin();
+
+        float4_t acc[TB];
+        const float4_t c0 = {0.f, 0.f, 0.f, 0.f};
+        if (nt == TB) {
+            // One branch-free stream of TB*8 MFMA steps; ops[] holds the gathered operands of a
+            // tile, and each is replaced by the next tile's as soon as it has been multiplied.
+            Operand<VEC> ops[kSteps];
+#pragma unroll
+            for (int s = 0; s < kSteps; s++) gather_issue<VEC, CodeT, REPL>(ops[s], cur[0], s, gather_base);
+#pragma unroll
+            for (int i = 0; i < TB * kSteps; i++) {
+                const int j = i / kSteps, s = i % kSteps;
+                Operand<VEC> &o = ops[s];
+                const int left = TB * kSteps - 1 - i;  // steps after this one
+                wait_lgkmcnt_upto((left < kSteps - 1 ? left : kSteps - 1) * kPieces);  // younger gathers in flight
+                o.pin();
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.value(), xr[s], s == 0 ? c0 : acc[j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                const int t = i + kSteps;
+                if (t < TB * kSteps) gather_issue<VEC, CodeT, REPL>(o, cur[t / kSteps], t % kSteps, gather_base);
+                // All gather addresses of the unit are computed: its ring slot takes the unit after next.
+                if (t == TB * kSteps - 1 || (TB == 1 && i == 0))
+                    if (q + 2 < n_units) load_unit(q + 2, cur);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            // Short last unit: tile by tile, nothing in flight from one tile to the next.
+#pragma unroll
+            for (int j = 0; j < TB; j++) {
+                acc[j] = c0;
+                if (j < nt) {
+                    Operand<VEC> ops[kSteps];
+#pragma unroll
+                    for (int s = 0; s < kSteps; s++) gather_issue<VEC, CodeT, REPL>(ops[s], cur[j], s, gather_base);
+#pragma unroll
+                    for (int s = 0; s < kSteps; s++) {
+                        wait_lgkmcnt_upto((kSteps - 1 - s) * kPieces);
+                        ops[s].pin();
+                        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ops[s].value(), xr[s], acc[j], 0, 0, 0);
                     }
                 }
             }
-            parity ^= 1;
         }
+
+        if (q > 0) __syncthreads();  // the reducers of the previous unit are done with the slots
+        if (r16 < M) {
+#pragma unroll
+            for (int j = 0; j < TB; j++)
+                if (j < nt) *reinterpret_cast<float4_t *>(smem + wr_addr + j * wr_stride) = acc[j];
+        }
+        __syncthreads();
+        for (int p = 0; p < n_passes; p++) {
+            int t = turn + p;
+            while (t >= n_waves) t -= n_waves;
+            if (w != t) continue;
+            const int slot = p * 64 + lane;
+            const int jq = (slot * recip_m) >> 16;  // slot / M = j*4 + kq
+            const int m = slot - jq * M;
+            const int tile = tile_begin + q * TB + (jq >> 2);
+            if (slot < n_slots && tile < tile_end) {
+                const float4_t *src = reinterpret_cast<const float4_t *>(smem + red_base + slot * kSlotPitch);
+                float4_t sum = src[0];
+                if (n_waves == kMaxWaves) {
+#pragma unroll
+                    for (int i = 1; i < kMaxWaves; i++) sum += src[i];
+                } else {
+                    for (int i = 1; i < n_waves; i++) sum += src[i];
+                }
+                // D[i][j] of the tile: this slot holds rows i = 4*kq .. 4*kq+3 of column j = m.
+                half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                *reinterpret_cast<half4_t *>(y + (int64_t)m * N + tile * kTileN + 4 * (jq & 3)) = h;
+            }
+        }
+        turn += n_passes;
+        while (turn >= n_waves) turn -= n_waves;
+    };
+
+    for (int q = 0; q < n_units; q += 2) {
+        process_unit(q, cwq[0]);
+        if (q + 1 < n_units) process_unit(q + 1, cwq[1]);
     }
 }
 
+#ifndef VQ_REPL_MIN
+#define VQ_REPL_MIN 2
+#endif
 constexpr size_t kDecodeLdsLimit = 160 * 1024;
 constexpr size_t kStageMinBytes = 32 * 1024;
-constexpr size_t kDisjointBudget = 96 * 1024;  // keep at least two workgroups per CU when staging beside the codebook
+constexpr size_t kDisjointBudget = 80 * 1024;  // keep two workgroups per CU when staging beside the codebook
 
-template <int VEC, typename CodeT, int STEPS>
-hipError_t launch_decode_steps(const ProblemB &p, hipStream_t s)
+template <int VEC, typename CodeT>
+hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
 {
-    typedef DecodeCfg<VEC, CodeT, STEPS> C;
-    constexpr int kSliceK = C::kSliceK;
-    const int slices = (p.K + kSliceK - 1) / kSliceK;
-    const int n_waves = slices < kMaxWaves ? slices : kMaxWaves;
-    const int n_chunks = (slices + n_waves - 1) / n_waves;
-    const int n_tiles = (p.N + kTileN - 1) / kTileN;
-    const int cb_bytes = p.entries * VEC * 2;
-    // Workgroups resident per CU: the kernel needs 129+ registers per lane, i.e. at most 3 waves
-    // per SIMD.
-    int per_cu = 12 / n_waves > 0 ? 12 / n_waves : 1;
+    typedef DecodeCfg<VEC, CodeT> C;
+    const int n_waves = p.K / kSliceK;
+    const int n_tiles = p.N / kTileN;
     const int cus = device_cu_count();
+    int per_cu = kMaxWaves / n_waves;  // workgroups resident per CU, by waves
     int grid = n_tiles < cus * per_cu ? n_tiles : cus * per_cu;
-    const int tiles_per_wg = (n_tiles + grid - 1) / grid;
-    // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time only
-    // when the workgroup gathers from it for several tiles.
-    const bool repl = p.entries <= 256 && tiles_per_wg >= 4;
-    const size_t base = (repl ? (size_t)p.entries * 256 : (size_t)((cb_bytes + 15) & ~15)) +
-                        (size_t)2 * n_waves * 64 * sizeof(float4_t);
-    const size_t stage = (size_t)n_waves * p.M * (kSliceK * 2 + 16);
+    int tiles_per_wg = (n_tiles + grid - 1) / grid;
+    // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time as
+    // soon as the workgroup gathers from it for more than one tile; so is the batched loop, whose
+    // short-unit path serves a workgroup with fewer tiles than a batch.
+    const bool repl = p.entries <= 256 && tiles_per_wg >= VQ_REPL_MIN;
+    const bool full = tiles_per_wg >= 2;
+    const int tb = full ? C::TB : 1;
+    const size_t table = repl ? (size_t)p.entries * 256 : (size_t)p.entries * VEC * 2;
+    const size_t base = table + (size_t)tb * 4 * p.M * kSlotPitch;
+    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * p.M * kStagePitch;
     size_t smem = base;
     int stage_off = -1, aliased = 0;
-    // Staging pays off when X is large enough for its scattered fetch to load the L1/L2 path;
-    // a small X is read directly (one LDS round trip less on the critical path).
-    if (n_chunks == 1 && (size_t)p.M * p.K * 2 > kStageMinBytes) {
-        if (base + stage <= kDisjointBudget) {
-            stage_off = (int)base;
-            smem = base + stage;
-        } else if (stage <= kDecodeLdsLimit) {
-            stage_off = 0;
-            aliased = 1;
-            smem = stage > base ? stage : base;
-        }
+    // X is staged beside the codebook and the slots when that leaves room for a second workgroup
+    // on the CU, over them otherwise.
+    if (base + stage <= kDisjointBudget) {
+        stage_off = (int)base;
+        smem = base + stage;
+    } else {
+        stage_off = 0;
+        aliased = 1;
+        smem = stage > base ? stage : base;
     }
     if ((size_t)per_cu * smem > kDecodeLdsLimit) {
         per_cu = (int)(kDecodeLdsLimit / smem) > 0 ? (int)(kDecodeLdsLimit / smem) : 1;
         grid = n_tiles < cus * per_cu ? n_tiles : cus * per_cu;
     }
-    auto kern = repl ? decode_kernel<VEC, CodeT, STEPS, true> : decode_kernel<VEC, CodeT, STEPS, false>;
+    auto kern = !full  ? decode_batched_kernel<VEC, CodeT, false, 1>
+                : repl ? decode_batched_kernel<VEC, CodeT, true, C::TB>
+                       : decode_batched_kernel<VEC, CodeT, false, C::TB>;
+    if (!full && repl) kern = decode_batched_kernel<VEC, CodeT, true, 1>;  // only where a full batch is one tile
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
-                       p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb, n_tiles / grid, n_tiles % grid, n_chunks, stage_off, aliased);
+                       p.y, p.M, p.K, p.N, p.entries, n_tiles / grid, n_tiles % grid, stage_off, aliased,
+                       (65536 + p.M - 1) / p.M);
     return hipGetLastError();
 }
 
-template <int VEC, typename CodeT>
-hipError_t launch_decode_typed(const ProblemB &p, hipStream_t s)
+// The batched kernel takes one codebook, K a multiple of 256 up to 4096 and N a multiple of 16.
+bool batched_supports(const ProblemB &p)
 {
-    // 512-wide K slices up to K = 4096 (eight waves cover it), 1024-wide beyond.
-    return p.K <= 8 * 512 ? launch_decode_steps<VEC, CodeT, 16>(p, s) : launch_decode_steps<VEC, CodeT, 32>(p, s);
+    // LDS: the plain codebook and the slots of the largest batch, and the staged X (which may lie over them)
+    const size_t base = (size_t)p.entries * p.vec * 2 + (size_t)4 * 4 * p.M * kSlotPitch;
+    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * p.M * kStagePitch;
+    return p.n_codebooks == 1 && p.K % kSliceK == 0 && p.K <= kSliceK * kMaxWaves && p.N % kTileN == 0 &&
+           base <= kDecodeLdsLimit && stage <= kDecodeLdsLimit;
 }
-
-template <int VEC, typename CodeT>
-bool decode_cfg_supports(const ProblemB &p)
-{
-    typedef DecodeCfg<VEC, CodeT> C;
-    return p.K % C::K_LANE == 0;  // whole 16-byte code loads, 16-byte aligned code rows
-}
-
-constexpr size_t kDecodeLdsBudget = 144 * 1024;  // codebook + reduction slots must fit the 160 KB LDS
 
 }  // namespace
 
 bool decode_supports(const ProblemB &p)
 {
-    if (p.M < 1 || p.M > kDecodeMaxM || p.N < 1 || p.K < 1) return false;
-    if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
-    if (p.n_codebooks > 1 && p.rows_per_cb % kTileN != 0) return false;
-    if ((size_t)p.entries * p.vec * 2 + 2 * kMaxWaves * 1024 > kDecodeLdsBudget) return false;
-    if (p.K % 8 != 0) return false;
-    if (((size_t)p.entries * p.vec * 2) % 16 != 0) return false;
-    const bool u8 = p.code_bits == 8;
-    switch (p.vec) {
-    case 8: return u8 ? decode_cfg_supports<8, uint8_t>(p) : decode_cfg_supports<8, uint16_t>(p);
-    case 4: return u8 ? decode_cfg_supports<4, uint8_t>(p) : decode_cfg_supports<4, uint16_t>(p);
-    default: return u8 ? decode_cfg_supports<2, uint8_t>(p) : decode_cfg_supports<2, uint16_t>(p);
-    }
+    return p.M >= 1 && p.M <= kDecodeMaxM && decode_general_supports(p);
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
-    // The kernel multiplies 16 rows of X at a time; taller X (up to kDecodeMaxM rows) goes in
+    // The kernels multiply 16 rows of X at a time; taller X (up to kDecodeMaxM rows) goes in
     // 16-row slabs, one launch each: still far better than a 256-row MFMA tile that is mostly
     // padding and fills only N/256 compute units.
     for (int m0 = 0; m0 < p.M; m0 += 16) {
@@ -441,10 +532,14 @@ hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
         q.y = p.y + (int64_t)m0 * p.N;
         q.M = p.M - m0 < 16 ? p.M - m0 : 16;
         hipError_t e;
-        switch (p.vec) {
-        case 8: e = u8 ? launch_decode_typed<8, uint8_t>(q, s) : launch_decode_typed<8, uint16_t>(q, s); break;
-        case 4: e = u8 ? launch_decode_typed<4, uint8_t>(q, s) : launch_decode_typed<4, uint16_t>(q, s); break;
-        default: e = u8 ? launch_decode_typed<2, uint8_t>(q, s) : launch_decode_typed<2, uint16_t>(q, s); break;
+        if (!batched_supports(q)) {
+            e = launch_decode_general(q, s);
+        } else {
+            switch (p.vec) {
+            case 8: e = u8 ? launch_decode_batched<8, uint8_t>(q, s) : launch_decode_batched<8, uint16_t>(q, s); break;
+            case 4: e = u8 ? launch_decode_batched<4, uint8_t>(q, s) : launch_decode_batched<4, uint16_t>(q, s); break;
+            default: e = u8 ? launch_decode_batched<2, uint8_t>(q, s) : launch_decode_batched<2, uint16_t>(q, s); break;
+            }
         }
         if (e != hipSuccess) return e;
     }
