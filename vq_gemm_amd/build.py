@@ -70,6 +70,26 @@ def _newer(target: str, deps) -> bool:
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
+# Kernels that issue loads by inline assembly and wait for them by hand keep values in registers
+# that the hardware is still writing; the compiler does not know, so a register it spills or copies
+# in that window would save stale data.  Their builds are therefore checked to be free of spills.
+NO_SPILL_KERNELS = {"vq_decode.hip": "decode_batched_kernel", "vq_prefill.hip": "prefill_kernelILi8E"}
+
+
+def _check_no_spills(asm_path: str, kernel_substr: str) -> None:
+    name, bad = None, []
+    with open(asm_path) as f:
+        for line in f:
+            line = line.strip()
+            if line.startswith(".name:"):
+                name = line.split(":", 1)[1].strip()
+            elif line.startswith(".vgpr_spill_count:") or line.startswith(".sgpr_spill_count:"):
+                if name and kernel_substr in name and int(line.split(":")[1]) != 0:
+                    bad.append(f"{name}: {line}")
+    if bad:
+        raise RuntimeError("register spills in a kernel that must have none:\n" + "\n".join(bad))
+
+
 def _headers():
     hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     inc = os.path.join(REPO_ROOT, "include")
@@ -88,7 +108,10 @@ def build_lib(force: bool = True, jobs: int = 6) -> str:
         s = os.path.join(CSRC, src)
         o = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
         if force or not _newer(o, [s] + hdrs):
-            _run([HIPCC] + HIP_FLAGS + ["-c", s, "-o", o])
+            extra = ["--save-temps=obj"] if src in NO_SPILL_KERNELS else []
+            _run([HIPCC] + HIP_FLAGS + extra + ["-c", s, "-o", o])
+            if extra:
+                _check_no_spills(o.replace(".o", f"-hip-amdgcn-amd-amdhsa-{ARCH}.s"), NO_SPILL_KERNELS[src])
         return o
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:

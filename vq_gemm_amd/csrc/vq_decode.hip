@@ -238,6 +238,10 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
 {
     typedef DecodeCfg<VEC, CodeT> C;
     typedef LaneCodes<VEC, CodeT> Codes;
+    // All kernel arguments are fetched at once: left to first use, each pointer costs the
+    // prologue a scalar-load round trip of its own.
+    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(M), "s"(K), "s"(N), "s"(entries), "s"(tiles_q),
+                 "s"(tiles_r), "s"(stage_off), "s"(aliased), "s"(recip_m));
     constexpr int kPieces = Operand<VEC>::kPieces;
     constexpr int kEntryBytes = VEC * 2;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -415,29 +419,47 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             for (int j = 0; j < TB; j++)
                 if (j < nt) *reinterpret_cast<float4_t *>(smem + wr_addr + j * wr_stride) = acc[j];
         }
-        __syncthreads();
-        for (int p = 0; p < n_passes; p++) {
-            int t = turn + p;
-            while (t >= n_waves) t -= n_waves;
-            if (w != t) continue;
-            const int slot = p * 64 + lane;
+        // A pass of the reduction: 64 slots, one per lane.  Where the slot goes is worked out
+        // first (`locate`), the sum and the store follow (`finish`).
+        struct Target { const float4_t *src; half_t *dst; bool live; };
+        auto locate = [&](int pass) {
+            const int slot = pass * 64 + lane;
             const int jq = (slot * recip_m) >> 16;  // slot / M = j*4 + kq
             const int m = slot - jq * M;
             const int tile = tile_begin + q * TB + (jq >> 2);
-            if (slot < n_slots && tile < tile_end) {
-                const float4_t *src = reinterpret_cast<const float4_t *>(smem + red_base + slot * kSlotPitch);
-                float4_t sum = src[0];
-                if (n_waves == kMaxWaves) {
+            Target t;
+            t.src = reinterpret_cast<const float4_t *>(smem + red_base + slot * kSlotPitch);
+            // D[i][j] of the tile: the slot holds rows i = 4*kq .. 4*kq+3 of column j = m.
+            t.dst = y + (int64_t)m * N + tile * kTileN + 4 * (jq & 3);
+            t.live = pass < n_passes && slot < n_slots && tile < tile_end;
+            return t;
+        };
+        auto finish = [&](const Target &t) {
+            if (!t.live) return;
+            float4_t sum;
+            if (n_waves == kMaxWaves) {
+                // four interleaved chains, to keep the run of dependent additions short
+                float4_t c[4];
 #pragma unroll
-                    for (int i = 1; i < kMaxWaves; i++) sum += src[i];
-                } else {
-                    for (int i = 1; i < n_waves; i++) sum += src[i];
-                }
-                // D[i][j] of the tile: this slot holds rows i = 4*kq .. 4*kq+3 of column j = m.
-                half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
-                *reinterpret_cast<half4_t *>(y + (int64_t)m * N + tile * kTileN + 4 * (jq & 3)) = h;
+                for (int i = 0; i < 4; i++) c[i] = t.src[i];
+#pragma unroll
+                for (int i = 4; i < kMaxWaves; i++) c[i & 3] += t.src[i];
+                sum = (c[0] + c[1]) + (c[2] + c[3]);
+            } else {
+                sum = t.src[0];
+                for (int i = 1; i < n_waves; i++) sum += t.src[i];
             }
-        }
+            half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+            *reinterpret_cast<half4_t *>(t.dst) = h;
+        };
+        // The waves take the passes in turn; a wave's first pass is located before the barrier,
+        // so that only the sum and the store follow it.
+        int pass = w - turn;
+        if (pass < 0) pass += n_waves;
+        const Target first = locate(pass);
+        __syncthreads();
+        finish(first);
+        for (pass += n_waves; pass < n_passes; pass += n_waves) finish(locate(pass));
         turn += n_passes;
         while (turn >= n_waves) turn -= n_waves;
     };
@@ -452,7 +474,6 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
 #define VQ_REPL_MIN 2
 #endif
 constexpr size_t kDecodeLdsLimit = 160 * 1024;
-constexpr size_t kStageMinBytes = 32 * 1024;
 constexpr size_t kDisjointBudget = 80 * 1024;  // keep two workgroups per CU when staging beside the codebook
 
 template <int VEC, typename CodeT>

@@ -175,7 +175,13 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         int k = super * C::K_SUPER + kg * C::K_LANE;
         if (TAIL && k >= K) k = 0;  // k-group 1 of a partial last super stage: any valid codes (operand is zeroed)
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) dst[nb] = load_16_untracked(code_row[nb] + k / VEC);
+        for (int nb = 0; nb < NB; nb++) {
+            // The codeword sizes below 16 bytes run out of registers; a register spilled while a
+            // hand-issued load is still writing it would save stale data, so these variants
+            // leave their code loads to the compiler's own (more conservative) waits.
+            if constexpr (VEC == 8) dst[nb] = load_16_untracked(code_row[nb] + k / VEC);
+            else dst[nb] = ld_global_16(code_row[nb] + k / VEC);
+        }
     };
 
     // ---- X staging: global -> LDS directly ------------------------------------------------
