@@ -47,8 +47,9 @@ def parse_args():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
     ap.add_argument("--probe", metavar="CONFIG", default=None,
-                    help="profiling aid: launch CONFIG (C1..C5) --steps times, cold-HBM rotation for the decode "
-                         "configs, followed by one 256 MiB device copy as a counter yardstick; prints no JSON")
+                    help="profiling aid: launch CONFIG (C1..C5, or a geometry-B shape M,K,N,vec,entries,code_bits) "
+                         "--steps times, cold-HBM rotation for the decode configs, followed by one 256 MiB "
+                         "device copy as a counter yardstick; prints no JSON")
     return ap.parse_args()
 
 
@@ -76,7 +77,12 @@ def main():
         torch.cuda.synchronize()
 
     if args.probe:
-        spec = CONFIGS[args.probe]
+        if args.probe in CONFIGS:
+            spec = CONFIGS[args.probe]
+        else:
+            from vq_gemm_amd.problems import GEOM_B, ProblemSpec
+            m, k, n, vec, entries, bits = (int(v) for v in args.probe.split(","))
+            spec = ProblemSpec("probe", GEOM_B, m, k, n, vec, entries, 1, bits)
         x, codes, cb = make_problem(spec, seed=42, device=dev)
         n_bufs = max(1, min(512, POOL_BYTES // spec.code_bytes)) if spec.M <= 16 else 1
         gen = torch.Generator(device=dev).manual_seed(1234)
