@@ -131,16 +131,25 @@ BATCHED_B = [
     ("u8v4_m2", 2, 4096, 16384, 4, 256, 8),
     ("u8v2_m16_k512", 16, 512, 16384, 2, 256, 8),
     ("u16v4_m9_e4096", 9, 4096, 12288, 4, 4096, 16),
+    # taller X: the 16-row slabs are a grid dimension of the same launch
+    ("u8v8_m100_slabs", 100, 1024, 4096, 8, 256, 8),
+    ("u16v4_m200_slabs", 200, 2048, 2048, 4, 4096, 16),
+    ("u8v8_m300_slabs", 300, 4096, 4096, 8, 256, 8),
+    # several codebooks: every workgroup works inside the rows of one
+    ("u8v8_m130_32_codebooks", 130, 4096, 4096, 8, 256, 8, 32),
+    ("u8v8_m2_7_codebooks", 2, 2048, 28672, 8, 256, 8, 7),
+    ("u16v4_m40_4_codebooks", 40, 1024, 8192, 4, 1024, 16, 4),
 ]
 
 
 @pytest.mark.parametrize("row", BATCHED_B, ids=[r[0] for r in BATCHED_B])
 def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
-    name, M, K, N, v, E, bits = row
-    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, 1, bits)
+    name, M, K, N, v, E, bits = row[:7]
+    G = row[7] if len(row) > 7 else 1
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
     x, codes, cb = make_problem(spec, seed=21, device=DEV)
     _say("batched decode", spec)
-    assert cabi.select_variant_b(M, K, N, v, E, 1, bits) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(M, K, N, v, E, G, bits) == cabi.VARIANT_DECODE
     y = cabi.e2e_gemm_b(x, codes, cb)
     torch.cuda.synchronize()
     w = vo.dequant_b(_np(codes), _np(cb))

@@ -74,8 +74,9 @@ ProblemB make_b(const void *x, const void *codes, const void *codebook, void *y,
 int select_b(const ProblemB &p, bool all_aligned16)
 {
     if (p.K == 0 || !all_aligned16) return VQGEMM_VARIANT_GENERIC;
-    if (decode_supports(p)) return VQGEMM_VARIANT_DECODE;  // M <= 64, in 16-row slabs
-    if (prefill_supports(p)) return VQGEMM_VARIANT_PREFILL;
+    const bool prefill_ok = prefill_supports(p);
+    if (decode_supports(p) && (!prefill_ok || decode_preferred(p))) return VQGEMM_VARIANT_DECODE;
+    if (prefill_ok) return VQGEMM_VARIANT_PREFILL;
     return VQGEMM_VARIANT_GENERIC;
 }
 

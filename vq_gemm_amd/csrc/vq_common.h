@@ -59,6 +59,8 @@ hipError_t launch_generic_b(const ProblemB &p, hipStream_t s);
 hipError_t launch_generic_a(const ProblemA &p, hipStream_t s);
 
 bool decode_supports(const ProblemB &p);
+// whether the decode path is expected to beat the prefill kernel on a shape it supports
+bool decode_preferred(const ProblemB &p);
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s);
 // the general kernel behind launch_decode_b: one slab of at most 16 rows of X
 bool decode_general_supports(const ProblemB &p);

@@ -31,7 +31,8 @@ constexpr int kTileN = 16;
 constexpr int kSliceK = 256;     // K owned by one wave
 constexpr int kSteps = 8;        // MFMA steps (32 k each) per slice
 constexpr int kMaxWaves = 16;    // 1024 threads, 128 registers per lane
-constexpr int kDecodeMaxM = 64;  // taller activations are served in 16-row slabs up to this height
+constexpr int kGeneralMaxM = 64;    // the general kernel: one launch per 16-row slab of X up to this height
+constexpr int kBatchedMaxM = 4096;  // the batched kernel: the slabs are a grid dimension
 constexpr int kStageK = 512;     // X is staged in pieces of 512 k of one row (1 KB, one wave instruction)
 constexpr int kStagePitch = kStageK * 2 + 16;  // LDS bytes per staged piece; the pad spreads rows over the banks
 
@@ -225,23 +226,33 @@ __device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff,
 //   * The partial results go to the LDS packed as [slot][wave], slot = (tile, k-group, X row)
 //     over the rows of X that exist only; a reducing wave takes 64 slots per pass, every lane
 //     summing the 16-byte entries of its slot, so a pass covers 16/M tiles.
-// `recip_m` = ceil(65536 / M), for the division of a slot number by M.
+// X taller than 16 rows is served by the second grid dimension: one 16-row slab per index.
+// `recip_tail` = ceil(65536 / rows of the last slab), for the division of a slot number by M.
 constexpr int kSlotPitch = 16 * kMaxWaves + 16;  // LDS bytes per slot; the pad spreads the slots over the banks
 
 template <int VEC, typename CodeT, bool REPL, int TB>
 __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
                                                                const CodeT *__restrict__ codes,
                                                                const half_t *__restrict__ cb,
-                                                               half_t *__restrict__ y, int M, int K, int N,
-                                                               int entries, int tiles_q, int tiles_r,
-                                                               int stage_off, int aliased, int recip_m)
+                                                               half_t *__restrict__ y, int m_total, int K, int N,
+                                                               int entries, int n_books, int wgs_per_cb,
+                                                               int books_per_wg, int tiles_per_cb, int tiles_q,
+                                                               int tiles_r, int stage_off, int aliased,
+                                                               int recip_tail)
 {
     typedef DecodeCfg<VEC, CodeT> C;
     typedef LaneCodes<VEC, CodeT> Codes;
     // All kernel arguments are fetched at once: left to first use, each pointer costs the
     // prologue a scalar-load round trip of its own.
-    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(M), "s"(K), "s"(N), "s"(entries), "s"(tiles_q),
-                 "s"(tiles_r), "s"(stage_off), "s"(aliased), "s"(recip_m));
+    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(m_total), "s"(K), "s"(N), "s"(entries),
+                 "s"(n_books), "s"(wgs_per_cb), "s"(books_per_wg), "s"(tiles_per_cb), "s"(tiles_q), "s"(tiles_r),
+                 "s"(stage_off), "s"(aliased), "s"(recip_tail));
+    // blockIdx.y picks the 16-row slab of X (and of Y) this workgroup multiplies.
+    const int slab_row = blockIdx.y * kTileN;
+    const int M = min(kTileN, m_total - slab_row);
+    const int recip_m = M == kTileN ? 65536 / kTileN : recip_tail;
+    x += (int64_t)slab_row * K;
+    y += (int64_t)slab_row * N;
     constexpr int kPieces = Operand<VEC>::kPieces;
     constexpr int kEntryBytes = VEC * 2;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -256,11 +267,19 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     const uint32_t gather_base = REPL ? (lane % (256 / kEntryBytes)) * kEntryBytes : 0;
     const uint32_t red_base = cb_slots * 16;
 
-    const int wg = blockIdx.x;
-    const int tile_begin = wg * tiles_q + min(wg, tiles_r);
-    const int tile_end = tile_begin + tiles_q + (wg < tiles_r ? 1 : 0);
-    if (tile_begin >= tile_end) return;
-    const int n_units = (tile_end - tile_begin + TB - 1) / TB;
+    // blockIdx.x picks the codebooks.  Either wgs_per_cb workgroups share the tiles_per_cb tiles
+    // of one codebook (a contiguous range each: tiles_q, one more for the first tiles_r; quotient
+    // and remainder computed by the host), or one workgroup takes books_per_wg whole codebooks in
+    // turn, keeping its X and replacing the table in the LDS between them.
+    const int book_begin = wgs_per_cb > 1 ? (int)blockIdx.x / wgs_per_cb : (int)blockIdx.x * books_per_wg;
+    const int book_end = min(n_books, book_begin + books_per_wg);
+    const int wg = wgs_per_cb > 1 ? (int)blockIdx.x - book_begin * wgs_per_cb : 0;
+    int book = book_begin;
+    int tile_begin = book * tiles_per_cb + wg * tiles_q + min(wg, tiles_r);
+    int tile_end = tile_begin + tiles_q + (wg < tiles_r ? 1 : 0);
+    if (book >= book_end || tile_begin >= tile_end) return;
+    cb += (int64_t)book * entries * VEC;
+    int n_units = (tile_end - tile_begin + TB - 1) / TB;
 
     // Codes: lane offset inside a tile, scalar base per tile.  The last unit may hold fewer than
     // TB tiles.
@@ -311,7 +330,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             for (int i = threadIdx.x; i < cb_slots; i += blockDim.x) cb_lds[i] = read_slot(i);
         }
     };
-    if (cb_in_regs) {
+    auto fetch_codebook = [&]() {
         // (whole waves past the end of the table issue no load: every vector memory instruction
         // of the prologue queues behind the others of the CU)
 #pragma unroll
@@ -319,7 +338,8 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             const int i = threadIdx.x + j * blockDim.x;
             if ((i & ~63) < cb_slots) cb_regs[j] = read_slot(i < cb_slots ? i : 0);
         }
-    }
+    };
+    if (cb_in_regs) fetch_codebook();
 
     // X slice of the wave -> registers, in MFMA operand order; rows past M are zero.
     const int k0 = w * kSliceK;
@@ -464,9 +484,35 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
         while (turn >= n_waves) turn -= n_waves;
     };
 
-    for (int q = 0; q < n_units; q += 2) {
-        process_unit(q, cwq[0]);
-        if (q + 1 < n_units) process_unit(q + 1, cwq[1]);
+    for (;;) {
+        for (int q = 0; q < n_units; q += 2) {
+            process_unit(q, cwq[0]);
+            if (q + 1 < n_units) process_unit(q + 1, cwq[1]);
+        }
+        if (++book >= book_end) break;
+        // Next codebook: all of its tiles (books_per_wg > 1 means whole codebooks).  Its first codes
+        // are requested before the table is replaced, to overlap the two latencies.
+        tile_begin = book * tiles_per_cb;
+        tile_end = tile_begin + tiles_per_cb;
+        n_units = (tiles_per_cb + TB - 1) / TB;
+        load_unit(0, cwq[0]);
+        if (n_units > 1) load_unit(1, cwq[1]);
+        cb += (int64_t)entries * VEC;
+        __syncthreads();  // every gather from the old table has been consumed, every slot read
+        {
+            // (the thread index goes through an empty asm so that nothing derived from it is kept
+            // in registers across the tile loop just to be reused here)
+            int tid = threadIdx.x;
+            asm volatile("" : "+v"(tid));
+            for (int i0 = tid; i0 < cb_slots; i0 += 2 * (int)blockDim.x) {
+                const int i1 = i0 + (int)blockDim.x;
+                const uint4_t a = read_slot(i0);
+                const uint4_t b = read_slot(i1 < cb_slots ? i1 : i0);
+                cb_lds[i0] = a;
+                if (i1 < cb_slots) cb_lds[i1] = b;
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -476,25 +522,54 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
 constexpr size_t kDecodeLdsLimit = 160 * 1024;
 constexpr size_t kDisjointBudget = 80 * 1024;  // keep two workgroups per CU when staging beside the codebook
 
+// Workgroups per 16-row slab of X and the tiles each of them gets.
+struct BatchedGrid {
+    int n_slabs, per_slab, wgs_per_cb, books_per_wg, tiles_per_cb, tiles_per_wg, per_cu;
+};
+
+BatchedGrid batched_grid(const ProblemB &p)
+{
+    BatchedGrid g;
+    const int n_waves = p.K / kSliceK;
+    g.tiles_per_cb = p.rows_per_cb / kTileN;
+    g.per_cu = kMaxWaves / n_waves;  // workgroups resident per CU, by waves
+    g.n_slabs = (p.M + kTileN - 1) / kTileN;
+    // As many workgroups as the device holds at once, shared among the slabs.  Within a slab a
+    // workgroup reads one codebook at a time: several workgroups share the tiles of a codebook,
+    // or one takes several whole codebooks in turn.
+    const int resident = device_cu_count() * g.per_cu;
+    int per_slab = resident / g.n_slabs;
+    if (per_slab < 1) per_slab = 1;
+    if (per_slab >= p.n_codebooks) {
+        const int per_cb = per_slab / p.n_codebooks;
+        g.wgs_per_cb = per_cb < g.tiles_per_cb ? per_cb : g.tiles_per_cb;
+        g.books_per_wg = 1;
+        g.per_slab = g.wgs_per_cb * p.n_codebooks;
+    } else {
+        g.wgs_per_cb = 1;
+        g.books_per_wg = (p.n_codebooks + per_slab - 1) / per_slab;
+        g.per_slab = (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg;
+    }
+    g.tiles_per_wg = (g.tiles_per_cb + g.wgs_per_cb - 1) / g.wgs_per_cb;  // per codebook
+    return g;
+}
+
 template <int VEC, typename CodeT>
 hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
 {
     typedef DecodeCfg<VEC, CodeT> C;
     const int n_waves = p.K / kSliceK;
-    const int n_tiles = p.N / kTileN;
-    const int cus = device_cu_count();
-    int per_cu = kMaxWaves / n_waves;  // workgroups resident per CU, by waves
-    int grid = n_tiles < cus * per_cu ? n_tiles : cus * per_cu;
-    int tiles_per_wg = (n_tiles + grid - 1) / grid;
+    const int m_slab = p.M < kTileN ? p.M : kTileN;  // rows of X one workgroup multiplies
+    const BatchedGrid g = batched_grid(p);
     // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time as
     // soon as the workgroup gathers from it for more than one tile; so is the batched loop, whose
     // short-unit path serves a workgroup with fewer tiles than a batch.
-    const bool repl = p.entries <= 256 && tiles_per_wg >= VQ_REPL_MIN;
-    const bool full = tiles_per_wg >= 2;
+    const bool repl = p.entries <= 256 && g.tiles_per_wg >= VQ_REPL_MIN;
+    const bool full = g.tiles_per_wg >= 2;
     const int tb = full ? C::TB : 1;
     const size_t table = repl ? (size_t)p.entries * 256 : (size_t)p.entries * VEC * 2;
-    const size_t base = table + (size_t)tb * 4 * p.M * kSlotPitch;
-    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * p.M * kStagePitch;
+    const size_t base = table + (size_t)tb * 4 * m_slab * kSlotPitch;
+    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * m_slab * kStagePitch;
     size_t smem = base;
     int stage_off = -1, aliased = 0;
     // X is staged beside the codebook and the slots when that leaves room for a second workgroup
@@ -507,29 +582,28 @@ hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
         aliased = 1;
         smem = stage > base ? stage : base;
     }
-    if ((size_t)per_cu * smem > kDecodeLdsLimit) {
-        per_cu = (int)(kDecodeLdsLimit / smem) > 0 ? (int)(kDecodeLdsLimit / smem) : 1;
-        grid = n_tiles < cus * per_cu ? n_tiles : cus * per_cu;
-    }
     auto kern = !full  ? decode_batched_kernel<VEC, CodeT, false, 1>
                 : repl ? decode_batched_kernel<VEC, CodeT, true, C::TB>
                        : decode_batched_kernel<VEC, CodeT, false, C::TB>;
     if (!full && repl) kern = decode_batched_kernel<VEC, CodeT, true, 1>;  // only where a full batch is one tile
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
-                       p.y, p.M, p.K, p.N, p.entries, n_tiles / grid, n_tiles % grid, stage_off, aliased,
-                       (65536 + p.M - 1) / p.M);
+    const int tail_rows = p.M - (g.n_slabs - 1) * kTileN;
+    hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(n_waves * 64), smem, s, p.x,
+                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.n_codebooks,
+                       g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, g.tiles_per_cb / g.wgs_per_cb,
+                       g.tiles_per_cb % g.wgs_per_cb, stage_off, aliased, (65536 + tail_rows - 1) / tail_rows);
     return hipGetLastError();
 }
 
-// The batched kernel takes one codebook, K a multiple of 256 up to 4096 and N a multiple of 16.
+// The batched kernel takes K a multiple of 256 up to 4096 and N (and the rows per codebook) a multiple of 16.
 bool batched_supports(const ProblemB &p)
 {
     // LDS: the plain codebook and the slots of the largest batch, and the staged X (which may lie over them)
-    const size_t base = (size_t)p.entries * p.vec * 2 + (size_t)4 * 4 * p.M * kSlotPitch;
-    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * p.M * kStagePitch;
-    return p.n_codebooks == 1 && p.K % kSliceK == 0 && p.K <= kSliceK * kMaxWaves && p.N % kTileN == 0 &&
+    const int m_slab = p.M < kTileN ? p.M : kTileN;
+    const size_t base = (size_t)p.entries * p.vec * 2 + (size_t)4 * 4 * m_slab * kSlotPitch;
+    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * m_slab * kStagePitch;
+    return p.rows_per_cb % kTileN == 0 && p.K % kSliceK == 0 && p.K <= kSliceK * kMaxWaves && p.N % kTileN == 0 &&
            base <= kDecodeLdsLimit && stage <= kDecodeLdsLimit;
 }
 
@@ -537,31 +611,51 @@ bool batched_supports(const ProblemB &p)
 
 bool decode_supports(const ProblemB &p)
 {
-    return p.M >= 1 && p.M <= kDecodeMaxM && decode_general_supports(p);
+    if (p.M < 1 || !decode_general_supports(p)) return false;
+    return p.M <= kGeneralMaxM || (p.M <= kBatchedMaxM && batched_supports(p));
+}
+
+// Rough times (us) of the two tiled kernels on a shape both can take; the automatic choice takes
+// the smaller.  The decode path costs a prologue plus ~0.6 us per tile and CU at K = 4096 (in
+// proportion below); the prefill kernel ~1.5 us per 64-deep stage of its 256x256 tiles, one
+// round of tiles per 256 CUs, however few of them there are.
+bool decode_preferred(const ProblemB &p)
+{
+    if (!decode_supports(p)) return false;
+    if (p.M <= kGeneralMaxM) return true;
+    const BatchedGrid g = batched_grid(p);
+    const int cus = device_cu_count();
+    // rounds of resident workgroups; per workgroup a prologue, its tiles (at 1/per_cu of the CU's
+    // throughput) and the codebook switches
+    const int rounds_d = (g.per_slab * g.n_slabs + cus * g.per_cu - 1) / (cus * g.per_cu);
+    const double t_decode = rounds_d * (3.0 + g.tiles_per_wg * g.books_per_wg * 0.6 * (p.K / 4096.0) * g.per_cu +
+                                        (g.books_per_wg - 1) * 1.5);
+    const int rounds_p = (((p.M + 255) / 256) * ((p.N + 255) / 256) + cus - 1) / cus;
+    const double t_prefill = 8.0 + rounds_p * (p.K / 64.0) * 1.5;
+    return t_decode <= t_prefill;
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
-    // The kernels multiply 16 rows of X at a time; taller X (up to kDecodeMaxM rows) goes in
-    // 16-row slabs, one launch each: still far better than a 256-row MFMA tile that is mostly
-    // padding and fills only N/256 compute units.
+    if (batched_supports(p)) {
+        // one launch, the 16-row slabs of X on the second grid dimension
+        switch (p.vec) {
+        case 8: return u8 ? launch_decode_batched<8, uint8_t>(p, s) : launch_decode_batched<8, uint16_t>(p, s);
+        case 4: return u8 ? launch_decode_batched<4, uint8_t>(p, s) : launch_decode_batched<4, uint16_t>(p, s);
+        default: return u8 ? launch_decode_batched<2, uint8_t>(p, s) : launch_decode_batched<2, uint16_t>(p, s);
+        }
+    }
+    // The general kernel multiplies 16 rows of X per launch; taller X goes in slabs, one launch
+    // each: still far better than a 256-row MFMA tile that is mostly padding and fills only
+    // N/256 compute units.
     for (int m0 = 0; m0 < p.M; m0 += 16) {
         ProblemB q = p;
         q.x = p.x + (int64_t)m0 * p.K;
         q.y = p.y + (int64_t)m0 * p.N;
         q.M = p.M - m0 < 16 ? p.M - m0 : 16;
-        hipError_t e;
-        if (!batched_supports(q)) {
-            e = launch_decode_general(q, s);
-        } else {
-            switch (p.vec) {
-            case 8: e = u8 ? launch_decode_batched<8, uint8_t>(q, s) : launch_decode_batched<8, uint16_t>(q, s); break;
-            case 4: e = u8 ? launch_decode_batched<4, uint8_t>(q, s) : launch_decode_batched<4, uint16_t>(q, s); break;
-            default: e = u8 ? launch_decode_batched<2, uint8_t>(q, s) : launch_decode_batched<2, uint16_t>(q, s); break;
-            }
-        }
+        const hipError_t e = launch_decode_general(q, s);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
