@@ -139,6 +139,13 @@ BATCHED_B = [
     ("u8v8_m130_32_codebooks", 130, 4096, 4096, 8, 256, 8, 32),
     ("u8v8_m2_7_codebooks", 2, 2048, 28672, 8, 256, 8, 7),
     ("u16v4_m40_4_codebooks", 40, 1024, 8192, 4, 1024, 16, 4),
+    # K beyond 16 slices of 256: chunks of K, sums carried in the LDS (uneven chunks: 43 = 15+14+14 slices)
+    ("u8v8_m1_k8192", 1, 8192, 8192, 8, 256, 8),
+    ("u8v8_m16_k11008", 16, 11008, 4096, 8, 256, 8),
+    ("u8v8_m40_k14336_4_codebooks", 40, 14336, 2048, 8, 256, 8, 4),
+    ("u16v4_m3_k6144", 3, 6144, 12288, 4, 4096, 16),
+    ("u8v8_m200_k8192", 200, 8192, 4096, 8, 256, 8),
+    ("u8v8_m1_k28672", 1, 28672, 8192, 8, 256, 8),
 ]
 
 

@@ -134,6 +134,14 @@ __device__ __forceinline__ void wait_lgkmcnt_upto(int n)
     }
 }
 
+// Returns v through an empty asm: the compiler cannot tell that it is loop invariant, so nothing
+// derived from it is computed ahead of the tile loop and kept in registers through it.
+__device__ __forceinline__ int opaque(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 // One 8-half MFMA operand as the pieces it is gathered in: one codeword per piece.
 template <int VEC> struct OperandPiece;
 template <> struct OperandPiece<8> { typedef uint4_t type; };
@@ -229,6 +237,8 @@ __device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff,
 // X taller than 16 rows is served by the second grid dimension: one 16-row slab per index.
 // `recip_tail` = ceil(65536 / rows of the last slab), for the division of a slot number by M.
 constexpr int kSlotPitch = 16 * kMaxWaves + 16;  // LDS bytes per slot; the pad spreads the slots over the banks
+// what the X staging area lies over (it is only live while X is being loaded)
+constexpr int kStageOverTable = 1, kStageOverSlots = 2;
 
 template <int VEC, typename CodeT, bool REPL, int TB>
 __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
@@ -237,7 +247,8 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
                                                                half_t *__restrict__ y, int m_total, int K, int N,
                                                                int entries, int n_books, int wgs_per_cb,
                                                                int books_per_wg, int tiles_per_cb, int tiles_q,
-                                                               int tiles_r, int stage_off, int aliased,
+                                                               int tiles_r, int n_chunks, int red_off,
+                                                               int stage_off, int stage_over, int acc_off,
                                                                int recip_tail)
 {
     typedef DecodeCfg<VEC, CodeT> C;
@@ -246,7 +257,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     // prologue a scalar-load round trip of its own.
     asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(m_total), "s"(K), "s"(N), "s"(entries),
                  "s"(n_books), "s"(wgs_per_cb), "s"(books_per_wg), "s"(tiles_per_cb), "s"(tiles_q), "s"(tiles_r),
-                 "s"(stage_off), "s"(aliased), "s"(recip_tail));
+                 "s"(n_chunks), "s"(red_off), "s"(stage_off), "s"(stage_over), "s"(acc_off), "s"(recip_tail));
     // blockIdx.y picks the 16-row slab of X (and of Y) this workgroup multiplies.
     const int slab_row = blockIdx.y * kTileN;
     const int M = min(kTileN, m_total - slab_row);
@@ -256,7 +267,10 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     constexpr int kPieces = Operand<VEC>::kPieces;
     constexpr int kEntryBytes = VEC * 2;
     extern __shared__ __align__(16) uint8_t smem[];
-    const int n_waves = blockDim.x >> 6;  // = K / 256: wave w owns K slice w
+    // K goes in n_chunks chunks of (at most) n_waves slices of 256 k: wave w owns slice w of the
+    // current chunk; the last chunk may leave the upper waves without one.
+    const int n_waves = blockDim.x >> 6;
+    const int total_slices = K / kSliceK;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int r16 = lane & 15;  // W row within the tile (A operand) / X row m (B operand)
@@ -265,7 +279,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     const int cb_slots = REPL ? entries * 16 : entries * kEntryBytes / 16;  // 16-byte slots of the LDS table
     uint4_t *cb_lds = reinterpret_cast<uint4_t *>(smem);
     const uint32_t gather_base = REPL ? (lane % (256 / kEntryBytes)) * kEntryBytes : 0;
-    const uint32_t red_base = cb_slots * 16;
+    const uint32_t red_base = red_off;
 
     // blockIdx.x picks the codebooks.  Either wgs_per_cb workgroups share the tiles_per_cb tiles
     // of one codebook (a contiguous range each: tiles_q, one more for the first tiles_r; quotient
@@ -280,17 +294,21 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     if (book >= book_end || tile_begin >= tile_end) return;
     cb += (int64_t)book * entries * VEC;
     int n_units = (tile_end - tile_begin + TB - 1) / TB;
+    int chunk = 0;
+    int n_act = min(n_waves, total_slices);  // waves with a slice in the current chunk
+    bool active = w < n_act;
 
-    // Codes: lane offset inside a tile, scalar base per tile.  The last unit may hold fewer than
-    // TB tiles.
+    // Codes: lane offset inside a tile and chunk, scalar base per tile and chunk.  The last unit
+    // may hold fewer than TB tiles.
     const uint32_t voff = (uint32_t)((r16 * J + (w * kSliceK + kq * C::K_LANE) / VEC) * (int)sizeof(CodeT));
     const int64_t tile_bytes = (int64_t)kTileN * J * (int)sizeof(CodeT);
+    const int chunk_bytes = n_waves * kSliceK / VEC * (int)sizeof(CodeT);
     auto load_unit = [&](int q, Codes (&cw)[TB]) {
 #pragma unroll
         for (int j = 0; j < TB; j++) {
             const int tile = tile_begin + q * TB + j;
             if (tile >= tile_end) break;
-            const uint8_t *sbase = reinterpret_cast<const uint8_t *>(codes) + tile * tile_bytes;
+            const uint8_t *sbase = reinterpret_cast<const uint8_t *>(codes) + tile * tile_bytes + chunk * chunk_bytes;
             if constexpr (C::LPT >= 1) cw[j].template load_async_s<0>(0, voff, sbase);
             if constexpr (C::LPT >= 2) cw[j].template load_async_s<4 * C::LB>(1, voff, sbase);
             if constexpr (C::LPT >= 3) cw[j].template load_async_s<8 * C::LB>(2, voff, sbase);
@@ -300,8 +318,12 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     };
     // Two units of codes are in flight: ring slot q % 2 holds unit q.
     Codes cwq[2][TB];
-    load_unit(0, cwq[0]);
-    if (n_units > 1) load_unit(1, cwq[1]);
+    auto load_first_units = [&]() {
+        if (!active) return;
+        load_unit(0, cwq[0]);
+        if (n_units > 1) load_unit(1, cwq[1]);
+    };
+    load_first_units();
 
     // Codebook: global -> registers -> LDS, fetched now, stored once the LDS is free.
     constexpr int kCbRegs = 4;
@@ -330,7 +352,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             for (int i = threadIdx.x; i < cb_slots; i += blockDim.x) cb_lds[i] = read_slot(i);
         }
     };
-    auto fetch_codebook = [&]() {
+    if (cb_in_regs) {
         // (whole waves past the end of the table issue no load: every vector memory instruction
         // of the prologue queues behind the others of the CU)
 #pragma unroll
@@ -338,36 +360,45 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             const int i = threadIdx.x + j * blockDim.x;
             if ((i & ~63) < cb_slots) cb_regs[j] = read_slot(i < cb_slots ? i : 0);
         }
-    };
-    if (cb_in_regs) fetch_codebook();
+    }
 
-    // X slice of the wave -> registers, in MFMA operand order; rows past M are zero.
-    const int k0 = w * kSliceK;
-    auto step_k = [&](int s) { return (s / C::SPL) * C::K_WAVE + kq * C::K_LANE + (s % C::SPL) * 8; };
+    // X slice of the wave -> registers, in MFMA operand order; rows past M are zero.  Through the
+    // LDS in pieces of 512 k of one row (1 KB, contiguous): a few whole-wave copies per workgroup
+    // instead of eight mostly idle loads per wave.  Every vector memory instruction of the
+    // prologue queues behind the others of the CU, so their number is what the first tile waits
+    // for.  Piece (row i, block b of the chunk) sits at (b*M + i) * kStagePitch.
     half8_t xr[kSteps];
-    {
-        // Through the LDS in pieces of 512 k of one row (1 KB, contiguous): a few whole-wave
-        // copies per workgroup instead of eight mostly idle loads per wave.  Every vector memory
-        // instruction of the prologue queues behind the others of the CU, so their number is
-        // what the first tile waits for.
-        const int n_blocks = K / kStageK + (K % kStageK ? 1 : 0);
+    auto stage_x = [&]() {
+        const int kc0 = chunk * n_waves * kSliceK;
+        const int n_blocks = (n_act * kSliceK + kStageK - 1) / kStageK;
+        const int ln = opaque(lane);
         for (int pc = w; pc < n_blocks * M; pc += n_waves) {
             const int b = pc / M, i = pc - b * M;
-            const int kl = b * kStageK + 8 * lane;
+            const int kl = kc0 + b * kStageK + 8 * ln;
             load_to_lds_16(stage_off + pc * kStagePitch, (uint32_t)((i * K + (kl < K ? kl : 0)) * 2), x);
         }
-        const uint32_t win = stage_off + ((k0 / kStageK) * M + r16) * kStagePitch + (k0 % kStageK) * 2;
-        if (!aliased) store_codebook();
-        wait_vmcnt<0>();
-        __syncthreads();  // pieces staged by the other waves
+    };
+    auto pick_x = [&]() {
+        const int k0 = w * kSliceK;  // inside the chunk
+        const int ln = opaque(lane);
+        const int row = ln & 15, kg = ln >> 4;
+        const uint32_t win = stage_off + ((k0 / kStageK) * M + row) * kStagePitch + (k0 % kStageK) * 2;
 #pragma unroll
         for (int s = 0; s < kSteps; s++) {
+            const int k = (s / C::SPL) * C::K_WAVE + kg * C::K_LANE + (s % C::SPL) * 8;
             uint4_t v = {0u, 0u, 0u, 0u};
-            if (r16 < M) v = *reinterpret_cast<const uint4_t *>(smem + win + step_k(s) * 2);
+            if (active && row < M) v = *reinterpret_cast<const uint4_t *>(smem + win + k * 2);
             xr[s] = as_half8(v);
         }
-        if (aliased) {
-            __syncthreads();  // every wave has picked up its X before the codebook overwrites it
+    };
+    stage_x();
+    if (!(stage_over & kStageOverTable)) store_codebook();
+    wait_vmcnt<0>();
+    __syncthreads();  // pieces staged by the other waves
+    pick_x();
+    if (stage_over) {
+        __syncthreads();  // every wave has picked up its X before the staging area is written again
+        if (stage_over & kStageOverTable) {
             store_codebook();
             __syncthreads();
         }
@@ -382,73 +413,77 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     int turn = 0;  // the wave that takes the next reduction pass
 
     auto process_unit = [&](int q, Codes (&cur)[TB]) {
-        // This unit's codes have landed when only the loads of the next unit are out (a short last
-        // unit has fewer of them: then everything is awaited).
         const int nt = min(TB, tile_end - (tile_begin + q * TB));  // tiles of this unit
-        if (tile_begin + (q + 2) * TB <= tile_end) wait_vmcnt<TB * C::LPT>();
-        else wait_vmcnt<0>();
-#pragma unroll
-        for (int j = 0; j < TB; j++) cur[j].pin();
-
         float4_t acc[TB];
         const float4_t c0 = {0.f, 0.f, 0.f, 0.f};
-        if (nt == TB) {
-            // One branch-free stream of TB*8 MFMA steps; ops[] holds the gathered operands of a
-            // tile, and each is replaced by the next tile's as soon as it has been multiplied.
-            Operand<VEC> ops[kSteps];
+        if (active) {
+            // This unit's codes have landed when only the loads of the next unit are out (a short
+            // last unit has fewer of them: then everything is awaited).
+            if (tile_begin + (q + 2) * TB <= tile_end) wait_vmcnt<TB * C::LPT>();
+            else wait_vmcnt<0>();
 #pragma unroll
-            for (int s = 0; s < kSteps; s++) gather_issue<VEC, CodeT, REPL>(ops[s], cur[0], s, gather_base);
+            for (int j = 0; j < TB; j++) cur[j].pin();
+
+            if (nt == TB) {
+                // One branch-free stream of TB*8 MFMA steps; ops[] holds the gathered operands of a
+                // tile, and each is replaced by the next tile's as soon as it has been multiplied.
+                Operand<VEC> ops[kSteps];
 #pragma unroll
-            for (int i = 0; i < TB * kSteps; i++) {
-                const int j = i / kSteps, s = i % kSteps;
-                Operand<VEC> &o = ops[s];
-                const int left = TB * kSteps - 1 - i;  // steps after this one
-                wait_lgkmcnt_upto((left < kSteps - 1 ? left : kSteps - 1) * kPieces);  // younger gathers in flight
-                o.pin();
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.value(), xr[s], s == 0 ? c0 : acc[j], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                const int t = i + kSteps;
-                if (t < TB * kSteps) gather_issue<VEC, CodeT, REPL>(o, cur[t / kSteps], t % kSteps, gather_base);
-                // All gather addresses of the unit are computed: its ring slot takes the unit after next.
-                if (t == TB * kSteps - 1 || (TB == 1 && i == 0))
-                    if (q + 2 < n_units) load_unit(q + 2, cur);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-            // Short last unit: tile by tile, nothing in flight from one tile to the next.
+                for (int s = 0; s < kSteps; s++) gather_issue<VEC, CodeT, REPL>(ops[s], cur[0], s, gather_base);
 #pragma unroll
-            for (int j = 0; j < TB; j++) {
-                acc[j] = c0;
-                if (j < nt) {
-                    Operand<VEC> ops[kSteps];
+                for (int i = 0; i < TB * kSteps; i++) {
+                    const int j = i / kSteps, s = i % kSteps;
+                    Operand<VEC> &o = ops[s];
+                    const int left = TB * kSteps - 1 - i;  // steps after this one
+                    wait_lgkmcnt_upto((left < kSteps - 1 ? left : kSteps - 1) * kPieces);  // younger gathers in flight
+                    o.pin();
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.value(), xr[s], s == 0 ? c0 : acc[j], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int t = i + kSteps;
+                    if (t < TB * kSteps) gather_issue<VEC, CodeT, REPL>(o, cur[t / kSteps], t % kSteps, gather_base);
+                    // All gather addresses of the unit are computed: its ring slot takes the unit after next.
+                    if (t == TB * kSteps - 1 || (TB == 1 && i == 0))
+                        if (q + 2 < n_units) load_unit(q + 2, cur);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                // Short last unit: tile by tile, nothing in flight from one tile to the next.
 #pragma unroll
-                    for (int s = 0; s < kSteps; s++) gather_issue<VEC, CodeT, REPL>(ops[s], cur[j], s, gather_base);
+                for (int j = 0; j < TB; j++) {
+                    acc[j] = c0;
+                    if (j < nt) {
+                        Operand<VEC> ops[kSteps];
 #pragma unroll
-                    for (int s = 0; s < kSteps; s++) {
-                        wait_lgkmcnt_upto((kSteps - 1 - s) * kPieces);
-                        ops[s].pin();
-                        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ops[s].value(), xr[s], acc[j], 0, 0, 0);
+                        for (int s = 0; s < kSteps; s++) gather_issue<VEC, CodeT, REPL>(ops[s], cur[j], s, gather_base);
+#pragma unroll
+                        for (int s = 0; s < kSteps; s++) {
+                            wait_lgkmcnt_upto((kSteps - 1 - s) * kPieces);
+                            ops[s].pin();
+                            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ops[s].value(), xr[s], acc[j], 0, 0, 0);
+                        }
                     }
                 }
             }
         }
 
         if (q > 0) __syncthreads();  // the reducers of the previous unit are done with the slots
-        if (r16 < M) {
+        if (active && r16 < M) {
 #pragma unroll
             for (int j = 0; j < TB; j++)
                 if (j < nt) *reinterpret_cast<float4_t *>(smem + wr_addr + j * wr_stride) = acc[j];
         }
         // A pass of the reduction: 64 slots, one per lane.  Where the slot goes is worked out
         // first (`locate`), the sum and the store follow (`finish`).
-        struct Target { const float4_t *src; half_t *dst; bool live; };
+        struct Target { uint32_t src, carry; half_t *dst; bool live; };  // LDS offsets, output address
         auto locate = [&](int pass) {
-            const int slot = pass * 64 + lane;
+            const int slot = pass * 64 + opaque(lane);
             const int jq = (slot * recip_m) >> 16;  // slot / M = j*4 + kq
             const int m = slot - jq * M;
             const int tile = tile_begin + q * TB + (jq >> 2);
             Target t;
-            t.src = reinterpret_cast<const float4_t *>(smem + red_base + slot * kSlotPitch);
+            t.src = red_base + slot * kSlotPitch;
+            // with several chunks the sums are carried from chunk to chunk in the LDS, one entry per slot of the range
+            t.carry = (uint32_t)acc_off + (uint32_t)(q * n_slots + slot) * 16u;
             // D[i][j] of the tile: the slot holds rows i = 4*kq .. 4*kq+3 of column j = m.
             t.dst = y + (int64_t)m * N + tile * kTileN + 4 * (jq & 3);
             t.live = pass < n_passes && slot < n_slots && tile < tile_end;
@@ -456,21 +491,28 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
         };
         auto finish = [&](const Target &t) {
             if (!t.live) return;
+            const float4_t *src = reinterpret_cast<const float4_t *>(smem + t.src);
             float4_t sum;
-            if (n_waves == kMaxWaves) {
+            if (n_act == kMaxWaves) {
                 // four interleaved chains, to keep the run of dependent additions short
                 float4_t c[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) c[i] = t.src[i];
+                for (int i = 0; i < 4; i++) c[i] = src[i];
 #pragma unroll
-                for (int i = 4; i < kMaxWaves; i++) c[i & 3] += t.src[i];
+                for (int i = 4; i < kMaxWaves; i++) c[i & 3] += src[i];
                 sum = (c[0] + c[1]) + (c[2] + c[3]);
             } else {
-                sum = t.src[0];
-                for (int i = 1; i < n_waves; i++) sum += t.src[i];
+                sum = src[0];
+                for (int i = 1; i < n_act; i++) sum += src[i];
             }
-            half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
-            *reinterpret_cast<half4_t *>(t.dst) = h;
+            float4_t *carry = reinterpret_cast<float4_t *>(smem + t.carry);
+            if (chunk > 0) sum += *carry;
+            if (chunk < n_chunks - 1) {
+                *carry = sum;
+            } else {
+                half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
+                *reinterpret_cast<half4_t *>(t.dst) = h;
+            }
         };
         // The waves take the passes in turn; a wave's first pass is located before the barrier,
         // so that only the sum and the store follow it.
@@ -489,17 +531,23 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             process_unit(q, cwq[0]);
             if (q + 1 < n_units) process_unit(q + 1, cwq[1]);
         }
-        if (++book >= book_end) break;
-        // Next codebook: all of its tiles (books_per_wg > 1 means whole codebooks).  Its first codes
-        // are requested before the table is replaced, to overlap the two latencies.
-        tile_begin = book * tiles_per_cb;
-        tile_end = tile_begin + tiles_per_cb;
-        n_units = (tiles_per_cb + TB - 1) / TB;
-        load_unit(0, cwq[0]);
-        if (n_units > 1) load_unit(1, cwq[1]);
-        cb += (int64_t)entries * VEC;
+        // Next chunk of K for the same tiles, or the next codebook (books_per_wg > 1 means whole
+        // codebooks: all of its tiles).
+        if (++chunk >= n_chunks) {
+            chunk = 0;
+            if (++book >= book_end) break;
+            tile_begin = book * tiles_per_cb;
+            tile_end = tile_begin + tiles_per_cb;
+            n_units = (tiles_per_cb + TB - 1) / TB;
+            cb += (int64_t)entries * VEC;
+        }
+        n_act = min(n_waves, total_slices - chunk * n_waves);
+        active = w < n_act;
+        // The first codes are requested before the table or X are replaced, to overlap the latencies.
+        load_first_units();
         __syncthreads();  // every gather from the old table has been consumed, every slot read
-        {
+        if (n_chunks > 1) stage_x();
+        if (chunk == 0) {
             // (the thread index goes through an empty asm so that nothing derived from it is kept
             // in registers across the tile loop just to be reused here)
             int tid = threadIdx.x;
@@ -512,7 +560,12 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
                 if (i1 < cb_slots) cb_lds[i1] = b;
             }
         }
-        __syncthreads();
+        if (n_chunks > 1) {
+            wait_vmcnt<0>();
+            __syncthreads();  // pieces staged by the other waves, and the new table
+            pick_x();
+        }
+        __syncthreads();  // X picked up before the slots (which the staging area may lie over) are written
     }
 }
 
@@ -522,17 +575,34 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
 constexpr size_t kDecodeLdsLimit = 160 * 1024;
 constexpr size_t kDisjointBudget = 80 * 1024;  // keep two workgroups per CU when staging beside the codebook
 
-// Workgroups per 16-row slab of X and the tiles each of them gets.
-struct BatchedGrid {
-    int n_slabs, per_slab, wgs_per_cb, books_per_wg, tiles_per_cb, tiles_per_wg, per_cu;
+// How the batched kernel is launched on a shape: the split of K, of X and of the tiles, and the
+// layout of the LDS.  `ok` is false when the shape is not for this kernel.
+struct BatchedPlan {
+    bool ok;
+    int n_waves, n_chunks;                        // waves per workgroup = slices per chunk of K
+    int n_slabs, per_slab;                        // grid
+    int wgs_per_cb, books_per_wg, tiles_per_cb;   // workgroups of a slab <-> codebooks
+    int tiles_per_wg;                             // per codebook
+    int per_cu;                                   // workgroups resident per CU, by waves
+    bool repl, full;                              // replicated table; batches of TB tiles (else of one)
+    int red_off, stage_off, stage_over, acc_off;  // LDS
+    size_t smem;
 };
 
-BatchedGrid batched_grid(const ProblemB &p)
+// K a multiple of 256, N and the rows per codebook multiples of 16; the LDS must hold the table,
+// the slots, the staged X and, when K goes in chunks, the carried sums of the workgroup's tiles.
+template <int VEC, typename CodeT>
+BatchedPlan plan_batched(const ProblemB &p)
 {
-    BatchedGrid g;
-    const int n_waves = p.K / kSliceK;
+    typedef DecodeCfg<VEC, CodeT> C;
+    BatchedPlan g = {};
+    if (p.K % kSliceK != 0 || p.N % kTileN != 0 || p.rows_per_cb % kTileN != 0) return g;
+    const int slices = p.K / kSliceK;
+    g.n_chunks = (slices + kMaxWaves - 1) / kMaxWaves;
+    g.n_waves = (slices + g.n_chunks - 1) / g.n_chunks;
+    const int m_slab = p.M < kTileN ? p.M : kTileN;  // rows of X one workgroup multiplies
     g.tiles_per_cb = p.rows_per_cb / kTileN;
-    g.per_cu = kMaxWaves / n_waves;  // workgroups resident per CU, by waves
+    g.per_cu = kMaxWaves / g.n_waves;
     g.n_slabs = (p.M + kTileN - 1) / kTileN;
     // As many workgroups as the device holds at once, shared among the slabs.  Within a slab a
     // workgroup reads one codebook at a time: several workgroups share the tiles of a codebook,
@@ -544,68 +614,92 @@ BatchedGrid batched_grid(const ProblemB &p)
         const int per_cb = per_slab / p.n_codebooks;
         g.wgs_per_cb = per_cb < g.tiles_per_cb ? per_cb : g.tiles_per_cb;
         g.books_per_wg = 1;
-        g.per_slab = g.wgs_per_cb * p.n_codebooks;
     } else {
         g.wgs_per_cb = 1;
         g.books_per_wg = (p.n_codebooks + per_slab - 1) / per_slab;
-        g.per_slab = (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg;
     }
-    g.tiles_per_wg = (g.tiles_per_cb + g.wgs_per_cb - 1) / g.wgs_per_cb;  // per codebook
-    return g;
+    const size_t plain = (size_t)p.entries * VEC * 2;
+    const size_t stage = (size_t)((g.n_waves * kSliceK + kStageK - 1) / kStageK) * m_slab * kStagePitch;
+    const size_t slot_bytes = (size_t)4 * m_slab * kSlotPitch;  // per tile of a batch
+    const size_t carry_bytes = (size_t)4 * m_slab * 16;         // per tile of the workgroup's range
+    for (;;) {
+        g.tiles_per_wg = (g.tiles_per_cb + g.wgs_per_cb - 1) / g.wgs_per_cb;
+        g.full = g.tiles_per_wg >= 2;
+        const int tb = g.full ? C::TB : 1;
+        const size_t slots = tb * slot_bytes;
+        const int units = (g.tiles_per_wg + tb - 1) / tb;
+        const size_t carry = g.n_chunks > 1 ? (size_t)units * tb * carry_bytes : 0;
+        // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time as
+        // soon as the workgroup gathers from it for more than one tile, where it fits.
+        for (int repl = (p.entries <= 256 && g.tiles_per_wg >= VQ_REPL_MIN) ? 1 : 0; repl >= 0; repl--) {
+            const size_t table = repl ? (size_t)p.entries * 256 : plain;
+            g.repl = repl != 0;
+            g.acc_off = g.n_chunks > 1 ? (int)table : -1;
+            g.red_off = (int)(table + carry);
+            if (g.n_chunks == 1 && table + carry + slots + stage <= kDisjointBudget) {
+                // everything side by side, and room for a second workgroup on the CU
+                g.stage_off = g.red_off + (int)slots;
+                g.stage_over = 0;
+                g.smem = table + slots + stage;
+                g.ok = true;
+                return g;
+            }
+            if (g.n_chunks == 1) {
+                // X staged over the table and the slots (both are written after X is picked up)
+                g.stage_off = 0;
+                g.stage_over = kStageOverTable | kStageOverSlots;
+                g.smem = stage > table + slots ? stage : table + slots;
+            } else {
+                // X staged over the slots only: table and carried sums live across the chunks
+                g.stage_off = g.red_off;
+                g.stage_over = kStageOverSlots;
+                g.smem = table + carry + (stage > slots ? stage : slots);
+            }
+            if (g.smem <= kDecodeLdsLimit) {
+                g.ok = true;
+                return g;
+            }
+        }
+        // Too many carried sums: fewer tiles per workgroup (more workgroups than are resident).
+        if (g.n_chunks == 1 || g.wgs_per_cb >= g.tiles_per_cb) return g;
+        if (g.books_per_wg > 1) g.books_per_wg = 1;  // one codebook per workgroup first
+        else g.wgs_per_cb = g.wgs_per_cb * 2 < g.tiles_per_cb ? g.wgs_per_cb * 2 : g.tiles_per_cb;
+    }
+}
+
+BatchedPlan plan_batched(const ProblemB &p)
+{
+    const bool u8 = p.code_bits == 8;
+    switch (p.vec) {
+    case 8: return u8 ? plan_batched<8, uint8_t>(p) : plan_batched<8, uint16_t>(p);
+    case 4: return u8 ? plan_batched<4, uint8_t>(p) : plan_batched<4, uint16_t>(p);
+    default: return u8 ? plan_batched<2, uint8_t>(p) : plan_batched<2, uint16_t>(p);
+    }
 }
 
 template <int VEC, typename CodeT>
 hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
 {
     typedef DecodeCfg<VEC, CodeT> C;
-    const int n_waves = p.K / kSliceK;
-    const int m_slab = p.M < kTileN ? p.M : kTileN;  // rows of X one workgroup multiplies
-    const BatchedGrid g = batched_grid(p);
-    // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time as
-    // soon as the workgroup gathers from it for more than one tile; so is the batched loop, whose
-    // short-unit path serves a workgroup with fewer tiles than a batch.
-    const bool repl = p.entries <= 256 && g.tiles_per_wg >= VQ_REPL_MIN;
-    const bool full = g.tiles_per_wg >= 2;
-    const int tb = full ? C::TB : 1;
-    const size_t table = repl ? (size_t)p.entries * 256 : (size_t)p.entries * VEC * 2;
-    const size_t base = table + (size_t)tb * 4 * m_slab * kSlotPitch;
-    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * m_slab * kStagePitch;
-    size_t smem = base;
-    int stage_off = -1, aliased = 0;
-    // X is staged beside the codebook and the slots when that leaves room for a second workgroup
-    // on the CU, over them otherwise.
-    if (base + stage <= kDisjointBudget) {
-        stage_off = (int)base;
-        smem = base + stage;
-    } else {
-        stage_off = 0;
-        aliased = 1;
-        smem = stage > base ? stage : base;
-    }
-    auto kern = !full  ? decode_batched_kernel<VEC, CodeT, false, 1>
-                : repl ? decode_batched_kernel<VEC, CodeT, true, C::TB>
-                       : decode_batched_kernel<VEC, CodeT, false, C::TB>;
-    if (!full && repl) kern = decode_batched_kernel<VEC, CodeT, true, 1>;  // only where a full batch is one tile
-    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
+    BatchedPlan g = plan_batched<VEC, CodeT>(p);
+    if (!g.ok) return hipErrorInvalidValue;
+    g.per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
+    auto kern = !g.full  ? decode_batched_kernel<VEC, CodeT, false, 1>
+                : g.repl ? decode_batched_kernel<VEC, CodeT, true, C::TB>
+                         : decode_batched_kernel<VEC, CodeT, false, C::TB>;
+    if (!g.full && g.repl) kern = decode_batched_kernel<VEC, CodeT, true, 1>;  // only where a full batch is one tile
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), g.smem);
     if (e != hipSuccess) return e;
     const int tail_rows = p.M - (g.n_slabs - 1) * kTileN;
-    hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(n_waves * 64), smem, s, p.x,
+    hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(g.n_waves * 64), g.smem, s, p.x,
                        static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.n_codebooks,
                        g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, g.tiles_per_cb / g.wgs_per_cb,
-                       g.tiles_per_cb % g.wgs_per_cb, stage_off, aliased, (65536 + tail_rows - 1) / tail_rows);
+                       g.tiles_per_cb % g.wgs_per_cb, g.n_chunks, g.red_off, g.stage_off, g.stage_over, g.acc_off,
+                       (65536 + tail_rows - 1) / tail_rows);
     return hipGetLastError();
 }
 
-// The batched kernel takes K a multiple of 256 up to 4096 and N (and the rows per codebook) a multiple of 16.
-bool batched_supports(const ProblemB &p)
-{
-    // LDS: the plain codebook and the slots of the largest batch, and the staged X (which may lie over them)
-    const int m_slab = p.M < kTileN ? p.M : kTileN;
-    const size_t base = (size_t)p.entries * p.vec * 2 + (size_t)4 * 4 * m_slab * kSlotPitch;
-    const size_t stage = (size_t)((p.K + kStageK - 1) / kStageK) * m_slab * kStagePitch;
-    return p.rows_per_cb % kTileN == 0 && p.K % kSliceK == 0 && p.K <= kSliceK * kMaxWaves && p.N % kTileN == 0 &&
-           base <= kDecodeLdsLimit && stage <= kDecodeLdsLimit;
-}
+bool batched_supports(const ProblemB &p) { return plan_batched(p).ok; }
 
 }  // namespace
 
@@ -616,22 +710,27 @@ bool decode_supports(const ProblemB &p)
 }
 
 // Rough times (us) of the two tiled kernels on a shape both can take; the automatic choice takes
-// the smaller.  The decode path costs a prologue plus ~0.6 us per tile and CU at K = 4096 (in
-// proportion below); the prefill kernel ~1.5 us per 64-deep stage of its 256x256 tiles, one
-// round of tiles per 256 CUs, however few of them there are.
+// the smaller.  Fitted to measurements on a 256-CU MI355X:
+//   decode path   per workgroup a prologue (3), then per codebook and chunk of K its tiles at
+//                 0.75 us per tile and 4096 k (1.25 when K goes in chunks: X is staged again per
+//                 chunk), plus 3.5 per change of codebook or chunk; workgroups beyond those
+//                 resident run in further rounds;
+//   prefill       0.85 + 0.9 * (fraction of the CUs that have a 256x256 tile) us per 64-deep
+//                 stage, one round of tiles per 256 CUs.
 bool decode_preferred(const ProblemB &p)
 {
     if (!decode_supports(p)) return false;
     if (p.M <= kGeneralMaxM) return true;
-    const BatchedGrid g = batched_grid(p);
+    const BatchedPlan g = plan_batched(p);
     const int cus = device_cu_count();
-    // rounds of resident workgroups; per workgroup a prologue, its tiles (at 1/per_cu of the CU's
-    // throughput) and the codebook switches
-    const int rounds_d = (g.per_slab * g.n_slabs + cus * g.per_cu - 1) / (cus * g.per_cu);
-    const double t_decode = rounds_d * (3.0 + g.tiles_per_wg * g.books_per_wg * 0.6 * (p.K / 4096.0) * g.per_cu +
-                                        (g.books_per_wg - 1) * 1.5);
-    const int rounds_p = (((p.M + 255) / 256) * ((p.N + 255) / 256) + cus - 1) / cus;
-    const double t_prefill = 8.0 + rounds_p * (p.K / 64.0) * 1.5;
+    const int per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
+    const int rounds_d = (per_slab * g.n_slabs + cus * g.per_cu - 1) / (cus * g.per_cu);
+    const double t_tile = (g.n_chunks == 1 ? 0.75 : 1.25) * g.n_waves / kMaxWaves * g.per_cu;
+    const int passes = g.books_per_wg * g.n_chunks;
+    const double t_decode = rounds_d * (3.0 + passes * g.tiles_per_wg * t_tile + (passes - 1) * 3.5);
+    const double tiles = (double)((p.M + 255) / 256) * ((p.N + 255) / 256);
+    const double frac = tiles < cus ? tiles / cus : 1.0;
+    const double t_prefill = 8.0 + (tiles < cus ? 1.0 : tiles / cus) * (p.K / 64.0) * (0.85 + 0.9 * frac);
     return t_decode <= t_prefill;
 }
 
