@@ -1,35 +1,42 @@
 // Prefill kernel (large M): Y[M,N] = X[M,K] . W^T with W given as codes + codebook.
 //
-// MFMA-bound.  A 256-thread workgroup (4 waves, 2x2) computes a 256x256 tile of Y with
-// v_mfma_f32_32x32x16_f16; each wave owns 128x128 of it (256 fp32 accumulator registers).
+// MFMA-bound, and on this part MFMA-bound means power-bound: with random fp16 operands the
+// matrix pipes draw enough power to pull the clock far below nominal, and what a tile costs is
+// the energy it spends.  Two things follow.  v_mfma_f32_16x16x32_f16 needs clearly less energy
+// per multiply-add than the 32x32x16 shape (a register-only loop reaches about 1.7 PFLOP/s with
+// it against 1.3 PFLOP/s).  And every byte moved counts: X is walked in whole 128-byte lines.
+//
+// A 256-thread workgroup (4 waves, 2x2) computes a 256x256 tile of Y; each wave owns 128x128 of
+// it as 8x8 pieces of 16x16 (256 fp32 accumulator registers, pinned in the AGPRs).
 //
 //   * W never exists as a tile anywhere: the codebooks of the workgroup's rows sit in the
 //     LDS and every lane gathers the codeword of "its" W row straight into the 8-half MFMA
-//     operand (vec = 8: one ds_read_b128 == one operand).  The order in which K is walked is
-//     free, so it is chosen to make a lane's codes contiguous: one 16-byte global load per
-//     lane feeds CPL/CPO MFMA steps.
-//   * X tiles (256 rows x 64 k) go global -> LDS directly (global_load_lds_dwordx4, no register
-//     staging) through four buffers (three when the codebooks are large), issued three stages
-//     ahead of their use so that an HBM miss is covered by two stages of MFMA work.
-//     The LDS has 64 banks of 4 bytes: two 128-byte tile rows form one 256-byte bank row and
+//     operand (vec = 8: one ds_read_b128 == one operand).
+//   * X tiles (256 rows x 64 k, one cache line per row) and code tiles (256 rows x the codes
+//     of 64 or 128 k) go global -> LDS directly (global_load_lds_dwordx4, no register staging)
+//     through four buffers (fewer when the codebooks are large), issued three stages ahead of
+//     their use so that an HBM miss is covered by two stages of MFMA work.
+//     The LDS has 64 banks of 4 bytes: two 128-byte X rows form one 256-byte bank row and
 //     the sixteen 16-byte chunks of a bank row are XOR-swizzled with the bank-row index, which
-//     makes the operand reads (32 consecutive rows x one chunk per half wave) conflict free.
+//     makes the operand reads (16 consecutive rows x one chunk per quarter wave) conflict free.
 //     A direct load fills 64 consecutive slots per wave, so each lane fetches whatever chunk
 //     the swizzle assigns to its slot.
-//   * The MFMA operands of step s+1 are fetched from the LDS while step s is multiplied, also
-//     across stage boundaries: the barrier that publishes stage i+2 sits a whole stage ahead
-//     of its first read.
+//   * One MFMA step (k = 32) is 64 MFMAs on 8 W pieces and 8 X pieces, walked as four 4x4
+//     quadrants.  The walk alternates between two orders so that every group of four pieces has
+//     its last use at least one quadrant (16 MFMAs, 256 cycles) before the group's successor is
+//     first needed: each quadrant re-loads exactly one group of four operands into the registers
+//     that just went dead, also across stage boundaries (the barrier that publishes stage i+2
+//     sits a whole stage ahead of its first read).  No operand is double buffered.
 //   * fp32 accumulation; one rounding to fp16 in the epilogue, which transposes through the
 //     LDS so that Y is written in 256-byte row segments.
 //
-// K order.  A lane of the 32x32x16 MFMA holds 8 consecutive k of one row; lanes 0-31 hold
-// k-group 0 and lanes 32-63 k-group 1.  A "super stage" is the K range fed by one 16-byte
-// code load per lane: lane group g covers the contiguous range
-// [S*2*K_LANE + g*K_LANE, +K_LANE).  LDS stage t of the super stage holds, for both groups,
-// the 32 k starting at offset t*32 of the group's range: two 64-byte pieces per X row.
-// K must be a multiple of K_LANE; when it is not a multiple of 2*K_LANE the last super stage
-// has no data for group 1 and the TAIL instantiation zeroes that group's W operand.
+// K is walked in order: stage i is k in [64 i, 64 i + 64), MFMA step s of it the 32 k from
+// 32 s on, and lane group g (lanes 16g..16g+15) holds the 8 k from 8 g on.  K must be a
+// multiple of the k that 16 bytes of codes cover; a last stage of 32 k runs in the TAIL
+// instantiation, which points the W operands of the missing step at zeros.
 #include "vq_common.h"
+
+#include <type_traits>
 
 namespace vq {
 
@@ -37,52 +44,28 @@ namespace {
 
 constexpr int BM = 256, BN = 256;     // workgroup tile
 constexpr int WM = 128, WN = 128;     // wave tile
-constexpr int MB = WM / 32, NB = WN / 32;
+constexpr int MP = WM / 16, NP = WN / 16;  // 16-row pieces of X and of W per wave
 constexpr int kThreads = 256;
-constexpr int kStageK = 64;           // k per LDS stage (4 MFMA steps)
+constexpr int kStageK = 64;           // k per LDS stage (2 MFMA steps)
 constexpr int kStageBytes = BM * kStageK * 2;  // 32 KB
-constexpr int kChunksPerThread = (BM * 8) / kThreads;  // 16-byte chunks of a stage per thread
+constexpr int kChunksPerThread = (BM * 8) / kThreads;  // 16-byte chunks of an X stage per thread
 
 template <int VEC, typename CodeT>
 struct PrefillCfg {
-    static constexpr int CPL = 16 / (int)sizeof(CodeT);
-    static constexpr int CPO = 8 / VEC;
-    static constexpr int K_LANE = CPL * VEC;          // k per lane per super stage
-    static constexpr int K_SUPER = 2 * K_LANE;        // k per super stage
-    static constexpr int STAGES = K_LANE / 32;        // LDS stages per super stage
-    static_assert(CPO >= 1 && STAGES >= 1, "unsupported code layout");
+    static constexpr int CSZ = (int)sizeof(CodeT);
+    static constexpr int CPO = 8 / VEC;                 // codes per 8-half operand
+    static constexpr int RB = CPO * CSZ;                // bytes of codes behind one operand (1, 2 or 4)
+    static constexpr int KC = (16 / CSZ) * VEC;         // k covered by 16 bytes of one row's codes
+    static constexpr int K_SUPER = KC > kStageK ? KC : kStageK;  // k per code tile (a "super stage")
+    static constexpr int STAGES = K_SUPER / kStageK;    // LDS stages per super stage (1 or 2)
+    static constexpr int CH = K_SUPER / KC;             // 16-byte chunks per row of a code tile (1 or 2)
+    static constexpr int HALF = 32 / VEC * CSZ;         // bytes of one row's codes per MFMA step
+    static constexpr int kTileBytes = CH * BN * 16;     // code tile in the LDS: [chunk][row][16 bytes]
+    static_assert(RB == 1 || RB == 2 || RB == 4, "unsupported code layout");
+    static_assert(STAGES == 1 || STAGES == 2, "unsupported code layout");
+    // code tiles in flight: the one being read plus those loaded ahead
+    static constexpr int code_bufs(int ns) { return STAGES == 1 ? ns : 3; }
 };
-
-template <typename CodeT>
-__device__ __forceinline__ uint32_t code_of(const uint4_t &cw, int c)
-{
-    if constexpr (sizeof(CodeT) == 1)
-        return (cw[c >> 2] >> (8 * (c & 3))) & 0xffu;
-    else
-        return (cw[c >> 1] >> (16 * (c & 1))) & 0xffffu;
-}
-
-// `book` must point into the LDS (the callers index the __shared__ array directly so that
-// the compiler emits ds_read, not flat loads).
-template <int VEC, typename CodeT>
-__device__ __forceinline__ half8_t gather8(const uint8_t *book, const uint4_t &cw, int c0)
-{
-    if constexpr (VEC == 8) {
-        return *reinterpret_cast<const half8_t *>(book + code_of<CodeT>(cw, c0) * 16u);
-    } else if constexpr (VEC == 4) {
-        const half4_t lo = *reinterpret_cast<const half4_t *>(book + code_of<CodeT>(cw, c0) * 8u);
-        const half4_t hi = *reinterpret_cast<const half4_t *>(book + code_of<CodeT>(cw, c0 + 1) * 8u);
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    } else {
-        static_assert(VEC == 2, "vector length must be 2, 4 or 8");
-        half2_t q[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) q[i] = *reinterpret_cast<const half2_t *>(book + code_of<CodeT>(cw, c0 + i) * 4u);
-        const half4_t lo = __builtin_shufflevector(q[0], q[1], 0, 1, 2, 3);
-        const half4_t hi = __builtin_shufflevector(q[2], q[3], 0, 1, 2, 3);
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-}
 
 // Byte offset inside a stage buffer of logical 16-byte chunk cc (0..7) of X-tile row `row`.
 __device__ __forceinline__ int x_offset(int row, int cc)
@@ -111,21 +94,66 @@ __device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff,
                  : "memory");
 }
 
-// 16-byte global load into registers outside the compiler's vmcnt bookkeeping (so that its own
-// waits never drain the LDS-bound loads in flight).  The result must not be touched before a
-// wait_vmcnt that covers it; pin_loaded() ties that wait to the registers.
-__device__ __forceinline__ uint4_t load_16_untracked(const void *p)
+// acc += a . b with the accumulator pinned to one AGPR tuple.  Left to itself the register
+// allocator renames the 64 four-register accumulators from MFMA to MFMA and pays for it with
+// copies at the loop edge and with spills.  The compiler cannot see into the statement, so the
+// callers keep dependent MFMAs (same accumulator) far apart and pad before the accumulators are
+// read back.
+__device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, const half8_t &b)
 {
-    uint4_t v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
-template <int NB_>
-__device__ __forceinline__ void pin_loaded(uint4_t (&r)[NB_])
+
+// floor(x / d) for 0 <= x and a quotient small enough that float rounding stays within one
+// (here: x < d + 256); `rcp` = 1.0f / d.
+__device__ __forceinline__ int small_div(int x, int d, float rcp)
 {
+    int qt = (int)((float)x * rcp);
+    const int rem = x - qt * d;
+    qt += rem >= d ? 1 : 0;
+    qt -= rem < 0 ? 1 : 0;
+    return qt;
+}
+
+// The RB bytes of codes behind one operand, zero-extended.
+template <int RB>
+__device__ __forceinline__ uint32_t read_codes(const uint8_t *p)
+{
+    if constexpr (RB == 1) return *p;
+    else if constexpr (RB == 2) return *reinterpret_cast<const uint16_t *>(p);
+    else return *reinterpret_cast<const uint32_t *>(p);
+}
+
+// Gathers the 8 halves of one MFMA operand: the codes packed in `cr` select codewords of the
+// codebook at LDS byte offset `book`.  With `zero` set the reads go to the 16 zero bytes at
+// `zero_off` instead (a step past the end of K).
+template <int VEC, typename CodeT, bool TAIL>
+__device__ __forceinline__ half8_t gather8(const uint8_t *lds, uint32_t book, uint32_t cr, bool zero, uint32_t zero_off)
+{
+    constexpr int CPO = 8 / VEC, BITS = 8 * (int)sizeof(CodeT);
+    auto at = [&](int c) {
+        const uint32_t code = CPO == 1 ? cr : (cr >> (BITS * c)) & ((1u << BITS) - 1u);
+        uint32_t a = book + code * (uint32_t)(VEC * 2);
+        if (TAIL) a = zero ? zero_off : a;
+        return lds + a;
+    };
+    if constexpr (VEC == 8) {
+        return *reinterpret_cast<const half8_t *>(at(0));
+    } else if constexpr (VEC == 4) {
+        const half4_t lo = *reinterpret_cast<const half4_t *>(at(0));
+        const half4_t hi = *reinterpret_cast<const half4_t *>(at(1));
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    } else {
+        static_assert(VEC == 2, "vector length must be 2, 4 or 8");
+        half2_t q[4];
 #pragma unroll
-    for (int i = 0; i < NB_; i++) asm volatile("" : "+v"(r[i]));
+        for (int i = 0; i < 4; i++) q[i] = *reinterpret_cast<const half2_t *>(at(i));
+        const half4_t lo = __builtin_shufflevector(q[0], q[1], 0, 1, 2, 3);
+        const half4_t hi = __builtin_shufflevector(q[2], q[3], 0, 1, 2, 3);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
 }
+
 
 template <int VEC, typename CodeT, bool TAIL, int NS>
 __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__restrict__ x,
@@ -136,18 +164,20 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                                                               int tiles_n, int cb_lds_count)
 {
     typedef PrefillCfg<VEC, CodeT> C;
-    static_assert(NS == 3 || NS == 4, "three or four X stages");
-    constexpr int D = NS - 1;                 // X loads run D stages ahead of the MFMAs
-    constexpr int kInFlight = (D - 2) * kChunksPerThread;  // loads allowed to stay in flight at a stage end
+    static_assert(NS >= 2 && NS <= 4, "two to four X stages");
+    constexpr int D = NS - 1;                 // loads run D stages ahead of the MFMAs
+    constexpr int NC = C::code_bufs(NS);
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr int kCbBase = NS * kStageBytes;
-
+    constexpr int kCodeBase = NS * kStageBytes;
+    constexpr int kCbBase = kCodeBase + NC * C::kTileBytes;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int wm = wave >> 1, wn = wave & 1;
-    const int l32 = lane & 31, kg = lane >> 5;
+    const int r16 = lane & 15, kg = lane >> 4;
     const int J = K / VEC;
     const int cb_bytes = entries * VEC * 2;
+    // 16 zero bytes behind the codebooks, whose region is padded to whole 1 KB copy steps
+    const uint32_t zero_off = kCbBase + ((cb_lds_count * cb_bytes + 1023) & ~1023);
 
     // Tile mapping.  Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.
     // Re-number them so that an XCD works on consecutive tiles of the (row band major) tile
@@ -157,37 +187,30 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
     const int tm = wg / tiles_n, tn = wg % tiles_n;
     const int m0 = tm * BM, n0 = tn * BN;
-    const int n_super = (K + C::K_SUPER - 1) / C::K_SUPER;
-    const int n_stage = n_super * C::STAGES;
+    const int n_stage = (K + kStageK - 1) / kStageK;
+    const int n_super = (n_stage + C::STAGES - 1) / C::STAGES;
 
-    // ---- per-lane W rows, codebook bases and code streams ---------------------------------
+    // ---- per-lane codebook bases ------------------------------------------------------------
     const int g_first = n0 / rows_per_cb;
-    uint32_t book[NB];  // byte offset of the lane's codebook inside smem
-    const CodeT *code_row[NB];
+    uint32_t book[NP];  // byte offset inside smem of the codebook of W row j*16 + r16 of the wave tile
+    {
+        const int n_base = min(n0 + wn * WN, N - 1);
+        const int g_base = n_base / rows_per_cb, rem_base = n_base - g_base * rows_per_cb;
+        const float rcp = 1.0f / (float)rows_per_cb;
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        const int n = min(n0 + wn * WN + nb * 32 + l32, N - 1);
-        book[nb] = kCbBase + (n / rows_per_cb - g_first) * cb_bytes;
-        code_row[nb] = codes + (int64_t)n * J;
-    }
-    auto issue_codes = [&](int super, uint4_t (&dst)[NB]) {
-        super = min(super, n_super - 1);  // past the end: harmless re-reads instead of branches
-        int k = super * C::K_SUPER + kg * C::K_LANE;
-        if (TAIL && k >= K) k = 0;  // k-group 1 of a partial last super stage: any valid codes (operand is zeroed)
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            // The codeword sizes below 16 bytes run out of registers; a register spilled while a
-            // hand-issued load is still writing it would save stale data, so these variants
-            // leave their code loads to the compiler's own (more conservative) waits.
-            if constexpr (VEC == 8) dst[nb] = load_16_untracked(code_row[nb] + k / VEC);
-            else dst[nb] = ld_global_16(code_row[nb] + k / VEC);
+        for (int j = 0; j < NP; j++) {
+            const int n = min(n0 + wn * WN + j * 16 + r16, N - 1);
+            const int g = g_base + small_div(n - n_base + rem_base, rows_per_cb, rcp);
+            book[j] = kCbBase + (g - g_first) * cb_bytes;
         }
-    };
+    }
 
-    // ---- X staging: global -> LDS directly ------------------------------------------------
-    // Load i of wave w fills the 64 consecutive 16-byte slots [(4i+w)*64, +64) of a stage buffer;
-    // the lane looks up which (row, chunk) lives in its slot under the swizzle and reads that.
+    // ---- staging: global -> LDS directly ----------------------------------------------------
+    // X load i of wave w fills the 64 consecutive 16-byte slots [(4i+w)*64, +64) of a stage
+    // buffer; the lane looks up which (row, chunk) lives in its slot under the swizzle and reads
+    // that.  Chunk cc of a row is the 8 k from 8 cc on.
     uint32_t x_voff[kChunksPerThread];
+    uint32_t x_voff_tail[TAIL ? kChunksPerThread : 1];  // last stage of 32 k: chunks 4..7 re-read chunks 0..3
 #pragma unroll
     for (int i = 0; i < kChunksPerThread; i++) {
         const int slot = (4 * i + wave) * 64 + lane;
@@ -195,144 +218,219 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         const int v = (slot & 15) ^ (bank_row & 15);
         const int row = 2 * bank_row + (v >> 3), cc = v & 7;
         const int gm = min(m0 + row, M - 1) - m0;
-        const int koff = (cc >> 2) * C::K_LANE + (cc & 3) * 8;
-        x_voff[i] = (uint32_t)(((int64_t)gm * K + koff) * 2);
+        x_voff[i] = (uint32_t)(((int64_t)gm * K + cc * 8) * 2);
+        if (TAIL) x_voff_tail[i] = x_voff[i] - (cc >= 4 ? 64u : 0u);
     }
     const half_t *x_tile = x + (int64_t)m0 * K;
-    // Load i (0..7) of a stage: one 16-byte chunk per lane, 1 KB per wave.
-    auto issue_x_one = [&](int stage, int buf, int i) {
-        stage = min(stage, n_stage - 1);  // past the end: harmless re-reads instead of branches
-        const int super = stage / C::STAGES;
-        const half_t *sbase = x_tile + super * C::K_SUPER + (stage % C::STAGES) * 32;
+    // X load i (0..7) of stage `stage` into buffer `buf`: one 16-byte chunk per lane, 1 KB per
+    // wave.  Past the end the last stage is read again (harmless) instead of branching.
+    auto issue_x = [&](int i, int buf, int stage) {
+        const bool is_last = stage >= n_stage - 1;
+        const half_t *sbase = x_tile + min(stage, n_stage - 1) * kStageK;
         uint32_t voff = x_voff[i];
-        if (TAIL && super == n_super - 1) {
-            // k-group 1 of the partial last super stage lies past K: read k-group 0's bytes again
-            // (that group's W operand is zeroed).
-            const int slot = (4 * i + wave) * 64 + lane;
-            const int hi = (((slot & 15) ^ ((slot >> 4) & 15)) >> 2) & 1;
-            voff -= hi ? C::K_LANE * 2 : 0;
-        }
+        if (TAIL) voff = is_last ? x_voff_tail[i] : voff;
         load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, voff, sbase);
     };
+    // Code tile of a super stage: chunk c of tile row w*64 + lane goes to [c][row]; 1 KB per wave.
+    const CodeT *code_tile = codes + (int64_t)n0 * J;
+    const uint32_t code_voff = (uint32_t)(min(wave * 64 + lane, N - 1 - n0) * J * C::CSZ);
+    auto issue_codes = [&](int c, int cbuf, int super) {
+        const bool is_last = super >= n_super - 1;
+        super = min(super, n_super - 1);
+        // a last stage of 32 k has only chunk 0; read it twice
+        const int chunk = (TAIL && is_last) ? 0 : c;
+        const uint8_t *sbase = reinterpret_cast<const uint8_t *>(code_tile) + (int64_t)super * (C::K_SUPER / VEC * C::CSZ) + chunk * 16;
+        load_to_lds_16(kCodeBase + cbuf * C::kTileBytes + c * (BN * 16) + wave * 1024, code_voff, sbase);
+    };
 
-    float16_t acc[NB][MB];
+    float4_t acc[NP][MP];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++)
+    for (int j = 0; j < NP; j++)
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[nb][mb][r] = 0.f;
+        for (int i = 0; i < MP; i++) acc[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Operand read offsets inside a stage buffer: row = wm*128 + mb*32 + l32, chunk = kg*4 + s.
-    int x_rd[MB][4];
+    // Operand read offsets inside a stage buffer: X piece i is rows wm*128 + i*16 + r16; the
+    // lane's chunk in MFMA step s is s*4 + kg.  Two pieces further is 16 bank rows (4 KB) on and
+    // leaves the swizzle unchanged.
+    int x_rd[2][2];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int par = 0; par < 2; par++)
 #pragma unroll
-        for (int s = 0; s < 4; s++) x_rd[mb][s] = x_offset(wm * WM + mb * 32 + l32, kg * 4 + s);
+        for (int s = 0; s < 2; s++) x_rd[par][s] = x_offset(wm * WM + par * 16 + r16, s * 4 + kg);
+    // Where the lane's codes of W piece 0 start inside a code tile.
+    const uint32_t code_rd = kCodeBase + (wn * WN + r16) * 16 + kg * C::RB;
 
-    half8_t wop[2][NB], xop[2][MB];
-    auto fetch_operands = [&](int set, int buf, const uint4_t (&c)[NB], int t, int s, bool last_super) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            half8_t w = gather8<VEC, CodeT>(smem + book[nb], c[nb], (t * 4 + s) * C::CPO);
-            if (TAIL && last_super && kg == 1) w = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            wop[set][nb] = w;
-        }
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-            xop[set][mb] = *reinterpret_cast<const half8_t *>(smem + buf * kStageBytes + x_rd[mb][s]);
+    half8_t wp[NP], xp[MP];
+    uint32_t cr[2][4];  // codes behind the two W groups whose gathers come next
+    // X piece i of MFMA step s out of stage buffer `buf`
+    auto load_x1 = [&](int i, int buf, int s) {
+        xp[i] = *reinterpret_cast<const half8_t *>(smem + buf * kStageBytes + x_rd[i & 1][s] + (i >> 1) * 4096);
+    };
+    // the codes of W piece j for MFMA step s of stage t (of its super stage) out of code buffer `cbuf`
+    auto load_c1 = [&](int set, int j, int cbuf, int t, int s) {
+        const int pos = (t % C::STAGES) * 2 * C::HALF + s * C::HALF;   // + kg*RB stays inside the 16-byte chunk
+        cr[set][j & 3] = read_codes<C::RB>(smem + code_rd + cbuf * C::kTileBytes + (pos / 16) * (BN * 16) + j * 256 + pos % 16);
+    };
+    // W piece j from the codes read before
+    auto load_w1 = [&](int set, int j, bool zero) {
+        wp[j] = gather8<VEC, CodeT, TAIL>(smem, book[j], cr[set][j & 3], zero, zero_off);
+    };
+    // MFMA f of group p of the 4x4 quadrant (jh, ih): a group is W piece p against the four X
+    // pieces, or (x_outer) X piece p against the four W pieces
+    auto mfma_one = [&](int jh, int ih, int p, int f, bool x_outer) {
+        const int j = jh * 4 + (x_outer ? f : p), i = ih * 4 + (x_outer ? p : f);
+        mfma_in_place(acc[j][i], wp[j], xp[i]);
     };
 
     // ---- prologue --------------------------------------------------------------------------
-    uint4_t cw[NB], cw1[NB], cw2[NB];  // codes of super stage S, S+1, S+2
-    issue_codes(0, cw);
-    issue_codes(1, cw1);
-    issue_codes(2, cw2);
-#pragma unroll
-    for (int d = 0; d < D; d++)
-#pragma unroll
-        for (int i = 0; i < kChunksPerThread; i++) issue_x_one(d, d, i);
+    // Loads complete in the order they were issued, so one count serves all of them: the
+    // codebooks first, then X stages 0..D-1 with the code tiles of the super stages that open
+    // there, then what the two quadrants ahead of stage 0 would have issued for stage D.
+    // loads a stage brings along: 8 of X, plus its code tile when it opens a super stage
+    auto loads_of = [](int stage_mod) constexpr { return kChunksPerThread + (stage_mod % C::STAGES == 0 ? C::CH : 0); };
     {
-        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)g_first * entries * VEC);
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(cb + (int64_t)g_first * entries * VEC);
         const int n16 = cb_lds_count * cb_bytes / 16;
         const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
-        for (int i = tid; i < n16; i += kThreads)
-            if (i < g_total_16) reinterpret_cast<uint4_t *>(smem + kCbBase)[i] = src[i];
+        // past the last codebook: read its last 16 bytes again
+        for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
+            load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
     }
-    wait_vmcnt<0>();
-    pin_loaded(cw);
-    pin_loaded(cw1);
-    pin_loaded(cw2);
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        if (d % C::STAGES == 0) {
+#pragma unroll
+            for (int c = 0; c < C::CH; c++) issue_codes(c, (d / C::STAGES) % NC, d / C::STAGES);
+        }
+#pragma unroll
+        for (int i = 0; i < kChunksPerThread; i++) issue_x(i, d, d);
+    }
+    if (D % C::STAGES == 0) {
+#pragma unroll
+        for (int c = 0; c < C::CH; c++) issue_codes(c, (D / C::STAGES) % NC, D / C::STAGES);
+    }
+    issue_x(0, D, D);
+    issue_x(1, D, D);
+    if (tid < 4) reinterpret_cast<uint32_t *>(smem + zero_off)[tid] = 0u;
+    {
+        // stage 0 (and everything older) must have landed; stages 1..D may be in flight
+        constexpr int in_flight = [&]() constexpr {
+            int n = 2 + (D % C::STAGES == 0 ? C::CH : 0);
+            for (int d = 1; d < D; d++) n += loads_of(d);
+            return n;
+        }();
+        wait_vmcnt<in_flight>();
+    }
     __syncthreads();
 
-    int buf = 0;  // buffer of the current stage; stage+j lives in (buf + j) % NS
-    fetch_operands(0, buf, cw, 0, 0, n_super == 1);
+    int buf = 0;   // X buffer of the current stage; stage+j lives in (buf + j) % NS
+    int cbuf = 0;  // code buffer of the current super stage; super+j lives in (cbuf + j) % NC
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        load_c1(0, p, cbuf, 0, 0);
+        load_c1(1, 4 + p, cbuf, 0, 0);
+    }
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        load_w1(0, p, false);
+        load_x1(p, buf, 0);
+    }
+
+    // One quadrant: four groups of four MFMAs.  A wave issues one instruction every four cycles
+    // and a 16x16x32 MFMA holds the matrix pipe for sixteen, so at most three other instructions
+    // fit between two MFMAs without starving the pipe: every MFMA is fenced and the other work
+    // is dealt out by hand.  In the middle of group p, LOADP(p) re-fills one operand register
+    // that went dead in the quadrant before and CODEP(p) reads the codes of a W piece that the
+    // next quadrant gathers; the operand loaded during the previous quadrant is walked in the
+    // outer position, so that every piece has 15 MFMAs between its load and its first use.  One
+    // of the stage's eight X loads follows group 0, a code tile load group 2.
+#define VQ_FENCE __builtin_amdgcn_sched_barrier(0)
+#define VQ_NONE(p) do {} while (0)
+#define VQ_QUADRANT(LOADP, CODEP, jh, ih, x_outer, xi, TGT)                         \
+    _Pragma("unroll") for (int p_ = 0; p_ < 4; p_++) {                              \
+        mfma_one(jh, ih, p_, 0, x_outer); VQ_FENCE;                                 \
+        mfma_one(jh, ih, p_, 1, x_outer); VQ_FENCE;                                 \
+        LOADP(p_); CODEP(p_); VQ_FENCE;                                             \
+        mfma_one(jh, ih, p_, 2, x_outer); VQ_FENCE;                                 \
+        mfma_one(jh, ih, p_, 3, x_outer); VQ_FENCE;                                 \
+        if (p_ == 0) { issue_x(xi, TGT##_buf, TGT##_stage); VQ_FENCE; }             \
+        if (p_ == 2 && TGT##_codes && xi < C::CH) { issue_codes(xi, TGT##_cbuf, TGT##_super); VQ_FENCE; } \
+    }
 
     for (int super = 0; super < n_super; super++) {
-        const bool last_super = super == n_super - 1;
-        const bool next_last = super + 1 == n_super - 1;
-#pragma unroll
-        for (int t = 0; t < C::STAGES; t++) {
+        // stage t (a compile-time 0 or 1) of the super stage
+        auto stage_body = [&](auto t_const) {
+            constexpr int t = decltype(t_const)::value;
             const int stage = super * C::STAGES + t;
             const int buf_next = buf + 1 == NS ? 0 : buf + 1;
-            // Stage+D goes into the buffer that was read during stage-1 (every wave has passed the
-            // barrier that ended it); its eight loads are spread over the four steps.
-            const int buf_load = buf == 0 ? NS - 1 : buf - 1;
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                const int cur = s & 1;
-                // Fetch the operands of the next step and multiply this step's.  A wave issues in
-                // order and an MFMA holds the matrix pipe for 32 cycles, so the LDS reads and their
-                // address arithmetic are dealt out between the MFMAs instead of ahead of them.
-                if (s < 3)
-                    fetch_operands(cur ^ 1, buf, cw, t, s + 1, last_super);
-                else if (t + 1 < C::STAGES)
-                    fetch_operands(cur ^ 1, buf_next, cw, t + 1, 0, last_super);
-                else
-                    fetch_operands(cur ^ 1, buf_next, cw1, 0, 0, next_last);
-                auto mfma = [&](int j) {
-                    const int nb = j / MB, mb = j % MB;
-                    acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wop[cur][nb], xop[cur][mb], acc[nb][mb], 0, 0, 0);
-                };
-#pragma unroll
-                for (int j = 0; j < 8; j++) mfma(j);
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // a few VALU (gather addresses)
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                issue_x_one(stage + D, buf_load, 2 * s);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 8; j < 12; j++) mfma(j);
-                __builtin_amdgcn_sched_barrier(0);
-                issue_x_one(stage + D, buf_load, 2 * s + 1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 12; j < 16; j++) mfma(j);
-                __builtin_amdgcn_sched_barrier(0);
+            // The barrier of a stage sits behind its last read of X (quadrant 6 of 8).  From there
+            // on the stage's buffer is free and the two quadrants left issue the first two of the
+            // eight X loads of stage+1+D into it (and that stage's code tile, when it opens a super
+            // stage); the first six quadrants issue loads 2..7 of stage+D into the buffer of
+            // stage-1.  A stage's loads so have two whole stages to land before the barrier that
+            // publishes them.
+            const int tgt_a_buf = buf == 0 ? NS - 1 : buf - 1, tgt_a_stage = stage + D;
+            constexpr bool tgt_a_codes = false;
+            const int tgt_a_cbuf = 0, tgt_a_super = 0;
+            const int tgt_b_buf = buf, tgt_b_stage = stage + 1 + D;
+            constexpr bool tgt_b_codes = (t + 1 + D) % C::STAGES == 0;
+            constexpr int d_super = (t + 1 + D) / C::STAGES;
+            const int tgt_b_super = super + d_super;
+            const int tgt_b_cbuf = (cbuf + d_super) % NC;
+            // the stage after this one: same super stage or the next
+            constexpr bool same_super = t + 1 < C::STAGES;
+            const int cbuf_n = same_super ? cbuf : (cbuf + 1 == NC ? 0 : cbuf + 1);
+            constexpr int t_n = same_super ? t + 1 : 0;
+            // a last stage of 32 k has no step 1
+            const bool no_b = TAIL && stage == n_stage - 1;
+            VQ_FENCE;
+            // step A (s = 0): W low/X low are in registers, the codes of W high in cr[1]
+#define L_WHI_A(p) load_w1(1, 4 + (p), false)
+#define L_XHI_A(p) load_x1(4 + (p), buf, 0)
+#define L_XLO_B(p) load_x1((p), buf, 1)
+#define L_WHI_B(p) load_w1(0, 4 + (p), no_b)
+#define L_WLO_B(p) load_w1(1, (p), no_b)
+#define L_XHI_B(p) load_x1(4 + (p), buf, 1)
+#define L_XLO_N(p) load_x1((p), buf_next, 0)
+#define L_WLO_N(p) load_w1(0, (p), false)
+#define C_WHI_B(p) load_c1(0, 4 + (p), cbuf, t, 1)
+#define C_WLO_B(p) load_c1(1, (p), cbuf, t, 1)
+#define C_WLO_N(p) load_c1(0, (p), cbuf_n, t_n, 0)
+#define C_WHI_N(p) load_c1(1, 4 + (p), cbuf_n, t_n, 0)
+            VQ_QUADRANT(L_WHI_A, VQ_NONE, 0, 0, false, 2, tgt_a);   // W low (just loaded) x X low
+            VQ_QUADRANT(L_XHI_A, VQ_NONE, 1, 0, false, 3, tgt_a);   // W high (just loaded) x X low
+            VQ_QUADRANT(L_XLO_B, C_WHI_B, 1, 1, true, 4, tgt_a);    // W high x X high (just loaded)
+            VQ_QUADRANT(L_WHI_B, C_WLO_B, 0, 1, false, 5, tgt_a);   // W low x X high
+            // step B (s = 1)
+            VQ_QUADRANT(L_WLO_B, VQ_NONE, 1, 0, false, 6, tgt_a);   // W high (just loaded) x X low
+            VQ_QUADRANT(L_XHI_B, VQ_NONE, 0, 0, false, 7, tgt_a);   // W low (just loaded) x X low
+            {
+                // Publish stage+1: in flight may be what stages +2..+D bring along.
+                constexpr int in_flight = [&]() constexpr {
+                    int n = 0;
+                    for (int d = 2; d <= D; d++) n += loads_of(t + d);
+                    return n;
+                }();
+                wait_vmcnt<in_flight>();
             }
-            // Publish stage+2: its loads (issued D-2 stages ago) must have landed in every wave.
-            wait_vmcnt<kInFlight>();
-            pin_loaded(cw2);
             __syncthreads();
+            VQ_QUADRANT(L_XLO_N, C_WLO_N, 0, 1, true, 0, tgt_b);    // W low x X high (just loaded)
+            VQ_QUADRANT(L_WLO_N, C_WHI_N, 1, 1, false, 1, tgt_b);   // W high x X high
             buf = buf_next;
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            cw[nb] = cw1[nb];
-            cw1[nb] = cw2[nb];
-        }
-        issue_codes(super + 3, cw2);
+        };
+        stage_body(std::integral_constant<int, 0>{});
+        if constexpr (C::STAGES == 2) stage_body(std::integral_constant<int, 1>{});
+        cbuf = cbuf + 1 == NC ? 0 : cbuf + 1;
     }
+#undef VQ_QUADRANT
+#undef VQ_FENCE
     // Drain the clamped loads still in flight before the stage buffers are reused.
     wait_vmcnt<0>();
-    pin_loaded(cw2);
     __syncthreads();
+    // the last MFMAs must have left the pipe before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
-    // ---- epilogue: D[i][j], i = W row = 8*(r/4) + 4*kg + r%4, j = X row = l32 --------------
+    // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its wave tile ------
     if ((N & 7) == 0) {
         // Through the LDS: each wave transposes its 128x128 fp16 block, 64 rows at a time, in a
         // private region (row pitch 272 bytes) and stores 256-byte row segments.
@@ -341,20 +439,17 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
 #pragma unroll
         for (int h = 0; h < 2; h++) {
 #pragma unroll
-            for (int mbh = 0; mbh < 2; mbh++) {
-                const int mb = 2 * h + mbh;
+            for (int ii = 0; ii < 4; ii++) {
+                const int i = 4 * h + ii;
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        half4_t hv = {(half_t)acc[nb][mb][4 * q], (half_t)acc[nb][mb][4 * q + 1],
-                                      (half_t)acc[nb][mb][4 * q + 2], (half_t)acc[nb][mb][4 * q + 3]};
-                        *reinterpret_cast<half4_t *>(stage_out + (mbh * 32 + l32) * kPitch + (nb * 32 + 8 * q + 4 * kg) * 2) = hv;
-                    }
+                for (int j = 0; j < NP; j++) {
+                    half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
+                    *reinterpret_cast<half4_t *>(stage_out + (ii * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) = hv;
+                }
             }
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int row = i * 4 + (lane >> 4), c = lane & 15;
+            for (int it = 0; it < 16; it++) {
+                const int row = it * 4 + (lane >> 4), c = lane & 15;
                 const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
                 const int m = m0 + wm * WM + h * 64 + row;
                 const int n = n0 + wn * WN + c * 8;
@@ -363,24 +458,20 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         }
     } else {
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++) {
-            const int m = m0 + wm * WM + mb * 32 + l32;
+        for (int i = 0; i < MP; i++) {
+            const int m = m0 + wm * WM + i * 16 + r16;
             if (m >= M) continue;
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
+            for (int j = 0; j < NP; j++) {
+                const int n = n0 + wn * WN + j * 16 + 4 * kg;
+                half_t *dst = y + (int64_t)m * N + n;
+                if ((N & 3) == 0 && n + 3 < N) {
+                    half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
+                    *reinterpret_cast<half4_t *>(dst) = hv;
+                } else {
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const int n = n0 + wn * WN + nb * 32 + 8 * q + 4 * kg;
-                    half_t *dst = y + (int64_t)m * N + n;
-                    if ((N & 3) == 0 && n + 3 < N) {
-                        half4_t h = {(half_t)acc[nb][mb][4 * q], (half_t)acc[nb][mb][4 * q + 1],
-                                     (half_t)acc[nb][mb][4 * q + 2], (half_t)acc[nb][mb][4 * q + 3]};
-                        *reinterpret_cast<half4_t *>(dst) = h;
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            if (n + r < N) dst[r] = (half_t)acc[nb][mb][4 * q + r];
-                    }
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < N) dst[e] = (half_t)acc[j][i][e];
                 }
             }
         }
@@ -400,25 +491,28 @@ int codebooks_per_tile(const ProblemB &p)
     return n < p.n_codebooks ? n : p.n_codebooks;
 }
 
+template <int VEC, typename CodeT>
 size_t lds_bytes(const ProblemB &p, int n_stages)
 {
-    return (size_t)n_stages * kStageBytes + (size_t)codebooks_per_tile(p) * p.entries * p.vec * 2;
+    typedef PrefillCfg<VEC, CodeT> C;
+    // X stages, code tiles, codebooks (padded to the 1 KB steps they are copied in), 16 zero bytes
+    const size_t books = ((size_t)codebooks_per_tile(p) * p.entries * p.vec * 2 + 1023) & ~(size_t)1023;
+    return (size_t)n_stages * kStageBytes + (size_t)C::code_bufs(n_stages) * C::kTileBytes + books + 16;
 }
-
-// Four X stages when the codebooks leave room for them, else three.
-int pick_stages(const ProblemB &p) { return lds_bytes(p, 4) <= kLdsLimit ? 4 : 3; }
 
 template <int VEC, typename CodeT>
 hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s)
 {
-    typedef PrefillCfg<VEC, CodeT> C;
     const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
     const int n_cb = codebooks_per_tile(p);
-    const int ns = pick_stages(p);
-    const size_t smem = lds_bytes(p, ns);
-    const bool tail = (p.K % C::K_SUPER) != 0;
-    auto kern = ns == 4 ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
-                        : (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>);
+    // Four X stages when the codebooks leave room for them, else three; two (every stage then
+    // waits for its own loads) only so that very large codebooks still run.
+    const int ns = lds_bytes<VEC, CodeT>(p, 4) <= kLdsLimit ? 4 : lds_bytes<VEC, CodeT>(p, 3) <= kLdsLimit ? 3 : 2;
+    const size_t smem = lds_bytes<VEC, CodeT>(p, ns);
+    const bool tail = (p.K % kStageK) != 0;
+    auto kern = ns == 4   ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
+                : ns == 3 ? (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>)
+                          : (tail ? prefill_kernel<VEC, CodeT, true, 2> : prefill_kernel<VEC, CodeT, false, 2>);
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
@@ -430,7 +524,10 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s)
 template <int VEC, typename CodeT>
 bool prefill_cfg_supports(const ProblemB &p)
 {
-    return p.K % PrefillCfg<VEC, CodeT>::K_LANE == 0;
+    // whole 16-byte code chunks per row, a tile's code offsets within 32 bits
+    return p.K % PrefillCfg<VEC, CodeT>::KC == 0 && lds_bytes<VEC, CodeT>(p, 2) <= kLdsLimit &&
+           (int64_t)BN * (p.K / VEC) * (int64_t)sizeof(CodeT) < ((int64_t)1 << 31) &&
+           (int64_t)BM * p.K * 2 < ((int64_t)1 << 32);
 }
 
 }  // namespace
@@ -440,7 +537,6 @@ bool prefill_supports(const ProblemB &p)
     if (p.M < 1 || p.N < 1 || p.K < 1) return false;
     if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
     if (((size_t)p.entries * p.vec * 2) % 16 != 0) return false;
-    if (lds_bytes(p, 3) > kLdsLimit) return false;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
     case 8: return u8 ? prefill_cfg_supports<8, uint8_t>(p) : prefill_cfg_supports<8, uint16_t>(p);
