@@ -11,11 +11,11 @@
 //
 //   * W never exists as a tile anywhere: the codebooks of the workgroup's rows sit in the
 //     LDS and every lane gathers the codeword of "its" W row straight into the 8-half MFMA
-//     operand (vec = 8: one ds_read_b128 == one operand).
+//     operand, in two 8-byte halves.
 //   * X tiles (256 rows x 64 k, one cache line per row) and code tiles (256 rows x the codes
 //     of 64 or 128 k) go global -> LDS directly (global_load_lds_dwordx4, no register staging)
-//     through four buffers (fewer when the codebooks are large), issued three stages ahead of
-//     their use so that an HBM miss is covered by two stages of MFMA work.
+//     through four buffers (fewer when the codebooks are large), issued so far ahead that a
+//     stage's loads have two whole stages of MFMA work to land.
 //     The LDS has 64 banks of 4 bytes: two 128-byte X rows form one 256-byte bank row and
 //     the sixteen 16-byte chunks of a bank row are XOR-swizzled with the bank-row index, which
 //     makes the operand reads (16 consecutive rows x one chunk per quarter wave) conflict free.
@@ -25,8 +25,7 @@
 //     quadrants.  The walk alternates between two orders so that every group of four pieces has
 //     its last use at least one quadrant (16 MFMAs, 256 cycles) before the group's successor is
 //     first needed: each quadrant re-loads exactly one group of four operands into the registers
-//     that just went dead, also across stage boundaries (the barrier that publishes stage i+2
-//     sits a whole stage ahead of its first read).  No operand is double buffered.
+//     that just went dead, also across stage boundaries.  No operand is double buffered.
 //   * fp32 accumulation; one rounding to fp16 in the epilogue, which transposes through the
 //     LDS so that Y is written in 256-byte row segments.
 //
@@ -124,36 +123,32 @@ __device__ __forceinline__ uint32_t read_codes(const uint8_t *p)
     else return *reinterpret_cast<const uint32_t *>(p);
 }
 
-// Gathers the 8 halves of one MFMA operand: the codes packed in `cr` select codewords of the
-// codebook at LDS byte offset `book`.  With `zero` set the reads go to the 16 zero bytes at
-// `zero_off` instead (a step past the end of K).
+// Gathers half `h` (4 halves) of one MFMA operand: the codes packed in `cr` select codewords of
+// the codebook at LDS byte offset `book`.  With `zero` set the reads go to the 16 zero bytes at
+// `zero_off` instead (a step past the end of K).  An operand is fetched in two halves because a
+// 16-byte gather with its bank conflicts holds the wave's issue longer than the gap between two
+// MFMAs.
 template <int VEC, typename CodeT, bool TAIL>
-__device__ __forceinline__ half8_t gather8(const uint8_t *lds, uint32_t book, uint32_t cr, bool zero, uint32_t zero_off)
+__device__ __forceinline__ half4_t gather4(const uint8_t *lds, uint32_t book, uint32_t cr, int h, bool zero, uint32_t zero_off)
 {
     constexpr int CPO = 8 / VEC, BITS = 8 * (int)sizeof(CodeT);
-    auto at = [&](int c) {
+    auto at = [&](int c, int byte_off) {
         const uint32_t code = CPO == 1 ? cr : (cr >> (BITS * c)) & ((1u << BITS) - 1u);
         uint32_t a = book + code * (uint32_t)(VEC * 2);
         if (TAIL) a = zero ? zero_off : a;
-        return lds + a;
+        return lds + a + byte_off;
     };
     if constexpr (VEC == 8) {
-        return *reinterpret_cast<const half8_t *>(at(0));
+        return *reinterpret_cast<const half4_t *>(at(0, 8 * h));
     } else if constexpr (VEC == 4) {
-        const half4_t lo = *reinterpret_cast<const half4_t *>(at(0));
-        const half4_t hi = *reinterpret_cast<const half4_t *>(at(1));
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return *reinterpret_cast<const half4_t *>(at(h, 0));
     } else {
         static_assert(VEC == 2, "vector length must be 2, 4 or 8");
-        half2_t q[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) q[i] = *reinterpret_cast<const half2_t *>(at(i));
-        const half4_t lo = __builtin_shufflevector(q[0], q[1], 0, 1, 2, 3);
-        const half4_t hi = __builtin_shufflevector(q[2], q[3], 0, 1, 2, 3);
-        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const half2_t q0 = *reinterpret_cast<const half2_t *>(at(2 * h, 0));
+        const half2_t q1 = *reinterpret_cast<const half2_t *>(at(2 * h + 1, 0));
+        return __builtin_shufflevector(q0, q1, 0, 1, 2, 3);
     }
 }
-
 
 template <int VEC, typename CodeT, bool TAIL, int NS>
 __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__restrict__ x,
@@ -173,6 +168,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int wm = wave >> 1, wn = wave & 1;
+    const bool mirrored = wm == 1;  // which of the two walks through a stage the wave takes
     const int r16 = lane & 15, kg = lane >> 4;
     const int J = K / VEC;
     const int cb_bytes = entries * VEC * 2;
@@ -260,7 +256,8 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     // Where the lane's codes of W piece 0 start inside a code tile.
     const uint32_t code_rd = kCodeBase + (wn * WN + r16) * 16 + kg * C::RB;
 
-    half8_t wp[NP], xp[MP];
+    half4_t wlo[NP], whi[NP];
+    half8_t xp[MP];
     uint32_t cr[2][4];  // codes behind the two W groups whose gathers come next
     // X piece i of MFMA step s out of stage buffer `buf`
     auto load_x1 = [&](int i, int buf, int s) {
@@ -271,15 +268,18 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         const int pos = (t % C::STAGES) * 2 * C::HALF + s * C::HALF;   // + kg*RB stays inside the 16-byte chunk
         cr[set][j & 3] = read_codes<C::RB>(smem + code_rd + cbuf * C::kTileBytes + (pos / 16) * (BN * 16) + j * 256 + pos % 16);
     };
-    // W piece j from the codes read before
+    // the two halves of W piece j from the codes read before
     auto load_w1 = [&](int set, int j, bool zero) {
-        wp[j] = gather8<VEC, CodeT, TAIL>(smem, book[j], cr[set][j & 3], zero, zero_off);
+        wlo[j] = gather4<VEC, CodeT, TAIL>(smem, book[j], cr[set][j & 3], 0, zero, zero_off);
+    };
+    auto load_w2 = [&](int set, int j, bool zero) {
+        whi[j] = gather4<VEC, CodeT, TAIL>(smem, book[j], cr[set][j & 3], 1, zero, zero_off);
     };
     // MFMA f of group p of the 4x4 quadrant (jh, ih): a group is W piece p against the four X
     // pieces, or (x_outer) X piece p against the four W pieces
     auto mfma_one = [&](int jh, int ih, int p, int f, bool x_outer) {
         const int j = jh * 4 + (x_outer ? f : p), i = ih * 4 + (x_outer ? p : f);
-        mfma_in_place(acc[j][i], wp[j], xp[i]);
+        mfma_in_place(acc[j][i], __builtin_shufflevector(wlo[j], whi[j], 0, 1, 2, 3, 4, 5, 6, 7), xp[i]);
     };
 
     // ---- prologue --------------------------------------------------------------------------
@@ -311,6 +311,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     }
     issue_x(0, D, D);
     issue_x(1, D, D);
+    if (mirrored) issue_x(2, D, D);  // the mirrored walk has three quadrants behind its barrier
     if (tid < 4) reinterpret_cast<uint32_t *>(smem + zero_off)[tid] = 0u;
     {
         // stage 0 (and everything older) must have landed; stages 1..D may be in flight
@@ -319,10 +320,10 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
             for (int d = 1; d < D; d++) n += loads_of(d);
             return n;
         }();
-        wait_vmcnt<in_flight>();
+        if (mirrored) wait_vmcnt<in_flight + 1>();
+        else wait_vmcnt<in_flight>();
     }
     __syncthreads();
-
     int buf = 0;   // X buffer of the current stage; stage+j lives in (buf + j) % NS
     int cbuf = 0;  // code buffer of the current super stage; super+j lives in (cbuf + j) % NC
 #pragma unroll
@@ -333,6 +334,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
 #pragma unroll
     for (int p = 0; p < 4; p++) {
         load_w1(0, p, false);
+        load_w2(0, p, false);
         load_x1(p, buf, 0);
     }
 
@@ -349,79 +351,167 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
 #define VQ_QUADRANT(LOADP, CODEP, jh, ih, x_outer, xi, TGT)                         \
     _Pragma("unroll") for (int p_ = 0; p_ < 4; p_++) {                              \
         mfma_one(jh, ih, p_, 0, x_outer); VQ_FENCE;                                 \
+        LOADP(p_); VQ_FENCE;                                                        \
         mfma_one(jh, ih, p_, 1, x_outer); VQ_FENCE;                                 \
-        LOADP(p_); CODEP(p_); VQ_FENCE;                                             \
+        LOADP##2(p_); CODEP(p_); VQ_FENCE;                                          \
         mfma_one(jh, ih, p_, 2, x_outer); VQ_FENCE;                                 \
-        mfma_one(jh, ih, p_, 3, x_outer); VQ_FENCE;                                 \
         if (p_ == 0) { issue_x(xi, TGT##_buf, TGT##_stage); VQ_FENCE; }             \
         if (p_ == 2 && TGT##_codes && xi < C::CH) { issue_codes(xi, TGT##_cbuf, TGT##_super); VQ_FENCE; } \
+        mfma_one(jh, ih, p_, 3, x_outer); VQ_FENCE;                                 \
     }
 
-    for (int super = 0; super < n_super; super++) {
-        // stage t (a compile-time 0 or 1) of the super stage
-        auto stage_body = [&](auto t_const) {
-            constexpr int t = decltype(t_const)::value;
-            const int stage = super * C::STAGES + t;
-            const int buf_next = buf + 1 == NS ? 0 : buf + 1;
-            // The barrier of a stage sits behind its last read of X (quadrant 6 of 8).  From there
-            // on the stage's buffer is free and the two quadrants left issue the first two of the
-            // eight X loads of stage+1+D into it (and that stage's code tile, when it opens a super
-            // stage); the first six quadrants issue loads 2..7 of stage+D into the buffer of
-            // stage-1.  A stage's loads so have two whole stages to land before the barrier that
-            // publishes them.
-            const int tgt_a_buf = buf == 0 ? NS - 1 : buf - 1, tgt_a_stage = stage + D;
-            constexpr bool tgt_a_codes = false;
-            const int tgt_a_cbuf = 0, tgt_a_super = 0;
-            const int tgt_b_buf = buf, tgt_b_stage = stage + 1 + D;
-            constexpr bool tgt_b_codes = (t + 1 + D) % C::STAGES == 0;
-            constexpr int d_super = (t + 1 + D) / C::STAGES;
-            const int tgt_b_super = super + d_super;
-            const int tgt_b_cbuf = (cbuf + d_super) % NC;
-            // the stage after this one: same super stage or the next
-            constexpr bool same_super = t + 1 < C::STAGES;
-            const int cbuf_n = same_super ? cbuf : (cbuf + 1 == NC ? 0 : cbuf + 1);
-            constexpr int t_n = same_super ? t + 1 : 0;
-            // a last stage of 32 k has no step 1
-            const bool no_b = TAIL && stage == n_stage - 1;
-            VQ_FENCE;
-            // step A (s = 0): W low/X low are in registers, the codes of W high in cr[1]
-#define L_WHI_A(p) load_w1(1, 4 + (p), false)
+    // Two walks.  Gathers are the expensive LDS reads (random codewords collide in the banks), and
+    // a walk loads W in four of its eight quadrants and X in the other four.  If every wave loaded
+    // W at the same time the LDS would be saturated in those quadrants and idle in the others, so
+    // the waves of the lower half of the tile take the mirrored walk (roles of W and X swapped):
+    // at any time two waves gather and two read X.
+    //
+    //   plain:     (Wl,Xl) (Wh,Xl) (Wh,Xh) (Wl,Xh) | (Wh,Xl) (Wl,Xl) | barrier | (Wl,Xh) (Wh,Xh)
+    //     loads     Wh      Xh      Xl'     Wh'       Wl'     Xh'                  Xl"     Wl"
+    //   mirrored:  (Wl,Xl) (Wl,Xh) (Wh,Xh) (Wh,Xl) | (Wl,Xh) | barrier | (Wl,Xl) (Wh,Xl) (Wh,Xh)
+    //     loads     Xh      Wh      Wl'     Xh'       Xl'                 Wh'     Wl"     Xl"
+    //
+    // (' = step B of the stage, " = step A of the next stage).  The barrier of a stage sits behind
+    // its last read of X and of its code tile.  From there on the stage's buffer is free and the
+    // quadrants left issue the first X loads of stage+1+D into it (and that stage's code tile,
+    // when it opens a super stage); the quadrants ahead of the barrier issue the rest of the eight
+    // X loads of stage+D into the buffer of stage-1.  A stage's loads so have two whole stages to
+    // land before the barrier that publishes them.
+#define VQ_STAGE_SETUP                                                              \
+    constexpr int t = decltype(t_const)::value;                                     \
+    const int stage = super * C::STAGES + t;                                        \
+    const int buf_next = buf + 1 == NS ? 0 : buf + 1;                               \
+    const int tgt_a_buf = buf == 0 ? NS - 1 : buf - 1, tgt_a_stage = stage + D;     \
+    constexpr bool tgt_a_codes = false;                                             \
+    const int tgt_a_cbuf = 0, tgt_a_super = 0;                                      \
+    const int tgt_b_buf = buf, tgt_b_stage = stage + 1 + D;                         \
+    constexpr bool tgt_b_codes = (t + 1 + D) % C::STAGES == 0;                      \
+    constexpr int d_super = (t + 1 + D) / C::STAGES;                                \
+    const int tgt_b_super = super + d_super;                                        \
+    const int tgt_b_cbuf = (cbuf + d_super) % NC;                                   \
+    /* the stage after this one: same super stage or the next */                   \
+    constexpr bool same_super = t + 1 < C::STAGES;                                  \
+    const int cbuf_n = same_super ? cbuf : (cbuf + 1 == NC ? 0 : cbuf + 1);         \
+    constexpr int t_n = same_super ? t + 1 : 0;                                     \
+    /* a last stage of 32 k has no step 1 */                                       \
+    const bool no_b = TAIL && stage == n_stage - 1;                                 \
+    /* publish stage+1: in flight may be what stages +2..+D bring along */         \
+    constexpr int in_flight = [&]() constexpr {                                     \
+        int n = 0;                                                                  \
+        for (int d = 2; d <= D; d++) n += loads_of(t + d);                          \
+        return n;                                                                   \
+    }();                                                                            \
+    VQ_FENCE
+
 #define L_XHI_A(p) load_x1(4 + (p), buf, 0)
 #define L_XLO_B(p) load_x1((p), buf, 1)
-#define L_WHI_B(p) load_w1(0, 4 + (p), no_b)
-#define L_WLO_B(p) load_w1(1, (p), no_b)
 #define L_XHI_B(p) load_x1(4 + (p), buf, 1)
 #define L_XLO_N(p) load_x1((p), buf_next, 0)
+#define L_XHI_A2(p) do {} while (0)
+#define L_XLO_B2(p) do {} while (0)
+#define L_XHI_B2(p) do {} while (0)
+#define L_XLO_N2(p) do {} while (0)
+    if (!mirrored) {
+        for (int super = 0; super < n_super; super++) {
+            // stage t (a compile-time 0 or 1) of the super stage
+            auto stage_body = [&](auto t_const) {
+                VQ_STAGE_SETUP;
+                // W low/X low are in registers, the codes of W high in cr[1]
+#define L_WHI_A(p) load_w1(1, 4 + (p), false)
+#define L_WHI_A2(p) load_w2(1, 4 + (p), false)
+#define L_WHI_B(p) load_w1(0, 4 + (p), no_b)
+#define L_WHI_B2(p) load_w2(0, 4 + (p), no_b)
+#define L_WLO_B(p) load_w1(1, (p), no_b)
+#define L_WLO_B2(p) load_w2(1, (p), no_b)
 #define L_WLO_N(p) load_w1(0, (p), false)
+#define L_WLO_N2(p) load_w2(0, (p), false)
 #define C_WHI_B(p) load_c1(0, 4 + (p), cbuf, t, 1)
 #define C_WLO_B(p) load_c1(1, (p), cbuf, t, 1)
 #define C_WLO_N(p) load_c1(0, (p), cbuf_n, t_n, 0)
 #define C_WHI_N(p) load_c1(1, 4 + (p), cbuf_n, t_n, 0)
-            VQ_QUADRANT(L_WHI_A, VQ_NONE, 0, 0, false, 2, tgt_a);   // W low (just loaded) x X low
-            VQ_QUADRANT(L_XHI_A, VQ_NONE, 1, 0, false, 3, tgt_a);   // W high (just loaded) x X low
-            VQ_QUADRANT(L_XLO_B, C_WHI_B, 1, 1, true, 4, tgt_a);    // W high x X high (just loaded)
-            VQ_QUADRANT(L_WHI_B, C_WLO_B, 0, 1, false, 5, tgt_a);   // W low x X high
-            // step B (s = 1)
-            VQ_QUADRANT(L_WLO_B, VQ_NONE, 1, 0, false, 6, tgt_a);   // W high (just loaded) x X low
-            VQ_QUADRANT(L_XHI_B, VQ_NONE, 0, 0, false, 7, tgt_a);   // W low (just loaded) x X low
-            {
-                // Publish stage+1: in flight may be what stages +2..+D bring along.
-                constexpr int in_flight = [&]() constexpr {
-                    int n = 0;
-                    for (int d = 2; d <= D; d++) n += loads_of(t + d);
-                    return n;
-                }();
+                VQ_QUADRANT(L_WHI_A, VQ_NONE, 0, 0, false, 2, tgt_a);   // W low (just loaded) x X low
+                VQ_QUADRANT(L_XHI_A, VQ_NONE, 1, 0, false, 3, tgt_a);   // W high (just loaded) x X low
+                VQ_QUADRANT(L_XLO_B, C_WHI_B, 1, 1, true, 4, tgt_a);    // W high x X high (just loaded)
+                VQ_QUADRANT(L_WHI_B, C_WLO_B, 0, 1, false, 5, tgt_a);   // W low x X high
+                VQ_QUADRANT(L_WLO_B, VQ_NONE, 1, 0, false, 6, tgt_a);   // W high' (just loaded) x X low'
+                VQ_QUADRANT(L_XHI_B, VQ_NONE, 0, 0, false, 7, tgt_a);   // W low' (just loaded) x X low'
                 wait_vmcnt<in_flight>();
-            }
-            __syncthreads();
-            VQ_QUADRANT(L_XLO_N, C_WLO_N, 0, 1, true, 0, tgt_b);    // W low x X high (just loaded)
-            VQ_QUADRANT(L_WLO_N, C_WHI_N, 1, 1, false, 1, tgt_b);   // W high x X high
-            buf = buf_next;
-        };
-        stage_body(std::integral_constant<int, 0>{});
-        if constexpr (C::STAGES == 2) stage_body(std::integral_constant<int, 1>{});
-        cbuf = cbuf + 1 == NC ? 0 : cbuf + 1;
+                __syncthreads();
+                VQ_QUADRANT(L_XLO_N, C_WLO_N, 0, 1, true, 0, tgt_b);    // W low' x X high' (just loaded)
+                VQ_QUADRANT(L_WLO_N, C_WHI_N, 1, 1, false, 1, tgt_b);   // W high' x X high'
+#undef L_WHI_A
+#undef L_WHI_A2
+#undef L_WHI_B
+#undef L_WHI_B2
+#undef L_WLO_B
+#undef L_WLO_B2
+#undef L_WLO_N
+#undef L_WLO_N2
+#undef C_WHI_B
+#undef C_WLO_B
+#undef C_WLO_N
+#undef C_WHI_N
+                buf = buf_next;
+            };
+            stage_body(std::integral_constant<int, 0>{});
+            if constexpr (C::STAGES == 2) stage_body(std::integral_constant<int, 1>{});
+            cbuf = cbuf + 1 == NC ? 0 : cbuf + 1;
+        }
+    } else {
+        for (int super = 0; super < n_super; super++) {
+            auto stage_body = [&](auto t_const) {
+                VQ_STAGE_SETUP;
+                // W low/X low are in registers
+#define C_WHI_A(p) load_c1(0, 4 + (p), cbuf, t, 0)
+#define L_WHI_A(p) load_w1(0, 4 + (p), false)
+#define L_WHI_A2(p) load_w2(0, 4 + (p), false)
+#define C_WLO_B(p) load_c1(1, (p), cbuf, t, 1)
+#define L_WLO_B(p) load_w1(1, (p), no_b)
+#define L_WLO_B2(p) load_w2(1, (p), no_b)
+#define C_WHI_B(p) load_c1(0, 4 + (p), cbuf, t, 1)
+#define L_WHI_B(p) load_w1(0, 4 + (p), no_b)
+#define L_WHI_B2(p) load_w2(0, 4 + (p), no_b)
+#define C_WLO_N(p) load_c1(1, (p), cbuf_n, t_n, 0)
+#define L_WLO_N(p) load_w1(1, (p), false)
+#define L_WLO_N2(p) load_w2(1, (p), false)
+                VQ_QUADRANT(L_XHI_A, C_WHI_A, 0, 0, true, 3, tgt_a);    // W low x X low (just loaded)
+                VQ_QUADRANT(L_WHI_A, C_WLO_B, 0, 1, true, 4, tgt_a);    // W low x X high (just loaded)
+                VQ_QUADRANT(L_WLO_B, VQ_NONE, 1, 1, false, 5, tgt_a);   // W high (just loaded) x X high
+                VQ_QUADRANT(L_XHI_B, VQ_NONE, 1, 0, false, 6, tgt_a);   // W high x X low
+                VQ_QUADRANT(L_XLO_B, C_WHI_B, 0, 1, true, 7, tgt_a);    // W low' x X high' (just loaded)
+                wait_vmcnt<in_flight>();
+                __syncthreads();
+                VQ_QUADRANT(L_WHI_B, C_WLO_N, 0, 0, true, 0, tgt_b);    // W low' x X low' (just loaded)
+                VQ_QUADRANT(L_WLO_N, VQ_NONE, 1, 0, false, 1, tgt_b);   // W high' (just loaded) x X low'
+                VQ_QUADRANT(L_XLO_N, VQ_NONE, 1, 1, false, 2, tgt_b);   // W high' x X high'
+#undef C_WHI_A
+#undef L_WHI_A
+#undef L_WHI_A2
+#undef C_WLO_B
+#undef L_WLO_B
+#undef L_WLO_B2
+#undef C_WHI_B
+#undef L_WHI_B
+#undef L_WHI_B2
+#undef C_WLO_N
+#undef L_WLO_N
+#undef L_WLO_N2
+                buf = buf_next;
+            };
+            stage_body(std::integral_constant<int, 0>{});
+            if constexpr (C::STAGES == 2) stage_body(std::integral_constant<int, 1>{});
+            cbuf = cbuf + 1 == NC ? 0 : cbuf + 1;
+        }
     }
+#undef L_XHI_A
+#undef L_XHI_A2
+#undef L_XLO_B2
+#undef L_XHI_B2
+#undef L_XLO_N2
+#undef L_XLO_B
+#undef L_XHI_B
+#undef L_XLO_N
+#undef VQ_STAGE_SETUP
 #undef VQ_QUADRANT
 #undef VQ_FENCE
     // Drain the clamped loads still in flight before the stage buffers are reused.
@@ -429,7 +519,6 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     __syncthreads();
     // the last MFMAs must have left the pipe before the accumulators are read
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-
     // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its wave tile ------
     if ((N & 7) == 0) {
         // Through the LDS: each wave transposes its 128x128 fp16 block, 64 rows at a time, in a
