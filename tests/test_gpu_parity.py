@@ -175,6 +175,50 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
     assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)
 
 
+# Shapes that walk the prefill kernel through each of its instantiations: both super-stage
+# lengths (one or two 64-k stages per code tile), one or two 16-byte code chunks per row, a last
+# stage of 32 k, four, three and two X buffers (large codebooks), several codebooks per 256-row
+# tile (aligned and not), ragged M and N, fewer stages than the pipeline is deep.
+PREFILL_B = [
+    # name, M, K, N, vec, E, bits, G
+    ("u8v8_one_super", 256, 128, 256, 8, 256, 8, 1),
+    ("u8v8_odd_supers_2_books_per_tile", 256, 384, 256, 8, 256, 8, 2),
+    ("u8v8_ragged_5_books", 1000, 1152, 1000, 8, 256, 8, 5),
+    ("u8v8_n_not_mult_of_8", 513, 1024, 1001, 8, 256, 8, 1),
+    ("u8v8_k11008_32_books", 600, 11008, 1024, 8, 256, 8, 32),
+    ("u16v8_k_odd_stages", 512, 1088, 512, 8, 1024, 16, 2),
+    ("u8v4", 512, 1088, 768, 4, 256, 8, 3),
+    ("u16v4_e4096_three_buffers", 512, 1024, 512, 4, 4096, 16, 1),
+    ("u16v4_e4096_tail32", 512, 1056, 512, 4, 4096, 16, 1),
+    ("u16v4_e4096_two_books_two_buffers", 300, 1056, 96, 4, 4096, 16, 2),
+    ("u8v2_tail32_ragged_n", 512, 1056, 520, 2, 256, 8, 1),
+    ("u8v2_k32_only_a_tail", 260, 32, 264, 2, 256, 8, 1),
+    ("u8v8_many_tiles", 2048, 2048, 4096, 8, 256, 8, 16),
+]
+
+
+@pytest.mark.parametrize("row", PREFILL_B, ids=[r[0] for r in PREFILL_B])
+def test_prefill_kernel_instantiations(row):
+    name, M, K, N, v, E, bits, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+    x, codes, cb = make_problem(spec, seed=33, device=DEV)
+    _say("prefill", spec)
+    y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_PREFILL)
+    torch.cuda.synchronize()
+    w = vo.dequant_b(_np(codes), _np(cb))
+    ref = _np(x).astype(np.float64) @ w.astype(np.float64).T
+    e1, e2 = vo.rel_err(_np(y), ref)
+    _say(f"  {name}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+    assert e1 <= TOL
+    # a permuted one-hot X reads W out bit for bit through the same kernel
+    eye = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+    cols = [(37 * m + 11) % K for m in range(M)]
+    eye[torch.arange(M), torch.tensor(cols)] = 1.0
+    yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_PREFILL)
+    assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_PREFILL), y)
+
+
 def test_every_m_from_1_to_16_on_the_decode_kernel():
     K, N = 1024, 80
     for M in range(1, 17):
