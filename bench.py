@@ -50,6 +50,9 @@ def parse_args():
                     help="profiling aid: launch CONFIG (C1..C5, or a geometry-B shape M,K,N,vec,entries,code_bits) "
                          "--steps times, cold-HBM rotation for the decode configs, followed by one 256 MiB "
                          "device copy as a counter yardstick; prints no JSON")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="run the register-only MFMA loop (vq_gemm_amd/lib/mfma_ceiling): what the matrix cores "
+                         "sustain on this device with random and with zero operands; prints no JSON")
     return ap.parse_args()
 
 
@@ -59,6 +62,14 @@ def main():
         print("bench.py measures the single-GPU VQ-GEMM path; this build has no multi-GPU leg "
               "(the path shards along N without any exchange). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.mfma_ceiling:
+        import subprocess
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vq_gemm_amd", "lib", "mfma_ceiling")
+        if not os.path.exists(exe):
+            print(f"{exe} is not built (python -m vq_gemm_amd.build)", file=sys.stderr)
+            sys.exit(2)
+        sys.exit(subprocess.run([exe]).returncode)
 
     import torch
 

@@ -3,6 +3,7 @@
 Artefacts (all under vq_gemm_amd/lib/):
   libvqgemm.so        the C-ABI library (HIP kernels + dispatch), no torch dependency
   libvqgemm_ref.so    hipBLASLt fp16 baseline
+  mfma_ceiling        stand-alone program: what a register-only MFMA loop sustains on the device
   vq_gemm_cuda_<k>.so one torch extension module per variant, named as the reference's
                       harness imports them (reference compile_kernels.py:55-68, bench.py:6-11)
 
@@ -134,6 +135,16 @@ def build_ref(force: bool = True) -> str:
     return out
 
 
+def build_ceiling(force: bool = True) -> str:
+    """Register-only MFMA loop (csrc/mfma_ceiling.hip), run by `bench.py --mfma-ceiling`."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(CSRC, "mfma_ceiling.hip")
+    out = os.path.join(LIB_DIR, "mfma_ceiling")
+    if force or not _newer(out, [src]):
+        _run([HIPCC] + [f for f in HIP_FLAGS if f != "-fPIC"] + [src, "-o", out])
+    return out
+
+
 def build_ext(keys=None, force: bool = True, jobs: int = 6):
     """Torch extension modules, one per variant key (host C++ only)."""
     import torch  # noqa: F401  (needed for its include/lib paths)
@@ -175,8 +186,9 @@ def build_ext(keys=None, force: bool = True, jobs: int = 6):
 def build_all(keys=None, force: bool = True):
     lib = build_lib(force=force)
     ref = build_ref(force=force)
+    ceiling = build_ceiling(force=force)
     exts = build_ext(keys, force=force)
-    return [lib, ref] + exts
+    return [lib, ref, ceiling] + exts
 
 
 if __name__ == "__main__":
