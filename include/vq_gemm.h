@@ -39,7 +39,7 @@ extern "C" {
 #define VQGEMM_VARIANT_DECODE 2   /* small and medium M, 16 rows of X per workgroup: K-sliced waves, 16x16x32 MFMA,
                                      LDS-resident codebook; M <= 4096 when K % 256 == 0, K <= 4096, N % 16 == 0 and
                                      (N / n_codebooks) % 16 == 0, M <= 64 otherwise */
-#define VQGEMM_VARIANT_PREFILL 3  /* large M: 32x32x16 MFMA tiles, codewords gathered into operands */
+#define VQGEMM_VARIANT_PREFILL 3  /* large M: 256x256 tiles of 16x16x32 MFMAs, codewords gathered into operands */
 #define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */
 
 /*
