@@ -37,7 +37,7 @@ extern "C" {
 #define VQGEMM_VARIANT_AUTO 0     /* pick by shape */
 #define VQGEMM_VARIANT_GENERIC 1  /* simple scalar kernel, any shape */
 #define VQGEMM_VARIANT_DECODE 2   /* small and medium M, 16 rows of X per workgroup: K-sliced waves, 16x16x32 MFMA,
-                                     LDS-resident codebook; M <= 4096 when K % 256 == 0, K <= 4096, N % 16 == 0 and
+                                     LDS-resident codebook; M <= 4096 when K % 256 == 0, N % 16 == 0 and
                                      (N / n_codebooks) % 16 == 0, M <= 64 otherwise */
 #define VQGEMM_VARIANT_PREFILL 3  /* large M: 256x256 tiles of 16x16x32 MFMAs, codewords gathered into operands */
 #define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */
@@ -75,6 +75,18 @@ int vqgemm_dequant_b(const void *codes, const void *codebook, void *w_out,
                      int32_t n_codebooks, int32_t code_bits, void *stream);
 int vqgemm_dequant_a(const void *w, const void *codebook, void *w_out,
                      int64_t K, int64_t Nc, void *stream);
+
+/*
+ * Nearest-codeword encoder, geometry B: the inverse of vqgemm_dequant_b for given codebooks,
+ *   codes_out[n, j] = argmin_e sum_t (w[n, j*vec + t] - codebook[n / (N/n_codebooks)][e][t])^2,
+ * w [N,K] fp16, codes_out [N, K/vec] uint8 or uint16.  Distances are accumulated in fp32 in vector
+ * order with a fused multiply-add; ties go to the lowest index.  vec must be 2, 4 or 8.
+ * No counterpart in the reference, whose harness multiplies random codes (bench.py:84): this is the
+ * assignment step of the quantiser that produces the codes the GEMM path consumes.
+ */
+int vqgemm_encode_b(const void *w, const void *codebook, void *codes_out,
+                    int64_t N, int64_t K, int32_t vec, int32_t entries,
+                    int32_t n_codebooks, int32_t code_bits, void *stream);
 
 /*
  * Plain fp16 GEMM o[M,N] = input[M,K] . w[K,N] (fp32 accumulate), the no-dequant control.

@@ -129,3 +129,16 @@ def gemm_nn(x, w) -> np.ndarray:
     I64 = ctypes.c_int64
     _check(lib().vqo_gemm_nn(_p(_u16(x)), _p(_u16(w)), _p(y), I64(M), I64(K), I64(N)))
     return y.view(np.float16)
+
+
+def encode_b(w, codebook, code_bits: int) -> np.ndarray:
+    """Nearest-codeword codes [N, K/v] of W [N,K] fp16 (fp32 fused-multiply-add distances,
+    lowest index on ties)."""
+    w = np.ascontiguousarray(w)
+    cb = _cb3(codebook)
+    G, E, v = cb.shape
+    N, K = w.shape
+    out = np.empty((N, K // v), dtype=np.uint8 if code_bits == 8 else np.uint16)
+    I64, I = ctypes.c_int64, ctypes.c_int
+    _check(lib().vqo_encode_b(_p(_u16(w)), _p(_u16(cb)), _p(out), I(code_bits), I64(N), I64(K), I(v), I(E), I(G)))
+    return out

@@ -8,12 +8,17 @@
  * that it shares no code (and no vectorised library routine) with the numpy restatement
  * it is cross-checked against.
  *
+ * The nearest-codeword encoder (vqo_encode_b) has no counterpart in the reference (which only
+ * ever multiplies random codes, bench.py:84); its rule is stated here and pinned by brute force
+ * in float64, exact-tie cases and the dequantise -> encode round trip.
+ *
  * Pinning status: every function here is pinned by tests/test_oracle.py (hand-computed
  * known answers, identities, cross-check against the numpy restatement).
  */
 #include <stdint.h>
 #include <stddef.h>
 #include <string.h>
+#include <math.h>
 
 /* ---- IEEE 754 binary16 <-> binary32, bit level, round-to-nearest-even ---- */
 static float h2f(uint16_t h)
@@ -186,5 +191,44 @@ int vqo_vq_gemm_a(const uint16_t *x, const uint8_t *w, const uint16_t *cb, uint1
                 }
                 y[m * Nout + n * ratio + r] = f2h(acc);
             }
+    return 0;
+}
+
+/*
+ * Nearest-codeword encoder, geometry B: codes[n,j] = argmin_e sum_t (W[n,j*v+t] - cb[g][e][t])^2.
+ * The distance is accumulated in binary32 in vector order with a fused multiply-add
+ * (acc = fma(d, d, acc), d = w - c in binary32); entry 0 starts as the best and a later entry
+ * replaces it only when strictly closer (ties keep the lowest index, a NaN distance never wins).
+ */
+int vqo_encode_b(const uint16_t *w, const uint16_t *cb, void *codes_out, int code_bits,
+                 int64_t N, int64_t K, int v, int E, int G)
+{
+    if (v <= 0 || G <= 0 || E <= 0 || K % v != 0 || N % G != 0 || (code_bits != 8 && code_bits != 16))
+        return -1;
+    if ((int64_t)E > ((int64_t)1 << code_bits))
+        return -1;
+    int64_t J = K / v, rpc = N / G;
+    for (int64_t n = 0; n < N; n++) {
+        const uint16_t *book = cb + (n / rpc) * (int64_t)E * v;
+        for (int64_t j = 0; j < J; j++) {
+            float best = 0.0f;
+            int64_t arg = 0;
+            for (int64_t e = 0; e < E; e++) {
+                float acc = 0.0f;
+                for (int t = 0; t < v; t++) {
+                    float d = h2f(w[n * K + j * v + t]) - h2f(book[e * v + t]);
+                    acc = fmaf(d, d, acc);
+                }
+                if (e == 0 || acc < best) {
+                    best = acc;
+                    arg = e;
+                }
+            }
+            if (code_bits == 8)
+                ((uint8_t *)codes_out)[n * J + j] = (uint8_t)arg;
+            else
+                ((uint16_t *)codes_out)[n * J + j] = (uint16_t)arg;
+        }
+    }
     return 0;
 }

@@ -132,3 +132,20 @@ def rel_err(y: np.ndarray, ref: np.ndarray, floor_frac: float = 1e-2):
     e1 = float(np.max(diff / np.maximum(np.abs(ref), tau)))
     e2 = float(np.max(diff) / max(float(np.max(np.abs(ref))), 1e-30))
     return e1, e2
+
+
+def encode_b_distances(w: np.ndarray, codebook: np.ndarray) -> np.ndarray:
+    """Squared distances [N, J, E] in float64 between every vector of W [N,K] and every entry of
+    its row's codebook: the brute-force statement the nearest-codeword encoder is checked against
+    (the encoder itself accumulates in float32, so it is compared through these distances, not
+    through an argmin that could differ on near-ties)."""
+    w = np.asarray(w)
+    cb = _as_cb3(codebook)
+    G, E, v = cb.shape
+    N, K = w.shape
+    if N % G != 0 or K % v != 0:
+        raise ValueError("N must be a multiple of the number of codebooks and K of the vector length")
+    wv = w.astype(np.float64).reshape(N, K // v, 1, v)
+    g = np.arange(N, dtype=np.int64) // (N // G)
+    books = cb.astype(np.float64)[g][:, None, :, :]      # [N,1,E,v]
+    return ((wv - books) ** 2).sum(axis=-1)

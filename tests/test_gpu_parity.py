@@ -219,6 +219,67 @@ def test_prefill_kernel_instantiations(row):
     assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_PREFILL), y)
 
 
+ENCODE_B = [
+    # name, N, K, vec, E, G, bits
+    ("u8v8_256", 64, 256, 8, 256, 1, 8),
+    ("u16v4_4096_two_books", 96, 128, 4, 4096, 2, 16),
+    ("u8v2_100_five_books", 50, 64, 2, 100, 5, 8),
+    ("u16v8_5000_chunked_codebook", 40, 64, 8, 5000, 1, 16),
+    ("u16v8_e300_ragged_block", 33, 136, 8, 300, 3, 16),
+]
+
+
+@pytest.mark.parametrize("row", ENCODE_B, ids=[r[0] for r in ENCODE_B])
+def test_encoder_matches_the_c_oracle_bit_for_bit(row):
+    name, N, K, v, E, G, bits = row
+    _say("encode", row)
+    g = torch.Generator(device="cpu").manual_seed(5)
+    cb = torch.randn(G, E, v, generator=g).half()
+    w = torch.randn(N, K, generator=g).half()
+    # a third of the vectors sit on or next to codebook entries (exact zeros, near-ties)
+    pick = torch.randint(0, E, (N, K // v), generator=g)
+    near = cb[(torch.arange(N) // (N // G))[:, None], pick].reshape(N, K)
+    mask = (torch.rand(N, K // v, generator=g) < 0.33).repeat_interleave(v, dim=1)
+    w = torch.where(mask, near, w)
+    codes = cabi.encode_b(w.to(DEV), cb.to(DEV), bits)
+    torch.cuda.synchronize()
+    want = c_oracle.encode_b(w.numpy(), cb.numpy(), bits)
+    assert codes.dtype == (torch.uint8 if bits == 8 else torch.uint16)
+    assert np.array_equal(_np(codes), want)
+    # the codes dequantise (bit-exactly) to what the oracle's codes dequantise to
+    assert np.array_equal(_np(cabi.dequant_b(codes, cb.to(DEV))), vo.dequant_b(want, cb.numpy()))
+
+
+def test_encoder_inverts_the_dequantiser_on_the_gpu():
+    spec = ProblemSpec("enc", GEOM_B, 1, 1024, 512, 8, 256, 4, 8, codebook_3d=True, codebook_std=1.0)
+    _, codes, cb = make_problem(spec, seed=8, device=DEV)
+    assert all(len({tuple(e) for e in _np(cb)[g].tolist()}) == 256 for g in range(4))
+    w = cabi.dequant_b(codes, cb)
+    assert torch.equal(cabi.encode_b(w, cb, 8), codes)
+
+
+def test_kmeans_quantiser_feeds_the_gemm_path():
+    from vq_gemm_amd.quantize import kmeans_quantize
+    g = torch.Generator(device="cpu").manual_seed(9)
+    N, K, v, E, G = 512, 1024, 8, 256, 2
+    # weights drawn around 64 centres per block: a 256-entry codebook can represent them well
+    centres = torch.randn(G, 64, v, generator=g) * 0.05
+    which = torch.randint(0, 64, (N, K // v), generator=g)
+    w = centres[(torch.arange(N) // (N // G))[:, None], which].reshape(N, K)
+    w = (w + torch.randn(N, K, generator=g) * 0.002).half().to(DEV)
+    codes, cb, hist = kmeans_quantize(w, v, E, n_codebooks=G, iters=6, seed=1)
+    _say("k-means mse per element:", ["%.3e" % h for h in hist])
+    assert codes.shape == (N, K // v) and codes.dtype == torch.uint8 and cb.shape == (G, E, v)
+    assert hist[-1] <= hist[0] and hist[-1] < 0.2 * float((w.float() ** 2).mean())
+    # the returned codes are the nearest entries of the returned codebook
+    assert torch.equal(cabi.encode_b(w, cb, 8), codes)
+    # and the pair drives the fused GEMM: same result as the oracle on the same codes
+    x = torch.randn(32, K, generator=g).half().to(DEV)
+    y = cabi.e2e_gemm_b(x, codes, cb)
+    torch.cuda.synchronize()
+    _check_gemm(y, x, codes, cb, what="quantised weights")
+
+
 def test_every_m_from_1_to_16_on_the_decode_kernel():
     K, N = 1024, 80
     for M in range(1, 17):

@@ -287,3 +287,55 @@ def test_golden_fixture(name):
     for got in (y, yc):
         e1, _ = vo.rel_err(got[ri][:, ci], data["y_samples_f64"])
         assert e1 <= 2e-3
+
+
+# ---- nearest-codeword encoder (the quantiser's assignment step) -------------------------------
+
+def _rand_encode_case(rng, N, K, v, E, G):
+    w = rng.standard_normal((N, K)).astype(np.float16)
+    cb = rng.standard_normal((G, E, v)).astype(np.float16)
+    return w, cb
+
+
+@pytest.mark.parametrize("N,K,v,E,G,bits", [(8, 32, 8, 16, 1, 8), (12, 24, 4, 300, 3, 16), (6, 20, 2, 7, 2, 8)])
+def test_encoder_picks_a_nearest_entry(N, K, v, E, G, bits):
+    """The C encoder (float32 fma distances) against brute force in float64: the entry it picks
+    is a nearest one up to float32 rounding of the distances."""
+    rng = np.random.default_rng(7)
+    w, cb = _rand_encode_case(rng, N, K, v, E, G)
+    codes = c_oracle.encode_b(w, cb, bits)
+    assert codes.dtype == (np.uint8 if bits == 8 else np.uint16) and codes.shape == (N, K // v)
+    d = vo.encode_b_distances(w, cb)                         # [N,J,E] float64
+    picked = np.take_along_axis(d, codes.astype(np.int64)[:, :, None], axis=2)[:, :, 0]
+    best = d.min(axis=2)
+    assert np.all(picked <= best * (1 + 1e-5) + 1e-12)
+    # where the nearest entry is clearly nearest (no near-tie) the index itself is pinned
+    second = np.partition(d, 1, axis=2)[:, :, 1]
+    clear = second > best * (1 + 1e-4) + 1e-9
+    assert clear.mean() > 0.9
+    assert np.array_equal(codes[clear], d.argmin(axis=2)[clear].astype(codes.dtype))
+
+
+def test_encoder_known_answers_and_ties():
+    # hand-made: 2-vectors, codebook {(0,0),(1,0),(0,1),(1,0) again}; ties go to the lowest index
+    cb = np.array([[[0, 0], [1, 0], [0, 1], [1, 0]]], dtype=np.float16)
+    w = np.array([[0.9, 0.1, 0.1, 0.8, 0.5, 0.0, 0.5, 0.5]], dtype=np.float16)
+    # (0.9,0.1)->1 (not its duplicate 3); (0.1,0.8)->2; (0.5,0)->tie of 0 and 1 -> 0;
+    # (0.5,0.5)-> d=0.5 for entries 0,1,2,3 -> 0
+    assert c_oracle.encode_b(w, cb, 8).tolist() == [[1, 2, 0, 0]]
+    assert c_oracle.encode_b(w, cb, 16).tolist() == [[1, 2, 0, 0]]
+
+
+def test_encoder_inverts_the_dequantiser():
+    """encode(dequant(codes)) == codes when the entries of a codebook are distinct (distance 0 is
+    reached by exactly one entry), per codebook block."""
+    rng = np.random.default_rng(11)
+    G, E, v, N, K = 2, 64, 4, 16, 32
+    cb = rng.standard_normal((G, E, v)).astype(np.float16)
+    assert all(len({tuple(e) for e in cb[g].tolist()}) == E for g in range(G))
+    codes = rng.integers(0, E, (N, K // v)).astype(np.uint8)
+    w = vo.dequant_b(codes, cb)
+    assert np.array_equal(c_oracle.encode_b(w, cb, 8), codes)
+    # a NaN vector keeps entry 0, whatever the codebook
+    w[3, 4:8] = np.nan
+    assert c_oracle.encode_b(w, cb, 8)[3, 1] == 0

@@ -23,6 +23,7 @@ _SIGNATURES = {
     "vqgemm_e2e_gemm_a": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _P]),
     "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_dequant_a": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
+    "vqgemm_encode_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _P]),
     "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
     "vqgemm_error_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -135,6 +136,21 @@ def dequant_b(codes, codebook, out=None):
     rc = lib().vqgemm_dequant_b(_ptr(codes), _ptr(codebook), _ptr(out), N, J * v, v, E, G, bits, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_dequant_b")
+    return out
+
+
+def encode_b(w, codebook, code_bits=None, out=None):
+    """Nearest-codeword codes [N, K/vec] of W [N,K] fp16 for the given codebook(s)."""
+    import torch
+    N, K = w.shape
+    G, E, v = _cb_dims(codebook)
+    if code_bits is None:
+        code_bits = 8 if E <= 256 else 16
+    if out is None:
+        out = torch.empty((N, K // v), dtype=torch.uint8 if code_bits == 8 else torch.uint16, device=w.device)
+    rc = lib().vqgemm_encode_b(_ptr(w), _ptr(codebook), _ptr(out), N, K, v, E, G, code_bits, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_encode_b")
     return out
 
 

@@ -205,6 +205,19 @@ int vqgemm_dequant_b(const void *codes, const void *codebook, void *w_out, int64
     return static_cast<int>(launch_dequant_b(p, static_cast<half_t *>(w_out), static_cast<hipStream_t>(stream)));
 }
 
+int vqgemm_encode_b(const void *w, const void *codebook, void *codes_out, int64_t N, int64_t K, int32_t vec,
+                    int32_t entries, int32_t n_codebooks, int32_t code_bits, void *stream)
+{
+    const int rc = check_b(0, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (N == 0 || K == 0) return VQGEMM_OK;
+    if (!w || !codebook || !codes_out) return VQGEMM_E_NULL;
+    if (!aligned(w, 2) || !aligned(codebook, 2) || !aligned(codes_out, code_bits / 8)) return VQGEMM_E_ALIGN;
+    const ProblemB p = make_b(nullptr, nullptr, codebook, nullptr, 0, K, N, vec, entries, n_codebooks, code_bits);
+    if (!encode_supports(p)) return VQGEMM_E_VARIANT;
+    return static_cast<int>(launch_encode_b(static_cast<const half_t *>(w), p, codes_out, static_cast<hipStream_t>(stream)));
+}
+
 int vqgemm_dequant_a(const void *w, const void *codebook, void *w_out, int64_t K, int64_t Nc, void *stream)
 {
     if (K < 0 || Nc < 0 || K > INT_MAX / 2 || Nc > INT_MAX / 4 || Nc % 4 != 0) return VQGEMM_E_SHAPE;

@@ -55,6 +55,10 @@ __device__ __forceinline__ half8_t as_half8(T v)
 hipError_t launch_dequant_b(const ProblemB &p, half_t *w_out, hipStream_t s);
 hipError_t launch_dequant_a(const ProblemA &p, half_t *w_out, hipStream_t s);
 
+// nearest-codeword codes of w[N,K] (p.x, p.y unused)
+bool encode_supports(const ProblemB &p);
+hipError_t launch_encode_b(const half_t *w, const ProblemB &p, void *codes_out, hipStream_t s);
+
 hipError_t launch_generic_b(const ProblemB &p, hipStream_t s);
 hipError_t launch_generic_a(const ProblemA &p, hipStream_t s);
 
