@@ -39,8 +39,10 @@ extern "C" {
 #define VQGEMM_VARIANT_DECODE 2   /* small and medium M, 16 rows of X per workgroup: K-sliced waves, 16x16x32 MFMA,
                                      LDS-resident codebook; M <= 4096 when K % 256 == 0, N % 16 == 0 and
                                      (N / n_codebooks) % 16 == 0, M <= 64 otherwise */
-#define VQGEMM_VARIANT_PREFILL 3  /* large M: 256x256 tiles of 16x16x32 MFMAs, codewords gathered into operands */
+#define VQGEMM_VARIANT_PREFILL 3  /* large M: 256x256 tiles of 16x16x32 MFMAs, codewords gathered into operands;
+                                     256x128 tiles when those put more compute units to work */
 #define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */
+#define VQGEMM_VARIANT_PREFILL_NARROW 5  /* the prefill kernel with 256x128 tiles, whatever the shape */
 
 /*
  * Fused VQ GEMM, geometry B.

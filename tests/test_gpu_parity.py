@@ -85,13 +85,13 @@ def test_e2e_gemm_b_all_variants(row):
     _say("e2e_gemm_b", spec, "auto ->", cabi.VARIANT_NAMES[auto])
     ran = []
     for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL,
-                    cabi.VARIANT_TWOPASS):
+                    cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_TWOPASS):
         _say("  variant", cabi.VARIANT_NAMES[variant])
         try:
             y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
         except cabi.VqGemmError as e:
             assert e.code == -4, e          # "variant cannot serve this shape" is the only accepted refusal
-            assert variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL)
+            assert variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW)
             continue
         torch.cuda.synchronize()
         _check_gemm(y, x, codes, cb, what=f"{spec.name}/{cabi.VARIANT_NAMES[variant]}")
@@ -101,7 +101,8 @@ def test_e2e_gemm_b_all_variants(row):
         assert cabi.VARIANT_DECODE in ran
 
 
-@pytest.mark.parametrize("variant", [cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_GENERIC])
+@pytest.mark.parametrize("variant", [cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
+                                     cabi.VARIANT_GENERIC])
 @pytest.mark.parametrize("vec,bits,E", [(8, 8, 256), (4, 16, 4096), (4, 8, 256), (8, 16, 512)])
 def test_one_hot_activations_return_weight_columns_bit_exactly(variant, vec, bits, E):
     """X = rows of the identity: Y[m,:] must equal W[:,m] exactly (1.0*w + zeros is exact), which
@@ -114,7 +115,11 @@ def test_one_hot_activations_return_weight_columns_bit_exactly(variant, vec, bit
         _say("one-hot", cabi.VARIANT_NAMES[variant], vec, bits, "k0", k0)
         x = torch.zeros(16, K, dtype=torch.float16, device=DEV)
         x[torch.arange(16), k0 + torch.arange(16)] = 1.0
-        y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
+        try:
+            y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
+        except cabi.VqGemmError as e:
+            assert variant == cabi.VARIANT_PREFILL_NARROW and e.code == -4 and E * vec * 2 >= 32768
+            pytest.skip("codebooks too large for the narrow tile")
         torch.cuda.synchronize()
         assert np.array_equal(_np(y).view(np.uint16), w[:, k0:k0 + 16].T.copy().view(np.uint16))
 
@@ -197,13 +202,19 @@ PREFILL_B = [
 ]
 
 
+@pytest.mark.parametrize("variant", [cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW])
 @pytest.mark.parametrize("row", PREFILL_B, ids=[r[0] for r in PREFILL_B])
-def test_prefill_kernel_instantiations(row):
+def test_prefill_kernel_instantiations(row, variant):
     name, M, K, N, v, E, bits, G = row
     spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
     x, codes, cb = make_problem(spec, seed=33, device=DEV)
-    _say("prefill", spec)
-    y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_PREFILL)
+    _say("prefill", cabi.VARIANT_NAMES[variant], spec)
+    try:
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
+    except cabi.VqGemmError as e:
+        # the 256x128 tile keeps four X buffers and does not take the largest codebooks
+        assert variant == cabi.VARIANT_PREFILL_NARROW and e.code == -4 and E * v * 2 >= 32768
+        pytest.skip("codebooks too large for the narrow tile")
     torch.cuda.synchronize()
     w = vo.dequant_b(_np(codes), _np(cb))
     ref = _np(x).astype(np.float64) @ w.astype(np.float64).T
@@ -214,9 +225,9 @@ def test_prefill_kernel_instantiations(row):
     eye = torch.zeros(M, K, dtype=torch.float16, device=DEV)
     cols = [(37 * m + 11) % K for m in range(M)]
     eye[torch.arange(M), torch.tensor(cols)] = 1.0
-    yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_PREFILL)
+    yw = cabi.e2e_gemm_b(eye, codes, cb, variant=variant)
     assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
-    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_PREFILL), y)
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=variant), y)
 
 
 ENCODE_B = [
@@ -294,7 +305,7 @@ def test_every_m_from_1_to_16_on_the_decode_kernel():
 def test_properties_constant_codes_zero_codebook_scaling():
     spec = ProblemSpec("prop", GEOM_B, 16, 1024, 128, 8, 256, 1, 8)
     x, codes, cb = make_problem(spec, seed=4, device=DEV)
-    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL):
+    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW):
         _say("properties", cabi.VARIANT_NAMES[variant])
         const = torch.full_like(codes, 37)
         y = cabi.e2e_gemm_b(x, const, cb, variant=variant)

@@ -71,7 +71,12 @@ bool decode_general_supports(const ProblemB &p);
 hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);
 
 bool prefill_supports(const ProblemB &p);
-hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s);
+// whether the 256x128 tile of the prefill kernel can serve the shape (a subset of prefill_supports)
+bool prefill_narrow_supports(const ProblemB &p);
+// expected time of the prefill kernel with the tile width it would choose, microseconds
+double prefill_cost_us(const ProblemB &p);
+// tile: 0 = the width expected to be faster, 1 = 256x256, 2 = 256x128
+hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile = 0);
 
 // o[M,N] = x[M,K] . w[K,N]
 hipError_t launch_gemm_nn(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);

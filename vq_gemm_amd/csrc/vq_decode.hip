@@ -728,9 +728,8 @@ bool decode_preferred(const ProblemB &p)
     const double t_tile = (g.n_chunks == 1 ? 0.75 : 1.25) * g.n_waves / kMaxWaves * g.per_cu;
     const int passes = g.books_per_wg * g.n_chunks;
     const double t_decode = rounds_d * (3.0 + passes * g.tiles_per_wg * t_tile + (passes - 1) * 3.5);
-    const double tiles = (double)((p.M + 255) / 256) * ((p.N + 255) / 256);
-    const double frac = tiles < cus ? tiles / cus : 1.0;
-    const double t_prefill = 8.0 + (tiles < cus ? 1.0 : tiles / cus) * (p.K / 64.0) * (0.85 + 0.9 * frac);
+    // the prefill kernel's own estimate for the tile width it would choose, plus launch and drain
+    const double t_prefill = prefill_supports(p) ? 3.0 + prefill_cost_us(p) : 1e30;
     return t_decode <= t_prefill;
 }
 

@@ -567,38 +567,374 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     }
 }
 
+// ---- the 256x128 tile ------------------------------------------------------------------------
+// When the 256x256 tiles of a problem are fewer than the compute units (medium M, small N), a
+// tile half as wide puts twice as many units to work: the same 256 threads (2x2 waves), 256
+// rows of X, 128 rows of W, each wave 128x64 as 8 X pieces x 4 W pieces.  Half the accumulators
+// leave room to double buffer every operand, so the schedule is plain: while MFMA step s
+// multiplies, all operands of step s+1 are loaded (per quadrant of 16 MFMAs: four X reads, two W
+// pieces gathered in halves, the codes of the two pieces after those), everything at least 16
+// MFMAs ahead of its use.  A stage is 64 MFMAs per wave.  Its barrier sits behind the first
+// quadrant: the loads of stage+3 (two per quadrant) start right behind it, into the buffer that
+// stage-1 was read from, and the data of stage+1 is read from the second quadrant on.
+constexpr int NPN = 4;                 // W pieces per wave in the narrow tile
+constexpr int WNN = NPN * 16, BNN = 2 * WNN;
+
+template <int VEC, typename CodeT, bool TAIL>
+__global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_t *__restrict__ x,
+                                                                     const CodeT *__restrict__ codes,
+                                                                     const half_t *__restrict__ cb,
+                                                                     half_t *__restrict__ y, int M, int K, int N,
+                                                                     int entries, int rows_per_cb, int tiles_m,
+                                                                     int tiles_n, int cb_lds_count)
+{
+    typedef PrefillCfg<VEC, CodeT> C;
+    constexpr int NS = 4, D = NS - 1;
+    constexpr int NC = C::code_bufs(NS);
+    constexpr int kTile = C::CH * BNN * 16;   // code tile: [chunk][128 rows][16 bytes]
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int kCodeBase = NS * kStageBytes;
+    constexpr int kCbBase = kCodeBase + NC * kTile;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, kg = lane >> 4;
+    const int J = K / VEC;
+    const int cb_bytes = entries * VEC * 2;
+    const uint32_t zero_off = kCbBase + ((cb_lds_count * cb_bytes + 1023) & ~1023);
+
+    int wg = blockIdx.x;
+    const int n_wg = tiles_m * tiles_n;
+    if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+    const int tm = wg / tiles_n, tn = wg % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BNN;
+    const int n_stage = (K + kStageK - 1) / kStageK;
+    const int n_super = (n_stage + C::STAGES - 1) / C::STAGES;
+
+    const int g_first = n0 / rows_per_cb;
+    uint32_t book[NPN];
+    {
+        const int n_base = min(n0 + wn * WNN, N - 1);
+        const int g_base = n_base / rows_per_cb, rem_base = n_base - g_base * rows_per_cb;
+        const float rcp = 1.0f / (float)rows_per_cb;
+#pragma unroll
+        for (int j = 0; j < NPN; j++) {
+            const int n = min(n0 + wn * WNN + j * 16 + r16, N - 1);
+            const int g = g_base + small_div(n - n_base + rem_base, rows_per_cb, rcp);
+            book[j] = kCbBase + (g - g_first) * cb_bytes;
+        }
+    }
+
+    uint32_t x_voff[kChunksPerThread];
+    uint32_t x_voff_tail[TAIL ? kChunksPerThread : 1];
+#pragma unroll
+    for (int i = 0; i < kChunksPerThread; i++) {
+        const int slot = (4 * i + wave) * 64 + lane;
+        const int bank_row = slot >> 4;
+        const int v = (slot & 15) ^ (bank_row & 15);
+        const int row = 2 * bank_row + (v >> 3), cc = v & 7;
+        const int gm = min(m0 + row, M - 1) - m0;
+        x_voff[i] = (uint32_t)(((int64_t)gm * K + cc * 8) * 2);
+        if (TAIL) x_voff_tail[i] = x_voff[i] - (cc >= 4 ? 64u : 0u);
+    }
+    const half_t *x_tile = x + (int64_t)m0 * K;
+    auto issue_x = [&](int i, int buf, int stage) {
+        const bool is_last = stage >= n_stage - 1;
+        const half_t *sbase = x_tile + min(stage, n_stage - 1) * kStageK;
+        uint32_t voff = x_voff[i];
+        if (TAIL) voff = is_last ? x_voff_tail[i] : voff;
+        load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, voff, sbase);
+    };
+    // The code tile has 128 rows, two waves' worth: the waves of the lower half of the tile load
+    // the same chunks to the same place again, which keeps every wave's load count the same.
+    const CodeT *code_tile = codes + (int64_t)n0 * J;
+    const uint32_t code_voff = (uint32_t)(min(wn * 64 + lane, N - 1 - n0) * J * C::CSZ);
+    auto issue_codes = [&](int c, int cbuf, int super) {
+        const bool is_last = super >= n_super - 1;
+        super = min(super, n_super - 1);
+        const int chunk = (TAIL && is_last) ? 0 : c;
+        const uint8_t *sbase = reinterpret_cast<const uint8_t *>(code_tile) + (int64_t)super * (C::K_SUPER / VEC * C::CSZ) + chunk * 16;
+        load_to_lds_16(kCodeBase + cbuf * kTile + c * (BNN * 16) + wn * 1024, code_voff, sbase);
+    };
+
+    float4_t acc[NPN][MP];
+#pragma unroll
+    for (int j = 0; j < NPN; j++)
+#pragma unroll
+        for (int i = 0; i < MP; i++) acc[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    int x_rd[2][2];
+#pragma unroll
+    for (int par = 0; par < 2; par++)
+#pragma unroll
+        for (int s = 0; s < 2; s++) x_rd[par][s] = x_offset(wm * WM + par * 16 + r16, s * 4 + kg);
+    const uint32_t code_rd = kCodeBase + (wn * WNN + r16) * 16 + kg * C::RB;
+
+    // operand set 0 serves MFMA step 0 of a stage, set 1 step 1
+    half4_t wlo[2][NPN], whi[2][NPN];
+    half8_t xp[2][MP];
+    uint32_t cr[2][2];  // codes behind the two W pairs whose gathers come next
+    auto load_x1 = [&](int set, int i, int buf, int s) {
+        xp[set][i] = *reinterpret_cast<const half8_t *>(smem + buf * kStageBytes + x_rd[i & 1][s] + (i >> 1) * 4096);
+    };
+    auto load_c1 = [&](int cset, int j, int cbuf, int t, int s) {
+        const int pos = (t % C::STAGES) * 2 * C::HALF + s * C::HALF;
+        cr[cset][j & 1] = read_codes<C::RB>(smem + code_rd + cbuf * kTile + (pos / 16) * (BNN * 16) + j * 256 + pos % 16);
+    };
+    auto load_w_half = [&](int set, int cset, int j, int h, bool zero) {
+        const half4_t v = gather4<VEC, CodeT, TAIL>(smem, book[j], cr[cset][j & 1], h, zero, zero_off);
+        if (h == 0) wlo[set][j] = v;
+        else whi[set][j] = v;
+    };
+    auto mfma_one = [&](int set, int j, int i) {
+        mfma_in_place(acc[j][i], __builtin_shufflevector(wlo[set][j], whi[set][j], 0, 1, 2, 3, 4, 5, 6, 7), xp[set][i]);
+    };
+
+    // ---- prologue: codebooks, stages 0 and 1, the first six X loads of stage 2 ------------------
+    auto loads_of = [](int stage_mod) constexpr { return kChunksPerThread + (stage_mod % C::STAGES == 0 ? C::CH : 0); };
+    {
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(cb + (int64_t)g_first * entries * VEC);
+        const int n16 = cb_lds_count * cb_bytes / 16;
+        const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
+        for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
+            load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
+    }
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        if (d % C::STAGES == 0) {
+#pragma unroll
+            for (int c = 0; c < C::CH; c++) issue_codes(c, (d / C::STAGES) % NC, d / C::STAGES);
+        }
+#pragma unroll
+        for (int i = 0; i < (d == D - 1 ? 6 : kChunksPerThread); i++) issue_x(i, d, d);
+    }
+    if (tid < 4) reinterpret_cast<uint32_t *>(smem + zero_off)[tid] = 0u;
+    {
+        // stage 0 (and everything older) must have landed
+        constexpr int in_flight = loads_of(1) + loads_of(2) - 2;
+        wait_vmcnt<in_flight>();
+    }
+    __syncthreads();
+
+    int buf = 0, cbuf = 0;
+    // step 0 of stage 0: all of its operands; and the codes of the first W pair of step 1
+#pragma unroll
+    for (int j = 0; j < NPN; j += 2) {
+        load_c1(0, j, cbuf, 0, 0);
+        load_c1(0, j + 1, cbuf, 0, 0);
+        load_w_half(0, 0, j, 0, false);
+        load_w_half(0, 0, j, 1, false);
+        load_w_half(0, 0, j + 1, 0, false);
+        load_w_half(0, 0, j + 1, 1, false);
+    }
+#pragma unroll
+    for (int i = 0; i < MP; i++) load_x1(0, i, buf, 0);
+    load_c1(0, 0, cbuf, 0, 1);
+    load_c1(0, 1, cbuf, 0, 1);
+
+#define VQ_FENCE __builtin_amdgcn_sched_barrier(0)
+    // One quadrant: W pieces 0..3 of operand set `set` against X pieces ih*4.. of the same set.
+    // Between the MFMAs: LX(p) one X read, LW(p) one half of a gather, LC(p) one code read
+    // (p = 0, 2), one X load global->LDS (p = 1, 3), the code tile chunks (p = 0, 2).
+#define VQ_NQUADRANT(set, ih, LX, LW, LC, xi, TGT)                                  \
+    _Pragma("unroll") for (int p_ = 0; p_ < 4; p_++) {                              \
+        mfma_one(set, p_, (ih) * 4 + 0); VQ_FENCE;                                  \
+        LX(p_); VQ_FENCE;                                                           \
+        mfma_one(set, p_, (ih) * 4 + 1); VQ_FENCE;                                  \
+        LW(p_); VQ_FENCE;                                                           \
+        mfma_one(set, p_, (ih) * 4 + 2); VQ_FENCE;                                  \
+        if ((p_ & 1) == 0) { LC(p_ >> 1); VQ_FENCE; }                               \
+        else { issue_x((xi) + (p_ >> 1), TGT##_buf, TGT##_stage); VQ_FENCE; }       \
+        mfma_one(set, p_, (ih) * 4 + 3); VQ_FENCE;                                  \
+        if ((p_ & 1) == 0 && TGT##_codes && (xi) == 0 && (p_ >> 1) < C::CH) {       \
+            issue_codes(p_ >> 1, TGT##_cbuf, TGT##_super); VQ_FENCE;                \
+        }                                                                           \
+    }
+
+    for (int super = 0; super < n_super; super++) {
+        auto stage_body = [&](auto t_const) {
+            constexpr int t = decltype(t_const)::value;
+            const int stage = super * C::STAGES + t;
+            const int buf_next = buf + 1 == NS ? 0 : buf + 1;
+            // first quadrant: X loads 6, 7 of stage+2; the others: X loads 0..5 of stage+3 and its code tile
+            const int tgt_a_buf = (buf + 2) % NS, tgt_a_stage = stage + 2;
+            constexpr bool tgt_a_codes = false;
+            const int tgt_a_cbuf = 0, tgt_a_super = 0;
+            const int tgt_b_buf = buf == 0 ? NS - 1 : buf - 1, tgt_b_stage = stage + D;
+            constexpr bool tgt_b_codes = (t + D) % C::STAGES == 0;
+            constexpr int d_super = (t + D) / C::STAGES;
+            const int tgt_b_super = super + d_super;
+            const int tgt_b_cbuf = (cbuf + d_super) % NC;
+            constexpr bool same_super = t + 1 < C::STAGES;
+            const int cbuf_n = same_super ? cbuf : (cbuf + 1 == NC ? 0 : cbuf + 1);
+            constexpr int t_n = same_super ? t + 1 : 0;
+            const bool no_b = TAIL && stage == n_stage - 1;
+            VQ_FENCE;
+            // step 0 multiplies (set 0); step 1's operands are loaded into set 1
+#define LX_B_LO(p) load_x1(1, (p), buf, 1)
+#define LX_B_HI(p) load_x1(1, 4 + (p), buf, 1)
+#define LW_B_01(p) load_w_half(1, 0, (p) >> 1, (p) & 1, no_b)
+#define LW_B_23(p) load_w_half(1, 1, 2 + ((p) >> 1), (p) & 1, no_b)
+#define LC_B_23(q) load_c1(1, 2 + (q), cbuf, t, 1)
+#define LC_N_01(q) load_c1(0, (q), cbuf_n, t_n, 0)
+            VQ_NQUADRANT(0, 0, LX_B_LO, LW_B_01, LC_B_23, 6, tgt_a);
+            // Publish stage+1: only what stage+2 brings along may still be in flight.
+            wait_vmcnt<loads_of(t + 2)>();
+            __syncthreads();
+            VQ_NQUADRANT(0, 1, LX_B_HI, LW_B_23, LC_N_01, 0, tgt_b);
+            // step 1 multiplies (set 1); the next stage's step 0 operands are loaded into set 0
+#define LX_N_LO(p) load_x1(0, (p), buf_next, 0)
+#define LX_N_HI(p) load_x1(0, 4 + (p), buf_next, 0)
+#define LW_N_01(p) load_w_half(0, 0, (p) >> 1, (p) & 1, false)
+#define LW_N_23(p) load_w_half(0, 1, 2 + ((p) >> 1), (p) & 1, false)
+#define LC_N_23(q) load_c1(1, 2 + (q), cbuf_n, t_n, 0)
+#define LC_NB_01(q) load_c1(0, (q), cbuf_n, t_n, 1)
+            VQ_NQUADRANT(1, 0, LX_N_LO, LW_N_01, LC_N_23, 2, tgt_b);
+            VQ_NQUADRANT(1, 1, LX_N_HI, LW_N_23, LC_NB_01, 4, tgt_b);
+#undef LX_B_LO
+#undef LX_B_HI
+#undef LW_B_01
+#undef LW_B_23
+#undef LC_B_23
+#undef LC_N_01
+#undef LX_N_LO
+#undef LX_N_HI
+#undef LW_N_01
+#undef LW_N_23
+#undef LC_N_23
+#undef LC_NB_01
+            buf = buf_next;
+        };
+        stage_body(std::integral_constant<int, 0>{});
+        if constexpr (C::STAGES == 2) stage_body(std::integral_constant<int, 1>{});
+        cbuf = cbuf + 1 == NC ? 0 : cbuf + 1;
+    }
+#undef VQ_NQUADRANT
+#undef VQ_FENCE
+    wait_vmcnt<0>();
+    __syncthreads();
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its 128x64 wave tile --
+    if ((N & 7) == 0) {
+        constexpr int kPitch = 144;  // 64 fp16 + 16 bytes: rows land in different banks
+        uint8_t *stage_out = smem + wave * (128 * kPitch);
+#pragma unroll
+        for (int i = 0; i < MP; i++)
+#pragma unroll
+            for (int j = 0; j < NPN; j++) {
+                half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
+                *reinterpret_cast<half4_t *>(stage_out + (i * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) = hv;
+            }
+#pragma unroll
+        for (int it = 0; it < 16; it++) {
+            const int row = it * 8 + (lane >> 3), c = lane & 7;
+            const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
+            const int m = m0 + wm * WM + row;
+            const int n = n0 + wn * WNN + c * 8;
+            if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MP; i++) {
+            const int m = m0 + wm * WM + i * 16 + r16;
+            if (m >= M) continue;
+#pragma unroll
+            for (int j = 0; j < NPN; j++) {
+                const int n = n0 + wn * WNN + j * 16 + 4 * kg;
+                half_t *dst = y + (int64_t)m * N + n;
+                if ((N & 3) == 0 && n + 3 < N) {
+                    half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
+                    *reinterpret_cast<half4_t *>(dst) = hv;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < N) dst[e] = (half_t)acc[j][i][e];
+                }
+            }
+        }
+    }
+}
+
 constexpr size_t kLdsLimit = 160 * 1024;
 
-int codebooks_per_tile(const ProblemB &p)
+int codebooks_per_tile(const ProblemB &p, int bn)
 {
-    // Worst case number of codebooks a 256-row band of W touches.
+    // Worst case number of codebooks a band of `bn` rows of W touches.
     int n;
     if (p.n_codebooks == 1) n = 1;
-    else if (p.rows_per_cb >= BN && p.rows_per_cb % BN == 0) n = 1;
-    else if (BN % p.rows_per_cb == 0) n = BN / p.rows_per_cb;
-    else n = (BN + p.rows_per_cb - 1) / p.rows_per_cb + 1;
+    else if (p.rows_per_cb >= bn && p.rows_per_cb % bn == 0) n = 1;
+    else if (bn % p.rows_per_cb == 0) n = bn / p.rows_per_cb;
+    else n = (bn + p.rows_per_cb - 1) / p.rows_per_cb + 1;
     return n < p.n_codebooks ? n : p.n_codebooks;
+}
+
+// codebooks of a tile, padded to the 1 KB steps they are copied in, plus 16 zero bytes
+size_t books_bytes(const ProblemB &p, int bn)
+{
+    return (((size_t)codebooks_per_tile(p, bn) * p.entries * p.vec * 2 + 1023) & ~(size_t)1023) + 16;
 }
 
 template <int VEC, typename CodeT>
 size_t lds_bytes(const ProblemB &p, int n_stages)
 {
     typedef PrefillCfg<VEC, CodeT> C;
-    // X stages, code tiles, codebooks (padded to the 1 KB steps they are copied in), 16 zero bytes
-    const size_t books = ((size_t)codebooks_per_tile(p) * p.entries * p.vec * 2 + 1023) & ~(size_t)1023;
-    return (size_t)n_stages * kStageBytes + (size_t)C::code_bufs(n_stages) * C::kTileBytes + books + 16;
+    return (size_t)n_stages * kStageBytes + (size_t)C::code_bufs(n_stages) * C::kTileBytes + books_bytes(p, BN);
 }
 
 template <int VEC, typename CodeT>
-hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s)
+size_t lds_bytes_narrow(const ProblemB &p)
 {
-    const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-    const int n_cb = codebooks_per_tile(p);
+    typedef PrefillCfg<VEC, CodeT> C;
+    return (size_t)4 * kStageBytes + (size_t)C::code_bufs(4) * C::CH * BNN * 16 + books_bytes(p, BNN);
+}
+
+// Microseconds a launch is expected to take with tiles of `bn` W rows, fitted to measurements: a
+// tile costs 5 us of prologue and epilogue plus K/64 stages of 1.0 us (256x256) or 0.56 us
+// (256x128) when the device is mostly idle, up to 1.6 times that when every compute unit works
+// (the clock the device holds under load); the tiles go over the compute units in rounds.
+double tile_cost_us(const ProblemB &p, int bn)
+{
+    const int64_t tiles = (int64_t)((p.M + BM - 1) / BM) * ((p.N + bn - 1) / bn);
+    const int cus = device_cu_count();
+    const double stages = p.K / 64.0 * (bn == BN ? 1.0 : 0.56);
+    const int64_t full = tiles / cus, rem = tiles % cus;
+    double t = (double)full * (5.0 + stages * 1.6);
+    if (rem) t += 5.0 + stages * (1.0 + 0.6 * (double)rem / cus);
+    return t;
+}
+
+// The narrow tile pays when it brings more compute units to work (fewer 256x256 tiles than units).
+template <int VEC, typename CodeT>
+bool use_narrow_tile(const ProblemB &p)
+{
+    if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return false;
+    return tile_cost_us(p, BNN) < 0.97 * tile_cost_us(p, BN);
+}
+
+template <int VEC, typename CodeT>
+hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
+{
+    const bool tail = (p.K % kStageK) != 0;
+    const int tiles_m = (p.M + BM - 1) / BM;
+    if (tile == 2 || (tile == 0 && use_narrow_tile<VEC, CodeT>(p))) {
+        if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return hipErrorInvalidValue;
+        const int tiles_n = (p.N + BNN - 1) / BNN;
+        const size_t smem = lds_bytes_narrow<VEC, CodeT>(p);
+        auto kern = tail ? prefill_narrow_kernel<VEC, CodeT, true> : prefill_narrow_kernel<VEC, CodeT, false>;
+        hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
+                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb,
+                           tiles_m, tiles_n, codebooks_per_tile(p, BNN));
+        return hipGetLastError();
+    }
+    const int tiles_n = (p.N + BN - 1) / BN;
+    const int n_cb = codebooks_per_tile(p, BN);
     // Four X stages when the codebooks leave room for them, else three; two (every stage then
     // waits for its own loads) only so that very large codebooks still run.
     const int ns = lds_bytes<VEC, CodeT>(p, 4) <= kLdsLimit ? 4 : lds_bytes<VEC, CodeT>(p, 3) <= kLdsLimit ? 3 : 2;
     const size_t smem = lds_bytes<VEC, CodeT>(p, ns);
-    const bool tail = (p.K % kStageK) != 0;
     auto kern = ns == 4   ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
                 : ns == 3 ? (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>)
                           : (tail ? prefill_kernel<VEC, CodeT, true, 2> : prefill_kernel<VEC, CodeT, false, 2>);
@@ -619,29 +955,62 @@ bool prefill_cfg_supports(const ProblemB &p)
            (int64_t)BM * p.K * 2 < ((int64_t)1 << 32);
 }
 
+// what[0]: the kernel serves the shape; what[1]: so does its narrow tile; what[2]: the narrow tile
+// is the one it would choose
+template <int VEC, typename CodeT>
+void prefill_cfg_query(const ProblemB &p, bool (&what)[3])
+{
+    what[0] = prefill_cfg_supports<VEC, CodeT>(p);
+    what[1] = what[0] && lds_bytes_narrow<VEC, CodeT>(p) <= kLdsLimit;
+    what[2] = what[1] && use_narrow_tile<VEC, CodeT>(p);
+}
+
+void prefill_query(const ProblemB &p, bool (&what)[3])
+{
+    what[0] = what[1] = what[2] = false;
+    if (p.M < 1 || p.N < 1 || p.K < 1) return;
+    if (p.vec != 2 && p.vec != 4 && p.vec != 8) return;
+    if (((size_t)p.entries * p.vec * 2) % 16 != 0) return;
+    const bool u8 = p.code_bits == 8;
+    switch (p.vec) {
+    case 8: return u8 ? prefill_cfg_query<8, uint8_t>(p, what) : prefill_cfg_query<8, uint16_t>(p, what);
+    case 4: return u8 ? prefill_cfg_query<4, uint8_t>(p, what) : prefill_cfg_query<4, uint16_t>(p, what);
+    default:
+        if (u8) prefill_cfg_query<2, uint8_t>(p, what);  // 16-bit codes of 2-vectors: generic kernel
+    }
+}
+
 }  // namespace
 
 bool prefill_supports(const ProblemB &p)
 {
-    if (p.M < 1 || p.N < 1 || p.K < 1) return false;
-    if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
-    if (((size_t)p.entries * p.vec * 2) % 16 != 0) return false;
-    const bool u8 = p.code_bits == 8;
-    switch (p.vec) {
-    case 8: return u8 ? prefill_cfg_supports<8, uint8_t>(p) : prefill_cfg_supports<8, uint16_t>(p);
-    case 4: return u8 ? prefill_cfg_supports<4, uint8_t>(p) : prefill_cfg_supports<4, uint16_t>(p);
-    default: return u8 ? prefill_cfg_supports<2, uint8_t>(p) : false;  // 16-bit codes of 2-vectors: generic kernel
-    }
+    bool what[3];
+    prefill_query(p, what);
+    return what[0];
 }
 
-hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s)
+bool prefill_narrow_supports(const ProblemB &p)
+{
+    bool what[3];
+    prefill_query(p, what);
+    return what[1];
+}
+
+double prefill_cost_us(const ProblemB &p)
+{
+    bool what[3];
+    prefill_query(p, what);
+    return tile_cost_us(p, what[2] ? BNN : BN);
+}
+
+hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile)
 {
     if (!prefill_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
-    case 8: return u8 ? launch_prefill_typed<8, uint8_t>(p, s) : launch_prefill_typed<8, uint16_t>(p, s);
-    case 4: return u8 ? launch_prefill_typed<4, uint8_t>(p, s) : launch_prefill_typed<4, uint16_t>(p, s);
-    default: return u8 ? launch_prefill_typed<2, uint8_t>(p, s) : hipErrorInvalidValue;
+    case 8: return u8 ? launch_prefill_typed<8, uint8_t>(p, s, tile) : launch_prefill_typed<8, uint16_t>(p, s, tile);
+    case 4: return u8 ? launch_prefill_typed<4, uint8_t>(p, s, tile) : launch_prefill_typed<4, uint16_t>(p, s, tile);
+    default: return u8 ? launch_prefill_typed<2, uint8_t>(p, s, tile) : hipErrorInvalidValue;
     }
 }
 
