@@ -291,6 +291,34 @@ def test_kmeans_quantiser_feeds_the_gemm_path():
     _check_gemm(y, x, codes, cb, what="quantised weights")
 
 
+def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
+    from vq_gemm_amd.nn import VQLinear
+    g = torch.Generator(device="cpu").manual_seed(12)
+    N, K = 768, 512
+    w = (torch.randn(N, K, generator=g) * 0.05).half().to(DEV)
+    bias = torch.randn(N, generator=g).half().to(DEV)
+    layer = VQLinear.from_float(w, vec=8, entries=256, n_codebooks=3, bias=bias, iters=3, seed=2)
+    _say(layer)
+    assert layer.in_features == K and layer.out_features == N
+    for shape in ((5, K), (2, 7, K), (300, K)):
+        x = torch.randn(*shape, generator=g).half().to(DEV)
+        y = layer(x)
+        torch.cuda.synchronize()
+        assert y.shape == (*shape[:-1], N) and y.dtype == torch.float16
+        wq = _np(layer.dequantized_weight()).astype(np.float64)
+        prod = _np(x).astype(np.float64).reshape(-1, K) @ wq.T
+        ref = prod + _np(bias).astype(np.float64)
+        # the bias is added to the fp16 product (a second rounding): the error is bounded by the
+        # roundings of the product and of the sum, not by the size of a sum that may cancel
+        err = np.abs(_np(y).reshape(-1, N).astype(np.float64) - ref)
+        assert np.all(err <= TOL * (np.abs(prod) + np.abs(ref)) + 1e-4)
+    # the layer survives a state_dict round trip
+    clone = VQLinear(torch.zeros_like(layer.codes), torch.zeros_like(layer.codebook), torch.zeros_like(bias))
+    clone.load_state_dict(layer.state_dict())
+    x = torch.randn(4, K, generator=g).half().to(DEV)
+    assert torch.equal(clone(x), layer(x))
+
+
 def test_every_m_from_1_to_16_on_the_decode_kernel():
     K, N = 1024, 80
     for M in range(1, 17):

@@ -1,0 +1,56 @@
+"""`VQLinear`: a linear layer whose weight is held as codes + codebooks and multiplied by the
+fused VQ GEMM (geometry B), the call site after the path.
+
+Inference only (no gradient flows to codes or codebooks).  The product runs in the HIP library
+through its C ABI; the optional bias is added by torch.  Nothing falls back to the CPU.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import cabi
+from .quantize import kmeans_quantize
+
+
+class VQLinear(torch.nn.Module):
+    """y = x @ W.T + bias with W[n, j*vec + t] = codebook[n // (N/G)][codes[n, j]][t]."""
+
+    def __init__(self, codes: torch.Tensor, codebook: torch.Tensor, bias: torch.Tensor | None = None):
+        super().__init__()
+        if codes.dtype not in (torch.uint8, torch.uint16) or codes.dim() != 2:
+            raise ValueError("codes must be a [N, K/vec] uint8 or uint16 tensor")
+        if codebook.dtype != torch.float16 or codebook.dim() not in (2, 3):
+            raise ValueError("codebook must be an fp16 [E, vec] or [G, E, vec] tensor")
+        self.register_buffer("codes", codes.contiguous())
+        self.register_buffer("codebook", codebook.contiguous())
+        self.register_buffer("bias", None if bias is None else bias.to(torch.float16).contiguous())
+        self.out_features = codes.shape[0]
+        self.in_features = codes.shape[1] * codebook.shape[-1]
+        if self.bias is not None and self.bias.shape != (self.out_features,):
+            raise ValueError("bias must have one entry per output feature")
+
+    @classmethod
+    def from_float(cls, weight: torch.Tensor, vec: int = 8, entries: int = 256, n_codebooks: int = 1,
+                   bias: torch.Tensor | None = None, iters: int = 10, seed: int = 0) -> "VQLinear":
+        """Quantise an fp16 weight [N, K] on the GPU (Lloyd iterations around the HIP encoder)."""
+        codes, codebook, _ = kmeans_quantize(weight.to(torch.float16), vec, entries, n_codebooks, iters, seed)
+        return cls(codes, codebook, bias)
+
+    def dequantized_weight(self) -> torch.Tensor:
+        return cabi.dequant_b(self.codes, self.codebook)
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.dtype != torch.float16 or x.shape[-1] != self.in_features:
+            raise ValueError(f"expected an fp16 input with {self.in_features} features")
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.in_features).contiguous()
+        y = cabi.e2e_gemm_b(x2, self.codes, self.codebook)
+        if self.bias is not None:
+            y += self.bias
+        return y.view(*lead, self.out_features)
+
+    def extra_repr(self) -> str:
+        g = 1 if self.codebook.dim() == 2 else self.codebook.shape[0]
+        return (f"in_features={self.in_features}, out_features={self.out_features}, vec={self.codebook.shape[-1]}, "
+                f"entries={self.codebook.shape[-2]}, codebooks={g}, bias={self.bias is not None}")
