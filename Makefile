@@ -24,8 +24,8 @@ test-gpu:
 
 # rocprofv3 takes the place of the reference's ncu target (reference Makefile:26-28)
 profile:
-	mkdir -p gpurun_out
-	cd /tmp && TMPDIR=/tmp rocprofv3 --kernel-trace --stats --output-format csv -d $(CURDIR)/gpurun_out/prof -o bench -- python3 $(CURDIR)/bench.py
+	mkdir -p build/prof
+	cd /tmp && TMPDIR=/tmp rocprofv3 --kernel-trace --stats --output-format csv -d $(CURDIR)/build/prof -o bench -- python3 $(CURDIR)/bench.py
 
 clean:
 	@rm -rf build vq_gemm_amd/lib oracle/libvq_oracle.so
