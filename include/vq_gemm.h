@@ -57,6 +57,18 @@ int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, vo
                       void *workspace, void *stream);
 
 /*
+ * The same with a bias: Y[m,n] = sum_k X[m,k] W[n,k] + bias[n], bias [N] fp16 (NULL = none), added
+ * to the fp32 sum before the one rounding to fp16.  No counterpart in the reference (its e2e_gemm
+ * has no epilogue); for call sites that hold a linear layer.  VQGEMM_VARIANT_TWOPASS does not take
+ * a bias; the tiled kernels want `bias` 8-byte aligned (the automatic choice falls back to the scalar
+ * kernel otherwise).
+ */
+int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codebook, const void *bias, void *y,
+                           int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                           int32_t n_codebooks, int32_t code_bits, int32_t variant,
+                           void *workspace, void *stream);
+
+/*
  * Fused VQ GEMM, geometry A (reference-native tensors, same entry point of the reference:
  * bind.cpp:3,7; indexing per strategy_2/bsz512/src.cu:163-176 and bench.py:46-56).
  * out is [M, 2*Nc].  `workspace` (K*2*Nc fp16) is required by TWOPASS; VQGEMM_VARIANT_AUTO takes the

@@ -291,6 +291,56 @@ def test_kmeans_quantiser_feeds_the_gemm_path():
     _check_gemm(y, x, codes, cb, what="quantised weights")
 
 
+BIAS_B = [
+    # name, M, K, N, vec, E, bits, G  -- every kernel with a bias input, ragged and aligned shapes
+    ("decode_one_tile", 1, 1024, 64, 8, 256, 8, 1),
+    ("decode_batched_many_tiles", 5, 4096, 8192, 8, 256, 8, 1),
+    ("decode_batched_chunked_k_books", 40, 8192, 2048, 8, 256, 8, 4),
+    ("decode_general_ragged_n", 7, 1024, 50, 8, 256, 8, 1),
+    ("decode_slabs_u16v4", 200, 2048, 2048, 4, 4096, 16, 1),
+    ("prefill_wide_ragged", 1000, 1152, 1000, 8, 256, 8, 5),
+    ("prefill_n_not_mult_of_8", 513, 1024, 1001, 8, 256, 8, 1),
+    ("prefill_narrow_choice", 1024, 1024, 1024, 8, 256, 8, 8),
+    ("prefill_tail32_v2", 512, 1056, 520, 2, 256, 8, 1),
+    ("generic_only_k_odd", 9, 72, 40, 8, 256, 8, 1),
+]
+
+
+@pytest.mark.parametrize("row", BIAS_B, ids=[r[0] for r in BIAS_B])
+def test_bias_is_added_before_the_rounding_in_every_kernel(row):
+    name, M, K, N, v, E, bits, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+    x, codes, cb = make_problem(spec, seed=44, device=DEV)
+    g = torch.Generator(device="cpu").manual_seed(45)
+    bias = torch.randn(N, generator=g).half().to(DEV)
+    # the unrounded product in float64 (the oracle's own GEMM returns it rounded to fp16)
+    w = vo.dequant_b(_np(codes), _np(cb)).astype(np.float64)
+    ref = _np(x).astype(np.float64) @ w.T + _np(bias).astype(np.float64)
+    ran = []
+    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL,
+                    cabi.VARIANT_PREFILL_NARROW):
+        _say("bias", name, cabi.VARIANT_NAMES[variant])
+        try:
+            y = cabi.e2e_gemm_b(x, codes, cb, variant=variant, bias=bias)
+        except cabi.VqGemmError as e:
+            assert e.code == -4 and variant not in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC), e
+            continue
+        torch.cuda.synchronize()
+        e1, e2 = vo.rel_err(_np(y), ref)
+        _say(f"    rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+        assert e1 <= TOL, (name, variant, e1)
+        # a zero bias changes nothing, bit for bit
+        assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=variant, bias=torch.zeros_like(bias)),
+                           cabi.e2e_gemm_b(x, codes, cb, variant=variant))
+        ran.append(variant)
+    assert cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran
+    assert len(ran) >= 3 or name.startswith("generic_only")
+    # the two-pass route has no bias input and says so
+    with pytest.raises(cabi.VqGemmError) as ei:
+        cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_TWOPASS, bias=bias)
+    assert ei.value.code == -4
+
+
 def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
     from vq_gemm_amd.nn import VQLinear
     g = torch.Generator(device="cpu").manual_seed(12)
@@ -306,12 +356,9 @@ def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
         torch.cuda.synchronize()
         assert y.shape == (*shape[:-1], N) and y.dtype == torch.float16
         wq = _np(layer.dequantized_weight()).astype(np.float64)
-        prod = _np(x).astype(np.float64).reshape(-1, K) @ wq.T
-        ref = prod + _np(bias).astype(np.float64)
-        # the bias is added to the fp16 product (a second rounding): the error is bounded by the
-        # roundings of the product and of the sum, not by the size of a sum that may cancel
-        err = np.abs(_np(y).reshape(-1, N).astype(np.float64) - ref)
-        assert np.all(err <= TOL * (np.abs(prod) + np.abs(ref)) + 1e-4)
+        ref = _np(x).astype(np.float64).reshape(-1, K) @ wq.T + _np(bias).astype(np.float64)
+        e1, _ = vo.rel_err(_np(y).reshape(-1, N), ref)
+        assert e1 <= TOL                 # the bias is added to the fp32 sums: still one rounding
     # the layer survives a state_dict round trip
     clone = VQLinear(torch.zeros_like(layer.codes), torch.zeros_like(layer.codebook), torch.zeros_like(bias))
     clone.load_state_dict(layer.state_dict())

@@ -20,6 +20,7 @@ _I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
 
 _SIGNATURES = {
     "vqgemm_e2e_gemm_b": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
+    "vqgemm_e2e_gemm_b_bias": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_a": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _P]),
     "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_dequant_a": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
@@ -93,8 +94,9 @@ def _cb_dims(codebook):
     return codebook.shape[0], codebook.shape[1], codebook.shape[2]
 
 
-def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=None):
-    """Geometry B fused GEMM through the C ABI.  Tensors must be contiguous device tensors."""
+def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=None, bias=None):
+    """Geometry B fused GEMM through the C ABI.  Tensors must be contiguous device tensors.
+    `bias` (fp16 [N]) is added to the fp32 sums inside the kernel."""
     import torch
     M, K = x.shape
     N = codes.shape[0]
@@ -104,8 +106,14 @@ def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=Non
         out = torch.empty((M, N), dtype=torch.float16, device=x.device)
     if variant == VARIANT_TWOPASS and workspace is None:
         workspace = torch.empty((N, K), dtype=torch.float16, device=x.device)
-    rc = lib().vqgemm_e2e_gemm_b(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(out), M, K, N, v, E, G, bits, variant,
-                                 _ptr(workspace), _stream())
+    if bias is None:
+        rc = lib().vqgemm_e2e_gemm_b(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(out), M, K, N, v, E, G, bits, variant,
+                                     _ptr(workspace), _stream())
+    else:
+        if bias.dtype != torch.float16 or bias.shape != (N,):
+            raise ValueError("bias must be an fp16 tensor with one entry per output column")
+        rc = lib().vqgemm_e2e_gemm_b_bias(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(bias), _ptr(out), M, K, N, v, E, G,
+                                          bits, variant, _ptr(workspace), _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_e2e_gemm_b")
     return out

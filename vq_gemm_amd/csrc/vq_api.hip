@@ -64,6 +64,7 @@ ProblemB make_b(const void *x, const void *codes, const void *codebook, void *y,
     p.codes = codes;
     p.cb = static_cast<const half_t *>(codebook);
     p.y = static_cast<half_t *>(y);
+    p.bias = nullptr;
     p.M = (int)M; p.K = (int)K; p.N = (int)N;
     p.vec = vec; p.entries = entries; p.n_codebooks = n_codebooks; p.code_bits = code_bits;
     p.rows_per_cb = N > 0 ? (int)(N / n_codebooks) : 1;
@@ -113,9 +114,9 @@ int vqgemm_select_variant_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_
     return select_b(p, true);
 }
 
-int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, void *y, int64_t M, int64_t K,
-                      int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits,
-                      int32_t variant, void *workspace, void *stream)
+int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codebook, const void *bias, void *y,
+                           int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks,
+                           int32_t code_bits, int32_t variant, void *workspace, void *stream)
 {
     int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
     if (rc != VQGEMM_OK) return rc;
@@ -124,8 +125,11 @@ int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, vo
     if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
     const uintptr_t code_align = code_bits / 8;
     if (!aligned(x, 2) || !aligned(y, 2) || !aligned(codebook, 2) || !aligned(codes, code_align)) return VQGEMM_E_ALIGN;
-    const bool a16 = aligned(x, 16) && aligned(y, 16) && aligned(codebook, 16) && aligned(codes, 16);
-    const ProblemB p = make_b(x, codes, codebook, y, M, K, N, vec, entries, n_codebooks, code_bits);
+    if (!aligned(bias, 2)) return VQGEMM_E_ALIGN;
+    // the tiled kernels read four bias values at a time
+    const bool a16 = aligned(x, 16) && aligned(y, 16) && aligned(codebook, 16) && aligned(codes, 16) && aligned(bias, 8);
+    ProblemB p = make_b(x, codes, codebook, y, M, K, N, vec, entries, n_codebooks, code_bits);
+    p.bias = static_cast<const half_t *>(bias);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (variant == VQGEMM_VARIANT_AUTO) variant = select_b(p, a16);
     hipError_t e = hipSuccess;
@@ -149,6 +153,7 @@ int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, vo
         e = launch_prefill_b(p, s, 2);
         break;
     case VQGEMM_VARIANT_TWOPASS:
+        if (bias) return VQGEMM_E_VARIANT;  // the plain GEMM of the two-pass route has no bias input
         if (!workspace) return VQGEMM_E_NULL;
         if (!aligned(workspace, 16)) return VQGEMM_E_ALIGN;
         e = launch_dequant_b(p, static_cast<half_t *>(workspace), s);
@@ -159,6 +164,14 @@ int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, vo
         return VQGEMM_E_VARIANT;
     }
     return static_cast<int>(e);
+}
+
+int vqgemm_e2e_gemm_b(const void *x, const void *codes, const void *codebook, void *y, int64_t M, int64_t K,
+                      int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits,
+                      int32_t variant, void *workspace, void *stream)
+{
+    return vqgemm_e2e_gemm_b_bias(x, codes, codebook, nullptr, y, M, K, N, vec, entries, n_codebooks, code_bits, variant,
+                                  workspace, stream);
 }
 
 int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *out, int64_t M, int64_t K,

@@ -23,6 +23,7 @@ struct ProblemB {
     const void *codes;    // [N, K/vec] u8 or u16
     const half_t *cb;     // [G, E, vec]
     half_t *y;            // [M,N]
+    const half_t *bias;   // [N] added to the fp32 sums before the rounding to fp16, or nullptr
     int M, K, N;
     int vec, entries, n_codebooks, code_bits;
     int rows_per_cb;      // N / G

@@ -244,8 +244,9 @@ template <int VEC, typename CodeT, bool REPL, int TB>
 __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
                                                                const CodeT *__restrict__ codes,
                                                                const half_t *__restrict__ cb,
-                                                               half_t *__restrict__ y, int m_total, int K, int N,
-                                                               int entries, int n_books, int wgs_per_cb,
+                                                               half_t *__restrict__ y,
+                                                               const half_t *__restrict__ bias, int m_total, int K,
+                                                               int N, int entries, int n_books, int wgs_per_cb,
                                                                int books_per_wg, int tiles_per_cb, int tiles_q,
                                                                int tiles_r, int n_chunks, int red_off,
                                                                int stage_off, int stage_over, int acc_off,
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     typedef LaneCodes<VEC, CodeT> Codes;
     // All kernel arguments are fetched at once: left to first use, each pointer costs the
     // prologue a scalar-load round trip of its own.
-    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(m_total), "s"(K), "s"(N), "s"(entries),
+    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(bias), "s"(m_total), "s"(K), "s"(N), "s"(entries),
                  "s"(n_books), "s"(wgs_per_cb), "s"(books_per_wg), "s"(tiles_per_cb), "s"(tiles_q), "s"(tiles_r),
                  "s"(n_chunks), "s"(red_off), "s"(stage_off), "s"(stage_over), "s"(acc_off), "s"(recip_tail));
     // blockIdx.y picks the 16-row slab of X (and of Y) this workgroup multiplies.
@@ -474,7 +475,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
         }
         // A pass of the reduction: 64 slots, one per lane.  Where the slot goes is worked out
         // first (`locate`), the sum and the store follow (`finish`).
-        struct Target { uint32_t src, carry; half_t *dst; bool live; };  // LDS offsets, output address
+        struct Target { uint32_t src, carry; half_t *dst; int n; bool live; };  // LDS offsets, output address, first W row
         auto locate = [&](int pass) {
             const int slot = pass * 64 + opaque(lane);
             const int jq = (slot * recip_m) >> 16;  // slot / M = j*4 + kq
@@ -485,7 +486,8 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             // with several chunks the sums are carried from chunk to chunk in the LDS, one entry per slot of the range
             t.carry = (uint32_t)acc_off + (uint32_t)(q * n_slots + slot) * 16u;
             // D[i][j] of the tile: the slot holds rows i = 4*kq .. 4*kq+3 of column j = m.
-            t.dst = y + (int64_t)m * N + tile * kTileN + 4 * (jq & 3);
+            t.n = tile * kTileN + 4 * (jq & 3);
+            t.dst = y + (int64_t)m * N + t.n;
             t.live = pass < n_passes && slot < n_slots && tile < tile_end;
             return t;
         };
@@ -510,6 +512,10 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             if (chunk < n_chunks - 1) {
                 *carry = sum;
             } else {
+                if (bias) {
+                    const half4_t b = *reinterpret_cast<const half4_t *>(bias + t.n);
+                    sum += float4_t{(float)b[0], (float)b[1], (float)b[2], (float)b[3]};
+                }
                 half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
                 *reinterpret_cast<half4_t *>(t.dst) = h;
             }
@@ -692,7 +698,7 @@ hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
     if (e != hipSuccess) return e;
     const int tail_rows = p.M - (g.n_slabs - 1) * kTileN;
     hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(g.n_waves * 64), g.smem, s, p.x,
-                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.n_codebooks,
+                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.n_codebooks,
                        g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, g.tiles_per_cb / g.wgs_per_cb,
                        g.tiles_per_cb % g.wgs_per_cb, g.n_chunks, g.red_off, g.stage_off, g.stage_over, g.acc_off,
                        (65536 + tail_rows - 1) / tail_rows);

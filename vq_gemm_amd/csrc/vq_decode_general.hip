@@ -111,7 +111,8 @@ template <int VEC, typename CodeT, int STEPS, bool REPL>
 __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__restrict__ x,
                                                       const CodeT *__restrict__ codes,
                                                       const half_t *__restrict__ cb,
-                                                      half_t *__restrict__ y, int M, int K, int N,
+                                                      half_t *__restrict__ y,
+                                                      const half_t *__restrict__ bias, int M, int K, int N,
                                                       int entries, int rows_per_cb, int tiles_q,
                                                       int tiles_r, int n_chunks, int stage_off,
                                                       int aliased)
@@ -322,6 +323,10 @@ __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__res
                 // D[i][j]: j = lane % 16 is the X row m, i = 4*(lane/16) + r is the W row.
                 const int m = r16;
                 const int n = tile * kTileN + 4 * kq;
+                if (bias) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) sum[r] += n + r < N ? (float)bias[n + r] : 0.f;
+                }
                 if (m < M) {
                     half_t *dst = y + (int64_t)m * N + n;
                     if ((N & 3) == 0 && n + 3 < N) {
@@ -387,7 +392,7 @@ hipError_t launch_decode_steps(const ProblemB &p, hipStream_t s)
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
-                       p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb, n_tiles / grid, n_tiles % grid, n_chunks, stage_off, aliased);
+                       p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb, n_tiles / grid, n_tiles % grid, n_chunks, stage_off, aliased);
     return hipGetLastError();
 }
 

@@ -10,7 +10,8 @@ template <typename CodeT>
 __global__ __launch_bounds__(256) void generic_b_kernel(const half_t *__restrict__ x,
                                                         const CodeT *__restrict__ codes,
                                                         const half_t *__restrict__ cb,
-                                                        half_t *__restrict__ y, int M, int K, int N,
+                                                        half_t *__restrict__ y,
+                                                        const half_t *__restrict__ bias, int M, int K, int N,
                                                         int vec, int entries, int rows_per_cb)
 {
     // blockDim = (64, 4): x index -> n (coalesced y stores), y index -> m.
@@ -19,6 +20,7 @@ __global__ __launch_bounds__(256) void generic_b_kernel(const half_t *__restrict
     const int J = K / vec;
     const half_t *book = cb + (int64_t)(n / rows_per_cb) * entries * vec;
     const CodeT *crow = codes + (int64_t)n * J;
+    const float b = bias ? (float)bias[n] : 0.0f;
     for (int m = blockIdx.y * blockDim.y + threadIdx.y; m < M; m += gridDim.y * blockDim.y) {
         const half_t *xrow = x + (int64_t)m * K;
         float acc = 0.0f;
@@ -28,7 +30,7 @@ __global__ __launch_bounds__(256) void generic_b_kernel(const half_t *__restrict
             const half_t *cw = book + (int64_t)c * vec;
             for (int t = 0; t < vec; t++) acc += (float)xrow[j * vec + t] * (float)cw[t];
         }
-        y[(int64_t)m * N + n] = (half_t)acc;
+        y[(int64_t)m * N + n] = (half_t)(acc + b);
     }
 }
 
@@ -39,10 +41,10 @@ hipError_t launch_generic_b(const ProblemB &p, hipStream_t s)
     dim3 grid((p.N + 63) / 64, (unsigned)(((p.M + 3) / 4) < 32768 ? (p.M + 3) / 4 : 32768));
     if (p.code_bits == 8)
         hipLaunchKernelGGL((generic_b_kernel<uint8_t>), grid, block, 0, s, p.x, static_cast<const uint8_t *>(p.codes),
-                           p.cb, p.y, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
+                           p.cb, p.y, p.bias, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
     else
         hipLaunchKernelGGL((generic_b_kernel<uint16_t>), grid, block, 0, s, p.x, static_cast<const uint16_t *>(p.codes),
-                           p.cb, p.y, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
+                           p.cb, p.y, p.bias, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
     return hipGetLastError();
 }
 

@@ -103,6 +103,16 @@ __device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, c
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
+// The four fp32 sums of an accumulator rounded to fp16, with the bias of their columns added first.
+template <bool HAS_BIAS>
+__device__ __forceinline__ half4_t round4(const float4_t &a, const float (&b)[4])
+{
+    if constexpr (HAS_BIAS)
+        return half4_t{(half_t)(a[0] + b[0]), (half_t)(a[1] + b[1]), (half_t)(a[2] + b[2]), (half_t)(a[3] + b[3])};
+    else
+        return half4_t{(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]};
+}
+
 // floor(x / d) for 0 <= x and a quotient small enough that float rounding stays within one
 // (here: x < d + 256); `rcp` = 1.0f / d.
 __device__ __forceinline__ int small_div(int x, int d, float rcp)
@@ -154,7 +164,8 @@ template <int VEC, typename CodeT, bool TAIL, int NS>
 __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__restrict__ x,
                                                               const CodeT *__restrict__ codes,
                                                               const half_t *__restrict__ cb,
-                                                              half_t *__restrict__ y, int M, int K, int N,
+                                                              half_t *__restrict__ y,
+                                                              const half_t *__restrict__ bias, int M, int K, int N,
                                                               int entries, int rows_per_cb, int tiles_m,
                                                               int tiles_n, int cb_lds_count)
 {
@@ -520,51 +531,63 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     // the last MFMAs must have left the pipe before the accumulators are read
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its wave tile ------
-    if ((N & 7) == 0) {
-        // Through the LDS: each wave transposes its 128x128 fp16 block, 64 rows at a time, in a
-        // private region (row pitch 272 bytes) and stores 256-byte row segments.
-        constexpr int kPitch = 272;
-        uint8_t *stage_out = smem + wave * (64 * kPitch);
+    auto epilogue = [&](auto has_bias_const) {
+        constexpr bool HB = decltype(has_bias_const)::value;
+        float bj[NP][4];
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
+        for (int j = 0; j < NP; j++)
 #pragma unroll
-            for (int ii = 0; ii < 4; ii++) {
-                const int i = 4 * h + ii;
+            for (int e = 0; e < 4; e++) {
+                const int n = n0 + wn * WN + j * 16 + 4 * kg + e;
+                bj[j][e] = HB && n < N ? (float)bias[n] : 0.f;
+            }
+        if ((N & 7) == 0) {
+            // Through the LDS: each wave transposes its 128x128 fp16 block, 64 rows at a time, in a
+            // private region (row pitch 272 bytes) and stores 256-byte row segments.
+            constexpr int kPitch = 272;
+            uint8_t *stage_out = smem + wave * (64 * kPitch);
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+#pragma unroll
+                for (int ii = 0; ii < 4; ii++) {
+                    const int i = 4 * h + ii;
+#pragma unroll
+                    for (int j = 0; j < NP; j++)
+                        *reinterpret_cast<half4_t *>(stage_out + (ii * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) =
+                            round4<HB>(acc[j][i], bj[j]);
+                }
+#pragma unroll
+                for (int it = 0; it < 16; it++) {
+                    const int row = it * 4 + (lane >> 4), c = lane & 15;
+                    const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
+                    const int m = m0 + wm * WM + h * 64 + row;
+                    const int n = n0 + wn * WN + c * 8;
+                    if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < MP; i++) {
+                const int m = m0 + wm * WM + i * 16 + r16;
+                if (m >= M) continue;
 #pragma unroll
                 for (int j = 0; j < NP; j++) {
-                    half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
-                    *reinterpret_cast<half4_t *>(stage_out + (ii * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) = hv;
-                }
-            }
+                    const int n = n0 + wn * WN + j * 16 + 4 * kg;
+                    half_t *dst = y + (int64_t)m * N + n;
+                    const half4_t hv = round4<HB>(acc[j][i], bj[j]);
+                    if ((N & 3) == 0 && n + 3 < N) {
+                        *reinterpret_cast<half4_t *>(dst) = hv;
+                    } else {
 #pragma unroll
-            for (int it = 0; it < 16; it++) {
-                const int row = it * 4 + (lane >> 4), c = lane & 15;
-                const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
-                const int m = m0 + wm * WM + h * 64 + row;
-                const int n = n0 + wn * WN + c * 8;
-                if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
-            }
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < MP; i++) {
-            const int m = m0 + wm * WM + i * 16 + r16;
-            if (m >= M) continue;
-#pragma unroll
-            for (int j = 0; j < NP; j++) {
-                const int n = n0 + wn * WN + j * 16 + 4 * kg;
-                half_t *dst = y + (int64_t)m * N + n;
-                if ((N & 3) == 0 && n + 3 < N) {
-                    half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
-                    *reinterpret_cast<half4_t *>(dst) = hv;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = (half_t)acc[j][i][e];
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < N) dst[e] = hv[e];
+                    }
                 }
             }
         }
-    }
+    };
+    if (bias) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
 }
 
 // ---- the 256x128 tile ------------------------------------------------------------------------
@@ -584,8 +607,9 @@ template <int VEC, typename CodeT, bool TAIL>
 __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_t *__restrict__ x,
                                                                      const CodeT *__restrict__ codes,
                                                                      const half_t *__restrict__ cb,
-                                                                     half_t *__restrict__ y, int M, int K, int N,
-                                                                     int entries, int rows_per_cb, int tiles_m,
+                                                                     half_t *__restrict__ y,
+                                                                     const half_t *__restrict__ bias, int M, int K,
+                                                                     int N, int entries, int rows_per_cb, int tiles_m,
                                                                      int tiles_n, int cb_lds_count)
 {
     typedef PrefillCfg<VEC, CodeT> C;
@@ -816,44 +840,56 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its 128x64 wave tile --
-    if ((N & 7) == 0) {
-        constexpr int kPitch = 144;  // 64 fp16 + 16 bytes: rows land in different banks
-        uint8_t *stage_out = smem + wave * (128 * kPitch);
+    auto epilogue = [&](auto has_bias_const) {
+        constexpr bool HB = decltype(has_bias_const)::value;
+        float bj[NPN][4];
 #pragma unroll
-        for (int i = 0; i < MP; i++)
+        for (int j = 0; j < NPN; j++)
 #pragma unroll
-            for (int j = 0; j < NPN; j++) {
-                half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
-                *reinterpret_cast<half4_t *>(stage_out + (i * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) = hv;
+            for (int e = 0; e < 4; e++) {
+                const int n = n0 + wn * WNN + j * 16 + 4 * kg + e;
+                bj[j][e] = HB && n < N ? (float)bias[n] : 0.f;
             }
+        if ((N & 7) == 0) {
+            constexpr int kPitch = 144;  // 64 fp16 + 16 bytes: rows land in different banks
+            uint8_t *stage_out = smem + wave * (128 * kPitch);
 #pragma unroll
-        for (int it = 0; it < 16; it++) {
-            const int row = it * 8 + (lane >> 3), c = lane & 7;
-            const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
-            const int m = m0 + wm * WM + row;
-            const int n = n0 + wn * WNN + c * 8;
-            if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
-        }
-    } else {
+            for (int i = 0; i < MP; i++)
 #pragma unroll
-        for (int i = 0; i < MP; i++) {
-            const int m = m0 + wm * WM + i * 16 + r16;
-            if (m >= M) continue;
+                for (int j = 0; j < NPN; j++)
+                    *reinterpret_cast<half4_t *>(stage_out + (i * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) =
+                        round4<HB>(acc[j][i], bj[j]);
 #pragma unroll
-            for (int j = 0; j < NPN; j++) {
-                const int n = n0 + wn * WNN + j * 16 + 4 * kg;
-                half_t *dst = y + (int64_t)m * N + n;
-                if ((N & 3) == 0 && n + 3 < N) {
-                    half4_t hv = {(half_t)acc[j][i][0], (half_t)acc[j][i][1], (half_t)acc[j][i][2], (half_t)acc[j][i][3]};
-                    *reinterpret_cast<half4_t *>(dst) = hv;
-                } else {
+            for (int it = 0; it < 16; it++) {
+                const int row = it * 8 + (lane >> 3), c = lane & 7;
+                const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
+                const int m = m0 + wm * WM + row;
+                const int n = n0 + wn * WNN + c * 8;
+                if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
+            }
+        } else {
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < N) dst[e] = (half_t)acc[j][i][e];
+            for (int i = 0; i < MP; i++) {
+                const int m = m0 + wm * WM + i * 16 + r16;
+                if (m >= M) continue;
+#pragma unroll
+                for (int j = 0; j < NPN; j++) {
+                    const int n = n0 + wn * WNN + j * 16 + 4 * kg;
+                    half_t *dst = y + (int64_t)m * N + n;
+                    const half4_t hv = round4<HB>(acc[j][i], bj[j]);
+                    if ((N & 3) == 0 && n + 3 < N) {
+                        *reinterpret_cast<half4_t *>(dst) = hv;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (n + e < N) dst[e] = hv[e];
+                    }
                 }
             }
         }
-    }
+    };
+    if (bias) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
 }
 
 constexpr size_t kLdsLimit = 160 * 1024;
@@ -925,7 +961,7 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
-                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb,
+                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
                            tiles_m, tiles_n, codebooks_per_tile(p, BNN));
         return hipGetLastError();
     }
@@ -941,7 +977,7 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
-                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.rows_per_cb,
+                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
                        tiles_m, tiles_n, n_cb);
     return hipGetLastError();
 }

@@ -2,7 +2,8 @@
 fused VQ GEMM (geometry B), the call site after the path.
 
 Inference only (no gradient flows to codes or codebooks).  The product runs in the HIP library
-through its C ABI; the optional bias is added by torch.  Nothing falls back to the CPU.
+through its C ABI, the optional bias is added inside the kernel before the result is rounded.
+Nothing falls back to the CPU.
 """
 from __future__ import annotations
 
@@ -45,9 +46,7 @@ class VQLinear(torch.nn.Module):
             raise ValueError(f"expected an fp16 input with {self.in_features} features")
         lead = x.shape[:-1]
         x2 = x.reshape(-1, self.in_features).contiguous()
-        y = cabi.e2e_gemm_b(x2, self.codes, self.codebook)
-        if self.bias is not None:
-            y += self.bias
+        y = cabi.e2e_gemm_b(x2, self.codes, self.codebook, bias=self.bias)
         return y.view(*lead, self.out_features)
 
     def extra_repr(self) -> str:
