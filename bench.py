@@ -56,6 +56,21 @@ def parse_args():
     return ap.parse_args()
 
 
+def mfma_ceiling_tflops():
+    """TFLOP/s of the register-only v_mfma_f32_16x16x32_f16 loop with random operands (None if the tool is not built)."""
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vq_gemm_amd", "lib", "mfma_ceiling")
+    if not os.path.exists(exe):
+        return None
+    try:
+        text = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=60).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    m = re.search(r"random operands, v_mfma_f32_16x16x32_f16: [\d.]+ us per launch, (\d+) TFLOP/s", text)
+    return float(m.group(1)) if m else None
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -252,6 +267,15 @@ def main():
         "deterministic_5_runs": main_res["deterministic_5_runs"],
         "other_configs": others,
     }
+    if others:
+        # what the matrix cores sustain on this device with random operands (register-only MFMA loop):
+        # the ceiling the MFMA-bound configurations are to be read against, next to the nominal peak
+        ceiling = mfma_ceiling_tflops()
+        if ceiling:
+            out["mfma_ceiling_random_operands_tflops"] = ceiling
+            for res in others.values():
+                if res["variant"].startswith("prefill"):
+                    res["frac_of_mfma_ceiling"] = res["tflops"] / ceiling
     print(json.dumps(out))
 
 
