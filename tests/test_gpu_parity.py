@@ -199,6 +199,8 @@ PREFILL_B = [
     ("u8v2_tail32_ragged_n", 512, 1056, 520, 2, 256, 8, 1),
     ("u8v2_k32_only_a_tail", 260, 32, 264, 2, 256, 8, 1),
     ("u8v8_many_tiles", 2048, 2048, 4096, 8, 256, 8, 16),
+    # more 256x256 tiles than a 256-CU device has units: whole rounds of them, the left-over columns in 256x128 tiles
+    ("u8v8_rounds_and_a_narrow_tail", 2048, 256, 8704, 8, 256, 8, 17),
 ]
 
 

@@ -166,9 +166,11 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                                                               const half_t *__restrict__ cb,
                                                               half_t *__restrict__ y,
                                                               const half_t *__restrict__ bias, int M, int K, int N,
-                                                              int entries, int rows_per_cb, int tiles_m,
-                                                              int tiles_n, int cb_lds_count)
+                                                              int n_begin, int ldn, int entries, int rows_per_cb,
+                                                              int tiles_m, int tiles_n, int cb_lds_count)
 {
+    // The launch covers the W rows (columns of Y) [n_begin, N) of a problem with ldn rows in all:
+    // ldn is the row stride of Y and counts the codebooks, N bounds the rows that are touched.
     typedef PrefillCfg<VEC, CodeT> C;
     static_assert(NS >= 2 && NS <= 4, "two to four X stages");
     constexpr int D = NS - 1;                 // loads run D stages ahead of the MFMAs
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     const int n_wg = tiles_m * tiles_n;
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
     const int tm = wg / tiles_n, tn = wg % tiles_n;
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = n_begin + tn * BN;
     const int n_stage = (K + kStageK - 1) / kStageK;
     const int n_super = (n_stage + C::STAGES - 1) / C::STAGES;
 
@@ -302,7 +304,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     {
         const uint8_t *src = reinterpret_cast<const uint8_t *>(cb + (int64_t)g_first * entries * VEC);
         const int n16 = cb_lds_count * cb_bytes / 16;
-        const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
+        const int g_total_16 = (int)(((int64_t)((ldn + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
         // past the last codebook: read its last 16 bytes again
         for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
             load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
@@ -541,7 +543,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                 const int n = n0 + wn * WN + j * 16 + 4 * kg + e;
                 bj[j][e] = HB && n < N ? (float)bias[n] : 0.f;
             }
-        if ((N & 7) == 0) {
+        if ((ldn & 7) == 0) {
             // Through the LDS: each wave transposes its 128x128 fp16 block, 64 rows at a time, in a
             // private region (row pitch 272 bytes) and stores 256-byte row segments.
             constexpr int kPitch = 272;
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                     const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
                     const int m = m0 + wm * WM + h * 64 + row;
                     const int n = n0 + wn * WN + c * 8;
-                    if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
+                    if (m < M && n < N) st_global_16(y + (int64_t)m * ldn + n, v);
                 }
             }
         } else {
@@ -573,9 +575,9 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
 #pragma unroll
                 for (int j = 0; j < NP; j++) {
                     const int n = n0 + wn * WN + j * 16 + 4 * kg;
-                    half_t *dst = y + (int64_t)m * N + n;
+                    half_t *dst = y + (int64_t)m * ldn + n;
                     const half4_t hv = round4<HB>(acc[j][i], bj[j]);
-                    if ((N & 3) == 0 && n + 3 < N) {
+                    if ((ldn & 3) == 0 && n + 3 < N) {
                         *reinterpret_cast<half4_t *>(dst) = hv;
                     } else {
 #pragma unroll
@@ -609,8 +611,9 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
                                                                      const half_t *__restrict__ cb,
                                                                      half_t *__restrict__ y,
                                                                      const half_t *__restrict__ bias, int M, int K,
-                                                                     int N, int entries, int rows_per_cb, int tiles_m,
-                                                                     int tiles_n, int cb_lds_count)
+                                                                     int N, int n_begin, int ldn, int entries,
+                                                                     int rows_per_cb, int tiles_m, int tiles_n,
+                                                                     int cb_lds_count)
 {
     typedef PrefillCfg<VEC, CodeT> C;
     constexpr int NS = 4, D = NS - 1;
@@ -631,7 +634,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
     const int n_wg = tiles_m * tiles_n;
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
     const int tm = wg / tiles_n, tn = wg % tiles_n;
-    const int m0 = tm * BM, n0 = tn * BNN;
+    const int m0 = tm * BM, n0 = n_begin + tn * BNN;
     const int n_stage = (K + kStageK - 1) / kStageK;
     const int n_super = (n_stage + C::STAGES - 1) / C::STAGES;
 
@@ -719,7 +722,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
     {
         const uint8_t *src = reinterpret_cast<const uint8_t *>(cb + (int64_t)g_first * entries * VEC);
         const int n16 = cb_lds_count * cb_bytes / 16;
-        const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
+        const int g_total_16 = (int)(((int64_t)((ldn + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
         for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
             load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
     }
@@ -850,7 +853,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
                 const int n = n0 + wn * WNN + j * 16 + 4 * kg + e;
                 bj[j][e] = HB && n < N ? (float)bias[n] : 0.f;
             }
-        if ((N & 7) == 0) {
+        if ((ldn & 7) == 0) {
             constexpr int kPitch = 144;  // 64 fp16 + 16 bytes: rows land in different banks
             uint8_t *stage_out = smem + wave * (128 * kPitch);
 #pragma unroll
@@ -865,7 +868,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
                 const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
                 const int m = m0 + wm * WM + row;
                 const int n = n0 + wn * WNN + c * 8;
-                if (m < M && n < N) st_global_16(y + (int64_t)m * N + n, v);
+                if (m < M && n < N) st_global_16(y + (int64_t)m * ldn + n, v);
             }
         } else {
 #pragma unroll
@@ -875,9 +878,9 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
 #pragma unroll
                 for (int j = 0; j < NPN; j++) {
                     const int n = n0 + wn * WNN + j * 16 + 4 * kg;
-                    half_t *dst = y + (int64_t)m * N + n;
+                    half_t *dst = y + (int64_t)m * ldn + n;
                     const half4_t hv = round4<HB>(acc[j][i], bj[j]);
-                    if ((N & 3) == 0 && n + 3 < N) {
+                    if ((ldn & 3) == 0 && n + 3 < N) {
                         *reinterpret_cast<half4_t *>(dst) = hv;
                     } else {
 #pragma unroll
@@ -925,13 +928,13 @@ size_t lds_bytes_narrow(const ProblemB &p)
     return (size_t)4 * kStageBytes + (size_t)C::code_bufs(4) * C::CH * BNN * 16 + books_bytes(p, BNN);
 }
 
-// Microseconds a launch is expected to take with tiles of `bn` W rows, fitted to measurements: a
-// tile costs 5 us of prologue and epilogue plus K/64 stages of 1.0 us (256x256) or 0.56 us
-// (256x128) when the device is mostly idle, up to 1.6 times that when every compute unit works
-// (the clock the device holds under load); the tiles go over the compute units in rounds.
-double tile_cost_us(const ProblemB &p, int bn)
+// Microseconds a launch over `cols` tile columns of `bn` W rows is expected to take, fitted to
+// measurements: a tile costs 5 us of prologue and epilogue plus K/64 stages of 1.0 us (256x256) or
+// 0.56 us (256x128) when the device is mostly idle, up to 1.6 times that when every compute unit
+// works (the clock the device holds under load); the tiles go over the compute units in rounds.
+double tile_cost_us(const ProblemB &p, int bn, int cols)
 {
-    const int64_t tiles = (int64_t)((p.M + BM - 1) / BM) * ((p.N + bn - 1) / bn);
+    const int64_t tiles = (int64_t)((p.M + BM - 1) / BM) * cols;
     const int cus = device_cu_count();
     const double stages = p.K / 64.0 * (bn == BN ? 1.0 : 0.56);
     const int64_t full = tiles / cus, rem = tiles % cus;
@@ -940,46 +943,75 @@ double tile_cost_us(const ProblemB &p, int bn)
     return t;
 }
 
-// The narrow tile pays when it brings more compute units to work (fewer 256x256 tiles than units).
+// How a launch is cut into tiles: W rows [0, n_split) in 256x256 tiles, [n_split, N) in 256x128
+// tiles (either part may be empty).  The narrow tile pays when it brings more compute units to
+// work: for the whole problem when its 256x256 tiles are fewer than the units, or for the columns
+// left over after whole rounds of 256x256 tiles (two launches then).
+struct TilePlan {
+    int n_split;
+    double cost_us;
+};
+
 template <int VEC, typename CodeT>
-bool use_narrow_tile(const ProblemB &p)
+TilePlan plan_tiles(const ProblemB &p)
 {
-    if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return false;
-    return tile_cost_us(p, BNN) < 0.97 * tile_cost_us(p, BN);
+    const int cols_wide = (p.N + BN - 1) / BN, cols_narrow = (p.N + BNN - 1) / BNN;
+    TilePlan best = {p.N, tile_cost_us(p, BN, cols_wide)};
+    if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return best;
+    const double all_narrow = tile_cost_us(p, BNN, cols_narrow);
+    if (all_narrow < 0.97 * best.cost_us) best = {0, all_narrow};
+    // whole rounds of wide tiles, the rest narrow
+    const int tiles_m = (p.M + BM - 1) / BM, cus = device_cu_count();
+    const int64_t rounds = (int64_t)tiles_m * cols_wide / cus;
+    const int cols_head = (int)(rounds * cus / tiles_m);
+    if (rounds >= 1 && cols_head >= 1 && cols_head < cols_wide) {
+        const int n_split = cols_head * BN;
+        const double t = tile_cost_us(p, BN, cols_head) + tile_cost_us(p, BNN, (p.N - n_split + BNN - 1) / BNN) + 3.0;
+        if (t < 0.97 * best.cost_us) best = {n_split, t};
+    }
+    return best;
 }
 
+// tile: 0 = as planned, 1 = 256x256 only, 2 = 256x128 only
 template <int VEC, typename CodeT>
 hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
 {
     const bool tail = (p.K % kStageK) != 0;
     const int tiles_m = (p.M + BM - 1) / BM;
-    if (tile == 2 || (tile == 0 && use_narrow_tile<VEC, CodeT>(p))) {
+    int n_split = p.N;
+    if (tile == 2) n_split = 0;
+    else if (tile == 0) n_split = plan_tiles<VEC, CodeT>(p).n_split;
+    if (n_split > 0) {
+        const int tiles_n = (n_split + BN - 1) / BN;
+        const int n_cb = codebooks_per_tile(p, BN);
+        // Four X stages when the codebooks leave room for them, else three; two (every stage then
+        // waits for its own loads) only so that very large codebooks still run.
+        const int ns = lds_bytes<VEC, CodeT>(p, 4) <= kLdsLimit ? 4 : lds_bytes<VEC, CodeT>(p, 3) <= kLdsLimit ? 3 : 2;
+        const size_t smem = lds_bytes<VEC, CodeT>(p, ns);
+        auto kern = ns == 4   ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
+                    : ns == 3 ? (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>)
+                              : (tail ? prefill_kernel<VEC, CodeT, true, 2> : prefill_kernel<VEC, CodeT, false, 2>);
+        hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
+                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, n_split, 0, p.N, p.entries,
+                           p.rows_per_cb, tiles_m, tiles_n, n_cb);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (n_split < p.N) {
         if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return hipErrorInvalidValue;
-        const int tiles_n = (p.N + BNN - 1) / BNN;
+        const int tiles_n = (p.N - n_split + BNN - 1) / BNN;
         const size_t smem = lds_bytes_narrow<VEC, CodeT>(p);
         auto kern = tail ? prefill_narrow_kernel<VEC, CodeT, true> : prefill_narrow_kernel<VEC, CodeT, false>;
         hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
-                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
-                           tiles_m, tiles_n, codebooks_per_tile(p, BNN));
+                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, n_split, p.N, p.entries,
+                           p.rows_per_cb, tiles_m, tiles_n, codebooks_per_tile(p, BNN));
         return hipGetLastError();
     }
-    const int tiles_n = (p.N + BN - 1) / BN;
-    const int n_cb = codebooks_per_tile(p, BN);
-    // Four X stages when the codebooks leave room for them, else three; two (every stage then
-    // waits for its own loads) only so that very large codebooks still run.
-    const int ns = lds_bytes<VEC, CodeT>(p, 4) <= kLdsLimit ? 4 : lds_bytes<VEC, CodeT>(p, 3) <= kLdsLimit ? 3 : 2;
-    const size_t smem = lds_bytes<VEC, CodeT>(p, ns);
-    auto kern = ns == 4   ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
-                : ns == 3 ? (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>)
-                          : (tail ? prefill_kernel<VEC, CodeT, true, 2> : prefill_kernel<VEC, CodeT, false, 2>);
-    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
-                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
-                       tiles_m, tiles_n, n_cb);
-    return hipGetLastError();
+    return hipSuccess;
 }
 
 template <int VEC, typename CodeT>
@@ -991,19 +1023,24 @@ bool prefill_cfg_supports(const ProblemB &p)
            (int64_t)BM * p.K * 2 < ((int64_t)1 << 32);
 }
 
-// what[0]: the kernel serves the shape; what[1]: so does its narrow tile; what[2]: the narrow tile
-// is the one it would choose
+// wide: the kernel serves the shape; narrow: so does its narrow tile; cost_us: expected time of
+// the launch as it would be cut into tiles
+struct PrefillQuery {
+    bool wide, narrow;
+    double cost_us;
+};
+
 template <int VEC, typename CodeT>
-void prefill_cfg_query(const ProblemB &p, bool (&what)[3])
+void prefill_cfg_query(const ProblemB &p, PrefillQuery &what)
 {
-    what[0] = prefill_cfg_supports<VEC, CodeT>(p);
-    what[1] = what[0] && lds_bytes_narrow<VEC, CodeT>(p) <= kLdsLimit;
-    what[2] = what[1] && use_narrow_tile<VEC, CodeT>(p);
+    what.wide = prefill_cfg_supports<VEC, CodeT>(p);
+    what.narrow = what.wide && lds_bytes_narrow<VEC, CodeT>(p) <= kLdsLimit;
+    what.cost_us = what.wide ? plan_tiles<VEC, CodeT>(p).cost_us : 1e30;
 }
 
-void prefill_query(const ProblemB &p, bool (&what)[3])
+void prefill_query(const ProblemB &p, PrefillQuery &what)
 {
-    what[0] = what[1] = what[2] = false;
+    what = {false, false, 1e30};
     if (p.M < 1 || p.N < 1 || p.K < 1) return;
     if (p.vec != 2 && p.vec != 4 && p.vec != 8) return;
     if (((size_t)p.entries * p.vec * 2) % 16 != 0) return;
@@ -1020,23 +1057,23 @@ void prefill_query(const ProblemB &p, bool (&what)[3])
 
 bool prefill_supports(const ProblemB &p)
 {
-    bool what[3];
+    PrefillQuery what;
     prefill_query(p, what);
-    return what[0];
+    return what.wide;
 }
 
 bool prefill_narrow_supports(const ProblemB &p)
 {
-    bool what[3];
+    PrefillQuery what;
     prefill_query(p, what);
-    return what[1];
+    return what.narrow;
 }
 
 double prefill_cost_us(const ProblemB &p)
 {
-    bool what[3];
+    PrefillQuery what;
     prefill_query(p, what);
-    return tile_cost_us(p, what[2] ? BNN : BN);
+    return what.cost_us;
 }
 
 hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile)
