@@ -103,6 +103,14 @@ __device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, c
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
+// 16-byte store of a result that this kernel does not read again: the non-temporal hint lets the
+// write leave the L2 as it is issued instead of waiting for the write-back at the end of the kernel
+// (all workgroups of a round finish at about the same time).
+__device__ __forceinline__ void st_global_16_streaming(void *p, uint4_t v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(p));
+}
+
 // The four fp32 sums of an accumulator rounded to fp16, with the bias of their columns added first.
 template <bool HAS_BIAS>
 __device__ __forceinline__ half4_t round4(const float4_t &a, const float (&b)[4])
@@ -564,7 +572,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                     const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
                     const int m = m0 + wm * WM + h * 64 + row;
                     const int n = n0 + wn * WN + c * 8;
-                    if (m < M && n < N) st_global_16(y + (int64_t)m * ldn + n, v);
+                    if (m < M && n < N) st_global_16_streaming(y + (int64_t)m * ldn + n, v);
                 }
             }
         } else {
@@ -868,7 +876,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
                 const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
                 const int m = m0 + wm * WM + row;
                 const int n = n0 + wn * WNN + c * 8;
-                if (m < M && n < N) st_global_16(y + (int64_t)m * ldn + n, v);
+                if (m < M && n < N) st_global_16_streaming(y + (int64_t)m * ldn + n, v);
             }
         } else {
 #pragma unroll
