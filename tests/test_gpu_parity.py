@@ -368,6 +368,43 @@ def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
     assert torch.equal(clone(x), layer(x))
 
 
+def test_random_shapes_agree_across_kernels():
+    """Seeded random shapes (ragged M and N, rows per codebook that are no multiple of anything, one
+    to many K stages, with and without bias): every kernel that accepts a shape agrees with the
+    scalar kernel, which test_small_b_all_variants pins against the oracle."""
+    import random
+    rnd = random.Random(2024)
+    done = 0
+    for case in range(60):
+        v = rnd.choice([2, 4, 8])
+        bits = rnd.choice([8, 16])
+        E = rnd.choice([16, 100, 256]) if bits == 8 else rnd.choice([300, 1024, 4096])
+        kc = (16 // (bits // 8)) * v
+        K = kc * rnd.choice([1, 2, 3, 5, 8, 9, 17])
+        G = rnd.choice([1, 1, 2, 3, 8])
+        N = G * rnd.choice([1, 5, 16, 37, 64, 128, 200, 512])
+        M = rnd.choice([1, 3, 16, 17, 100, 255, 257, 600, 1500])
+        if N * K > 20_000_000 or M * N > 2_000_000:
+            continue
+        spec = ProblemSpec("rnd", GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+        x, codes, cb = make_problem(spec, seed=case, device=DEV)
+        bias = torch.randn(N, generator=torch.Generator().manual_seed(case)).half().to(DEV) if case % 3 == 0 else None
+        _say("random shape", case, spec, "bias" if bias is not None else "")
+        ref = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_GENERIC, bias=bias).float()
+        scale = max(ref.abs().max().item(), 1e-3)
+        for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW):
+            try:
+                y = cabi.e2e_gemm_b(x, codes, cb, variant=variant, bias=bias)
+            except cabi.VqGemmError as e:
+                assert e.code == -4 and variant != cabi.VARIANT_AUTO, e
+                continue
+            torch.cuda.synchronize()
+            err = ((y.float() - ref).abs().max() / scale).item()
+            assert err <= TOL, (case, spec, cabi.VARIANT_NAMES[variant], err)
+        done += 1
+    assert done >= 40
+
+
 def test_every_m_from_1_to_16_on_the_decode_kernel():
     K, N = 1024, 80
     for M in range(1, 17):
