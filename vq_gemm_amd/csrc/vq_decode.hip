@@ -240,23 +240,29 @@ constexpr int kSlotPitch = 16 * kMaxWaves + 16;  // LDS bytes per slot; the pad 
 // what the X staging area lies over (it is only live while X is being loaded)
 constexpr int kStageOverTable = 1, kStageOverSlots = 2;
 
-template <int VEC, typename CodeT, bool REPL, int TB>
+__device__ __forceinline__ const half_t *bias_of() { return nullptr; }
+__device__ __forceinline__ const half_t *bias_of(const half_t *b) { return b; }
+
+template <int VEC, typename CodeT, bool REPL, int TB, typename... Bias>
 __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
                                                                const CodeT *__restrict__ codes,
                                                                const half_t *__restrict__ cb,
-                                                               half_t *__restrict__ y,
-                                                               const half_t *__restrict__ bias, int m_total, int K,
-                                                               int N, int entries, int n_books, int wgs_per_cb,
+                                                               half_t *__restrict__ y, int m_total, int K, int N,
+                                                               int entries, int n_books, int wgs_per_cb,
                                                                int books_per_wg, int tiles_per_cb, int tiles_q,
                                                                int tiles_r, int n_chunks, int red_off,
                                                                int stage_off, int stage_over, int acc_off,
-                                                               int recip_tail)
+                                                               int recip_tail, Bias... bias_arg)
 {
     typedef DecodeCfg<VEC, CodeT> C;
     typedef LaneCodes<VEC, CodeT> Codes;
+    // The bias pointer is a kernel argument only in the instantiation that adds one, so that a
+    // launch without bias fetches and tests nothing for it.
+    constexpr bool kHasBias = sizeof...(Bias) > 0;
+    const half_t *bias = bias_of(bias_arg...);
     // All kernel arguments are fetched at once: left to first use, each pointer costs the
     // prologue a scalar-load round trip of its own.
-    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(bias), "s"(m_total), "s"(K), "s"(N), "s"(entries),
+    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(m_total), "s"(K), "s"(N), "s"(entries),
                  "s"(n_books), "s"(wgs_per_cb), "s"(books_per_wg), "s"(tiles_per_cb), "s"(tiles_q), "s"(tiles_r),
                  "s"(n_chunks), "s"(red_off), "s"(stage_off), "s"(stage_over), "s"(acc_off), "s"(recip_tail));
     // blockIdx.y picks the 16-row slab of X (and of Y) this workgroup multiplies.
@@ -512,7 +518,7 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             if (chunk < n_chunks - 1) {
                 *carry = sum;
             } else {
-                if (bias) {
+                if constexpr (kHasBias) {
                     const half4_t b = *reinterpret_cast<const half4_t *>(bias + t.n);
                     sum += float4_t{(float)b[0], (float)b[1], (float)b[2], (float)b[3]};
                 }
@@ -690,19 +696,29 @@ hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
     BatchedPlan g = plan_batched<VEC, CodeT>(p);
     if (!g.ok) return hipErrorInvalidValue;
     g.per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
-    auto kern = !g.full  ? decode_batched_kernel<VEC, CodeT, false, 1>
-                : g.repl ? decode_batched_kernel<VEC, CodeT, true, C::TB>
-                         : decode_batched_kernel<VEC, CodeT, false, C::TB>;
-    if (!g.full && g.repl) kern = decode_batched_kernel<VEC, CodeT, true, 1>;  // only where a full batch is one tile
-    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), g.smem);
-    if (e != hipSuccess) return e;
     const int tail_rows = p.M - (g.n_slabs - 1) * kTileN;
-    hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(g.n_waves * 64), g.smem, s, p.x,
-                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.n_codebooks,
-                       g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, g.tiles_per_cb / g.wgs_per_cb,
-                       g.tiles_per_cb % g.wgs_per_cb, g.n_chunks, g.red_off, g.stage_off, g.stage_over, g.acc_off,
-                       (65536 + tail_rows - 1) / tail_rows);
-    return hipGetLastError();
+    // the same launch for the instantiation with a bias argument and the one without
+    auto launch = [&](auto kern, auto... bias) {
+        hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), g.smem);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(g.n_waves * 64), g.smem, s, p.x,
+                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.n_codebooks,
+                           g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, g.tiles_per_cb / g.wgs_per_cb,
+                           g.tiles_per_cb % g.wgs_per_cb, g.n_chunks, g.red_off, g.stage_off, g.stage_over, g.acc_off,
+                           (65536 + tail_rows - 1) / tail_rows, bias...);
+        return hipGetLastError();
+    };
+    // a full batch of one tile is the only case with a replicated table and TB = 1
+    const int tb = g.full ? C::TB : 1;
+    if (p.bias) {
+        if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, const half_t *>, p.bias)
+                                   : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, const half_t *>, p.bias);
+        return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, const half_t *>, p.bias)
+                       : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, const half_t *>, p.bias);
+    }
+    if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1>)
+                               : launch(decode_batched_kernel<VEC, CodeT, true, C::TB>);
+    return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1>) : launch(decode_batched_kernel<VEC, CodeT, false, C::TB>);
 }
 
 bool batched_supports(const ProblemB &p) { return plan_batched(p).ok; }
