@@ -499,6 +499,43 @@ def test_plain_gemm_and_hipblaslt_baseline(M, K, N):
         assert e1 <= TOL, e1
 
 
+# shapes the tiled kernel takes (K a multiple of 64, N of 8, X taller than 96 rows): few tiles -> 256x128
+# tiles, a full device -> 256x256 tiles; ragged M and N
+TILED_GEMM = [(300, 128, 520), (512, 192, 1288), (1024, 256, 136), (1024, 128, 16384), (2048, 4096, 1280),
+              (700, 64, 16392)]
+
+
+@pytest.mark.parametrize("M,K,N", TILED_GEMM)
+def test_plain_gemm_tiled_kernel(M, K, N):
+    g = torch.Generator().manual_seed(7)
+    w = (torch.randn(K, N, generator=g) * 0.05).half().to(DEV)
+    # one-hot rows of X read W out through the matrix cores: exact
+    idx = torch.randint(0, K, (M,), generator=g).to(DEV)
+    x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+    x[torch.arange(M, device=DEV), idx] = 1
+    _say("tiled gemm one-hot", M, K, N)
+    y = cabi.gemm_f16(x, w)
+    torch.cuda.synchronize()
+    assert torch.equal(y, w[idx])
+    x = torch.randn(M, K, generator=g).half().to(DEV)
+    _say("tiled gemm random", M, K, N)
+    y = cabi.gemm_f16(x, w)
+    torch.cuda.synchronize()
+    ref = (x.double() @ w.double()).cpu().numpy()
+    e1, _ = vo.rel_err(_np(y), ref)
+    assert e1 <= TOL, e1
+    # and the [N,K] layout, through the two-pass route of the VQ entry point
+    if K % 8 == 0 and M <= 1024:
+        spec = ProblemSpec("t", GEOM_B, M, K, N, 8, 256, 1, 8)
+        x, codes, cb = make_problem(spec, seed=8, device=DEV)
+        _say("tiled gemm two-pass", M, K, N)
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_TWOPASS)
+        torch.cuda.synchronize()
+        wd = cabi.dequant_b(codes, cb)
+        e1, _ = vo.rel_err(_np(y), (x.double() @ wd.double().T).cpu().numpy())
+        assert e1 <= TOL, e1
+
+
 # ------------------------------------------------------------------ the measured configurations at full size
 def test_config_c1_full_against_golden_and_oracle():
     import json, os

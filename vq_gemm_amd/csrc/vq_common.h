@@ -83,6 +83,11 @@ hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile = 0);
 hipError_t launch_gemm_nn(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);
 // y[M,N] = x[M,K] . w[N,K]^T
 hipError_t launch_gemm_nt(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);
+// the tiled kernel behind the two above (w_is_kn: w is [K,N], else [N,K]) and the shapes it takes;
+// tile: 0 = the width expected to be faster, 1 = 256x256, 2 = 256x128
+bool gemm_tiled_supports(const half_t *x, const half_t *w, int M, int K, int N, bool w_is_kn);
+hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, bool w_is_kn, hipStream_t s,
+                             int tile = 0);
 
 int device_cu_count();
 

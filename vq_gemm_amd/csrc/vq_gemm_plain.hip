@@ -1,5 +1,5 @@
-// Plain fp16 GEMM on the matrix cores, the no-dequant control of the VQ path and the second
-// pass of the two-pass (dequantise, then multiply) strategy.
+// Plain fp16 GEMM on the matrix cores, any shape: the kernel behind the tiled one of
+// vq_gemm_tiled.hip, for short X and for shapes that one does not take.
 //   NN: y[M,N] = x[M,K] . w[K,N]      NT: y[M,N] = x[M,K] . w[N,K]^T
 // 128x128 workgroup tile, 4 waves of 64x64, v_mfma_f32_32x32x16_f16, 32-deep K steps staged
 // through padded LDS rows with register prefetch of the next step.  Shape-agnostic (edges
@@ -141,13 +141,20 @@ hipError_t launch_plain(const half_t *x, const half_t *w, half_t *y, int M, int 
 
 }  // namespace
 
+// X shorter than this stays on the 128x128 kernel: a 256-row tile would be mostly padding.
+#ifndef VQ_TILED_MIN_M
+#define VQ_TILED_MIN_M 97
+#endif
+
 hipError_t launch_gemm_nn(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s)
 {
+    if (M >= VQ_TILED_MIN_M && gemm_tiled_supports(x, w, M, K, N, true)) return launch_gemm_tiled(x, w, y, M, K, N, true, s);
     return launch_plain<true>(x, w, y, M, K, N, s);
 }
 
 hipError_t launch_gemm_nt(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s)
 {
+    if (M >= VQ_TILED_MIN_M && gemm_tiled_supports(x, w, M, K, N, false)) return launch_gemm_tiled(x, w, y, M, K, N, false, s);
     return launch_plain<false>(x, w, y, M, K, N, s);
 }
 

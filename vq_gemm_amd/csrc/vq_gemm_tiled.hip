@@ -1,0 +1,375 @@
+// Plain fp16 GEMM with the tile of the prefill kernel: the no-dequant control of the VQ path
+// (reference strategy_1/src.cu:171-265, strategy_2/bsz128/src.cu:318-515) and the second pass of
+// the two-pass strategy.
+//   NN: y[M,N] = x[M,K] . w[K,N]      NT: y[M,N] = x[M,K] . w[N,K]^T
+//
+// Same frame as the VQ kernel: 256 threads (2x2 waves), a 256x256 tile of Y, 128x128 per wave as
+// 8x8 pieces of 16x16 with v_mfma_f32_16x16x32_f16, the accumulators pinned in the AGPRs, every
+// MFMA fenced and the other instructions dealt out between them by hand.  What differs is where
+// the W operand comes from: W is staged through the LDS like X instead of being gathered from a
+// codebook, which doubles the LDS bytes per k.
+//
+//   * A stage is 32 k (one MFMA step): 256 rows of X x 64 bytes and the matching 16 KB of W,
+//     global -> LDS directly.  Five stages fill the 160 KB; the loads of stage s+5 are issued
+//     while step s multiplies and have three whole steps to land.
+//   * Every operand is double buffered in registers: while step s multiplies, the 16 operands of
+//     step s+1 are read from the LDS.  One barrier per step publishes the next stage and frees
+//     the buffer of the stage just consumed.
+//   * X (and W in the NT layout) lies in the LDS as 64-byte rows, four to a 256-byte bank row,
+//     XOR-swizzled so that the 16 rows x one 16-byte chunk a quarter wave reads fall into 16
+//     different bank groups.
+//   * W in the NN layout ([K,N], n contiguous) lies as 32 k-rows of 512 bytes and is read with
+//     the transposing LDS read ds_read_b64_tr_b16: within 16 lanes, source lane 4d+q supplies
+//     row d, columns 4q..4q+3, and lane l receives column l of rows 0..3 - four consecutive k
+//     of one n, half an MFMA operand.  The 16-byte chunks of a k-row are XOR-swizzled with the
+//     row number so that the rows one instruction touches fall into different bank windows.
+//
+//   * A tile half as wide (256x128, 128x64 per wave, six stages of 24 KB) puts twice as many
+//     compute units to work when the 256x256 tiles are fewer than the units.
+//
+// K must be a multiple of 64 (and N a multiple of 8 in the NN layout); other shapes stay on the
+// simple kernel of vq_gemm_plain.hip.
+#include "vq_common.h"
+
+#include <type_traits>
+
+namespace vq {
+
+namespace {
+
+constexpr int BM = 256;
+constexpr int WM = 128;
+constexpr int MP = WM / 16;
+constexpr int kThreads = 256;
+constexpr int kStepK = 32;                           // k per stage
+constexpr int kXBytes = BM * kStepK * 2;             // the X part of a stage: 16 KB
+constexpr int kXLoads = kXBytes / (kThreads * 16);   // 16-byte chunks per thread: 4
+
+// The tile: NP 16-row pieces of W per wave (8: 256x256 tile, 4: 256x128).
+template <int NP>
+struct TileCfg {
+    static_assert(NP == 8 || NP == 4, "8 or 4 pieces of W per wave");
+    static constexpr int WN = NP * 16, BN = 2 * WN;
+    static constexpr int kWBytes = BN * kStepK * 2;                // the W part of a stage
+    static constexpr int kWLoads = kWBytes / (kThreads * 16);      // 4 or 2
+    static constexpr int kStageBytes = kXBytes + kWBytes;          // 32 or 24 KB
+    static constexpr int NS = NP == 8 ? 5 : 6;                     // stages in the LDS
+    static constexpr int kLoads = kXLoads + kWLoads;               // loads per thread and stage
+    static constexpr int kChunksPerK = BN / 8;                     // 16-byte chunks of a k-row (NN layout)
+    static constexpr size_t kLdsBytes = (size_t)NS * kStageBytes;
+};
+
+typedef short short4_t __attribute__((__vector_size__(4 * sizeof(short))));
+
+// s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
+// compiler knows nothing about this transfer, so every consumer sits behind an explicit
+// wait_vmcnt + barrier.  `lds_base` must be wave-uniform.
+__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(sbase)
+                 : "memory");
+}
+
+// acc += a . b with the accumulator pinned to one AGPR tuple (the register allocator otherwise
+// renames the 64 accumulators from MFMA to MFMA and fills the loop with copies).  The callers keep
+// MFMAs on one accumulator 64 MFMAs apart and pad before the accumulators are read back.
+__device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, const half8_t &b)
+{
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+__device__ __forceinline__ void st_global_16_streaming(void *p, uint4_t v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(p));
+}
+
+// Row-major part (X, or W in the NT layout): byte offset of 16-byte chunk cc (0..3) of row `row`.
+__device__ __forceinline__ int row_offset(int row, int cc)
+{
+    const int bank_row = row >> 2;
+    const int pos = (((row & 3) << 2) | cc) ^ (bank_row & 3);
+    return (bank_row * 16 + pos) * 16;
+}
+
+// k-major part (W in the NN layout): the XOR applied to the chunk index of k-row `k` (below 16).
+__device__ __forceinline__ int kmajor_swizzle(int k) { return 2 * ((k & 3) | (((k >> 3) & 1) << 2)); }
+
+template <bool W_IS_KN, int NP>
+__global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *__restrict__ x,
+                                                                 const half_t *__restrict__ w,
+                                                                 half_t *__restrict__ y, int M, int K, int N,
+                                                                 int tiles_m, int tiles_n)
+{
+    typedef TileCfg<NP> C;
+    constexpr int NS = C::NS, WN = C::WN, BN = C::BN, kStageBytes = C::kStageBytes;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, kg = lane >> 4;
+
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: re-number them so
+    // that an XCD works on consecutive tiles of the row-band-major order.
+    int wg = blockIdx.x;
+    const int n_wg = tiles_m * tiles_n;
+    if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+    const int tm = wg / tiles_n, tn = wg % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int n_stage = K / kStepK;
+
+    // ---- staging: global -> LDS ---------------------------------------------------------------
+    // Load i of wave v fills the 64 consecutive 16-byte slots [(4i+v)*64, +64) of a part; the lane
+    // looks up which chunk lives in its slot under the swizzle and fetches that.
+    uint32_t x_voff[kXLoads], w_voff[C::kWLoads];
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) {
+        const int slot = (4 * i + wave) * 64 + lane;
+        const int bank_row = slot >> 4;
+        const int pos = (slot & 15) ^ (bank_row & 3);
+        const int row = 4 * bank_row + (pos >> 2), cc = pos & 3;
+        x_voff[i] = (uint32_t)(((int64_t)(min(m0 + row, M - 1) - m0) * K + cc * 8) * 2);
+        if (!W_IS_KN && i < C::kWLoads) w_voff[i] = (uint32_t)(((int64_t)(min(n0 + row, N - 1) - n0) * K + cc * 8) * 2);
+        if (W_IS_KN && i < C::kWLoads) {
+            const int k = slot / C::kChunksPerK;
+            const int c = (slot % C::kChunksPerK) ^ kmajor_swizzle(k);
+            w_voff[i] = (uint32_t)(((int64_t)k * N + (min(n0 + c * 8, N - 8) - n0)) * 2);
+        }
+    }
+    // Where the loads of the stage NS ahead of the current one read (the last stage again once K is
+    // used up: harmless, and every stage so brings the same number of loads); moved on once per step.
+    const int64_t w_step = W_IS_KN ? (int64_t)kStepK * N : kStepK;
+    const int first_ahead = min(NS, n_stage - 1);
+    const half_t *x_ahead = x + (int64_t)m0 * K + first_ahead * kStepK;
+    const half_t *w_ahead = (W_IS_KN ? w + n0 : w + (int64_t)n0 * K) + first_ahead * w_step;
+    // Load i of a stage into buffer `buf` from the stage bases xb / wb: first the X part, then the W part.
+    auto issue = [&](int i, int buf, const half_t *xb, const half_t *wb) {
+        if (i < kXLoads) load_to_lds_16(buf * kStageBytes + (4 * i + wave) * 1024, x_voff[i], xb);
+        else load_to_lds_16(buf * kStageBytes + kXBytes + (4 * (i - kXLoads) + wave) * 1024, w_voff[i - kXLoads], wb);
+    };
+
+    float4_t acc[NP][MP];
+#pragma unroll
+    for (int j = 0; j < NP; j++)
+#pragma unroll
+        for (int i = 0; i < MP; i++) acc[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // ---- operand reads ------------------------------------------------------------------------
+    // X piece i is rows wm*128 + i*16 + r16, the lane's chunk is kg; a piece further is four bank
+    // rows (1 KB) on and leaves the swizzle unchanged.
+    const int x_rd = row_offset(wm * WM + r16, kg);
+    int w_rd[NP];
+    if (W_IS_KN) {
+        // Source lane (kg, s = r16) of a transposing read supplies row kg*8 + h*4 + s/4, columns
+        // piece*16 + 4*(s%4) .. +3: 8 bytes in chunk 2*piece + (s%4)/2 of its k-row.
+        const int k = kg * 8 + (r16 >> 2);  // + 4h: four rows on, same swizzle
+#pragma unroll
+        for (int j = 0; j < NP; j++) {
+            const int chunk = (wn * (WN / 8) + 2 * j + ((r16 & 3) >> 1)) ^ kmajor_swizzle(k);
+            w_rd[j] = kXBytes + (k * C::kChunksPerK + chunk) * 16 + (r16 & 1) * 8;
+        }
+    } else {
+        w_rd[0] = kXBytes + row_offset(wn * WN + r16, kg);
+    }
+    half8_t xs[2][MP];
+    half4_t wlo[2][NP], whi[2][NP];
+    auto load_x = [&](int set, int i, int buf) {
+        xs[set][i] = *reinterpret_cast<const half8_t *>(smem + buf * kStageBytes + x_rd + i * 1024);
+    };
+    // half h of W piece j (NT: h = 0 reads the whole operand, h = 1 nothing)
+    auto load_w = [&](int set, int j, int h, int buf) {
+        if constexpr (W_IS_KN) {
+            typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+            const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (lds_short4_t *)(smem + buf * kStageBytes + w_rd[j] + h * (4 * C::kChunksPerK * 16)));
+            if (h == 0) wlo[set][j] = __builtin_bit_cast(half4_t, v);
+            else whi[set][j] = __builtin_bit_cast(half4_t, v);
+        } else {
+            if (h == 0) {
+                const half8_t v = *reinterpret_cast<const half8_t *>(smem + buf * kStageBytes + w_rd[0] + j * 1024);
+                wlo[set][j] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+                whi[set][j] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+            }
+        }
+    };
+
+    // ---- prologue -----------------------------------------------------------------------------
+    // Loads complete in the order they were issued, so one count serves all of them.
+#pragma unroll
+    for (int d = 0; d < NS; d++) {
+        const int st = min(d, n_stage - 1);
+#pragma unroll
+        for (int i = 0; i < C::kLoads; i++)
+            issue(i, d, x + (int64_t)m0 * K + st * kStepK, (W_IS_KN ? w + n0 : w + (int64_t)n0 * K) + st * w_step);
+    }
+    wait_vmcnt<(NS - 1) * C::kLoads>();  // stage 0 has landed
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MP; i++) load_x(0, i, 0);
+#pragma unroll
+    for (int j = 0; j < NP; j++) {
+        load_w(0, j, 0, 0);
+        load_w(0, j, 1, 0);
+    }
+
+    // ---- main loop ----------------------------------------------------------------------------
+    // Step `stage` multiplies register set `set` while the operands of the next step are read into
+    // the other set and the loads of stage + NS are issued into the buffer this step's operands
+    // came from.  A wave issues one instruction every four cycles and an MFMA holds the pipe for
+    // sixteen: at most three other instructions fit between two MFMAs.
+    constexpr int kReads = MP + (W_IS_KN ? 2 * NP : NP);
+    constexpr int kReadGap = NP == 8 ? 2 : 1;   // MFMAs from one operand read to the next
+    constexpr int kLoadGap = NP == 8 ? 8 : 5;   // MFMAs from one global load to the next
+    static_assert(kReads * kReadGap <= NP * MP - 14, "the reads of a step end well ahead of its last MFMA");
+    static_assert(1 + (C::kLoads - 1) * kLoadGap < NP * MP, "the loads of a stage fit into a step");
+#define VQ_FENCE __builtin_amdgcn_sched_barrier(0)
+    int buf = 0;  // buffer of the current stage
+    auto step = [&](auto set_const, int stage) {
+        constexpr int set = decltype(set_const)::value;
+        const int buf_next = buf + 1 == NS ? 0 : buf + 1;
+        // Stage + 1 has landed when only the stages behind it are in flight; every wave has finished
+        // reading this stage's buffer (its reads were issued a step ago and are waited for here,
+        // where they have long completed).
+        wait_vmcnt<(NS - 2) * C::kLoads>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        VQ_FENCE;
+#pragma unroll
+        for (int m = 0; m < NP * MP; m++) {
+            // 4x4 quadrants of the pieces: (0,0) (1,0) (1,1) (0,1) for 8 pieces of W, (0,0) (0,1) for 4
+            const int q = m >> 4, p = (m >> 2) & 3, f = m & 3;
+            const int jh = NP == 8 ? ((q == 1 || q == 2) ? 1 : 0) : 0;
+            const int ih = NP == 8 ? q >> 1 : q;
+            const int j = jh * 4 + p, i = ih * 4 + f;
+            mfma_in_place(acc[j][i], __builtin_shufflevector(wlo[set][j], whi[set][j], 0, 1, 2, 3, 4, 5, 6, 7),
+                          xs[set][i]);
+            VQ_FENCE;
+            if (m % kReadGap == 0 && m / kReadGap < kReads) {
+                const int r = m / kReadGap;
+                if (r < MP) load_x(set ^ 1, r, buf_next);
+                else if (W_IS_KN) load_w(set ^ 1, (r - MP) >> 1, (r - MP) & 1, buf_next);
+                else load_w(set ^ 1, r - MP, 0, buf_next);
+                VQ_FENCE;
+            }
+            if (m % kLoadGap == 1 && m / kLoadGap < C::kLoads) {
+                issue(m / kLoadGap, buf, x_ahead, w_ahead);
+                VQ_FENCE;
+            }
+        }
+        const bool more = stage + NS + 1 < n_stage;
+        x_ahead += more ? kStepK : 0;
+        w_ahead += more ? w_step : 0;
+        buf = buf_next;
+    };
+    for (int stage = 0; stage < n_stage; stage += 2) {
+        step(std::integral_constant<int, 0>{}, stage);
+        step(std::integral_constant<int, 1>{}, stage + 1);
+    }
+#undef VQ_FENCE
+    // Drain the clamped loads still in flight before the stage buffers are reused.
+    wait_vmcnt<0>();
+    __syncthreads();
+    // the last MFMAs must have left the pipe before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its wave tile ----------
+    auto round4 = [](const float4_t &a) { return half4_t{(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]}; };
+    if ((N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        // Through the LDS: each wave transposes its fp16 block, 64 rows at a time, in a
+        // private region (padded rows) and stores whole row segments.
+        constexpr int kPitch = WN * 2 + 16;
+        constexpr int kRowChunks = WN / 8, kRowsPerPass = 64 / kRowChunks;
+        uint8_t *stage_out = smem + wave * (64 * kPitch);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int ii = 0; ii < 4; ii++) {
+                const int i = 4 * h + ii;
+#pragma unroll
+                for (int j = 0; j < NP; j++)
+                    *reinterpret_cast<half4_t *>(stage_out + (ii * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) = round4(acc[j][i]);
+            }
+#pragma unroll
+            for (int it = 0; it < 64 / kRowsPerPass; it++) {
+                const int row = it * kRowsPerPass + lane / kRowChunks, c = lane % kRowChunks;
+                const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
+                const int m = m0 + wm * WM + h * 64 + row;
+                const int n = n0 + wn * WN + c * 8;
+                if (m < M && n < N) st_global_16_streaming(y + (int64_t)m * N + n, v);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MP; i++) {
+            const int m = m0 + wm * WM + i * 16 + r16;
+            if (m >= M) continue;
+#pragma unroll
+            for (int j = 0; j < NP; j++) {
+                const int n = n0 + wn * WN + j * 16 + 4 * kg;
+                half_t *dst = y + (int64_t)m * N + n;
+                const half4_t hv = round4(acc[j][i]);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < N) dst[e] = hv[e];
+            }
+        }
+    }
+}
+
+template <bool W_IS_KN, int NP>
+hipError_t launch_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s)
+{
+    typedef TileCfg<NP> C;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + C::BN - 1) / C::BN;
+    auto kern = gemm_tiled_kernel<W_IS_KN, NP>;
+    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), C::kLdsBytes);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), C::kLdsBytes, s, x, w, y, M, K, N,
+                       tiles_m, tiles_n);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+// K in whole pairs of stages, 16-byte aligned operands and rows, lane offsets within 32 bits.
+bool gemm_tiled_supports(const half_t *x, const half_t *w, int M, int K, int N, bool w_is_kn)
+{
+    if (M < 1 || N < 1 || K < 2 * kStepK || K % (2 * kStepK) != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(w) & 15) != 0) return false;
+    if (w_is_kn && (N % 8 != 0 || (int64_t)kStepK * N * 2 >= (int64_t)1 << 31)) return false;
+    return (int64_t)BM * K * 2 < (int64_t)1 << 31;
+}
+
+// tile: 0 = the width expected to be faster, 1 = 256x256, 2 = 256x128
+hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, bool w_is_kn, hipStream_t s,
+                             int tile)
+{
+    if (!gemm_tiled_supports(x, w, M, K, N, w_is_kn)) return hipErrorInvalidValue;
+    if (tile == 0) {
+        // Rounds of tiles over the compute units.  A tile costs K/64 times a per-stage time that
+        // grows with the share of the units at work (the clock drops under load): fitted to
+        // measurements, 1.2 us for the wide tile and 0.68 us for the narrow one on an idle device,
+        // 1.6 times that on a full one.
+        const int cus = device_cu_count();
+        const int64_t tiles_m = (M + BM - 1) / BM;
+        auto cost = [&](int64_t tiles, double per_stage) {
+            const int64_t rounds = (tiles + cus - 1) / cus;
+            const double busy = (double)tiles / (double)(rounds * cus);
+            return (double)rounds * (5.0 + K / 64.0 * per_stage * (1.0 + 0.6 * busy));
+        };
+        tile = cost(tiles_m * ((N + 127) / 128), 0.68) < cost(tiles_m * ((N + 255) / 256), 1.2) ? 2 : 1;
+    }
+    if (tile == 2) return w_is_kn ? launch_tiled<true, 4>(x, w, y, M, K, N, s) : launch_tiled<false, 4>(x, w, y, M, K, N, s);
+    return w_is_kn ? launch_tiled<true, 8>(x, w, y, M, K, N, s) : launch_tiled<false, 8>(x, w, y, M, K, N, s);
+}
+
+}  // namespace vq
