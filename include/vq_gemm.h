@@ -70,13 +70,24 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
 
 /*
  * Fused VQ GEMM, geometry A (reference-native tensors, same entry point of the reference:
- * bind.cpp:3,7; indexing per strategy_2/bsz512/src.cu:163-176 and bench.py:46-56).
- * out is [M, 2*Nc].  `workspace` (K*2*Nc fp16) is required by TWOPASS; VQGEMM_VARIANT_AUTO takes the
- * two-pass route when it is given and the scalar kernel when it is NULL.
+ * bind.cpp:3,7; kernels strategy_2/bsz128/src.cu:213-253 and siblings, indexing per
+ * strategy_2/bsz512/src.cu:163-176 and bench.py:46-56).  out is [M, 2*Nc].
+ * VQGEMM_VARIANT_PREFILL is the fused tiled kernel (256x128 tiles; codebooks and code bytes in the
+ * LDS, W dequantised there two MFMA steps ahead of its use): K % 64 == 0, Nc % 16 == 0, x, w and
+ * codebook 16-byte aligned.  VQGEMM_VARIANT_TWOPASS needs `workspace` (K*2*Nc fp16).
+ * VQGEMM_VARIANT_AUTO takes the fused kernel for M > 96 where it applies (with `workspace` given:
+ * only while its tiles are at most one per compute unit, the two-pass route being faster beyond),
+ * else the two-pass route when `workspace` is given and the scalar kernel when it is NULL.
  */
 int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *out,
                       int64_t M, int64_t K, int64_t Nc, int32_t variant,
                       void *workspace, void *stream);
+
+/*
+ * Which kernel VQGEMM_VARIANT_AUTO resolves to for a geometry-A shape with 16-byte aligned operands
+ * (host only, no GPU call), so that a caller can tell whether the workspace will be used.
+ */
+int vqgemm_select_variant_a(int64_t M, int64_t K, int64_t Nc, int32_t has_workspace);
 
 /*
  * Stand-alone dequantisation to fp16 in HBM.

@@ -463,7 +463,10 @@ def test_empty_problems_and_rejections_on_device():
 
 
 # ------------------------------------------------------------------ geometry A (reference-native tensors)
-@pytest.mark.parametrize("M,K,Nc", [(32, 256, 64), (5, 96, 8), (130, 512, 132)])
+# the last four are shapes the fused tiled kernel takes (K % 64 == 0, Nc % 16 == 0, M > 96): ragged M and N,
+# K of two stages only, a single 16-column piece of codes
+@pytest.mark.parametrize("M,K,Nc", [(32, 256, 64), (5, 96, 8), (130, 512, 132), (300, 128, 80), (257, 64, 16),
+                                    (1000, 1024, 400), (520, 2048, 640)])
 def test_geometry_a(M, K, Nc):
     spec = ProblemSpec("A", GEOM_A, M, K, 2 * Nc, 2, 256, Nc // 4, 8, codebook_std=1.0)
     x, w, cb = make_problem(spec, seed=5, device=DEV)
@@ -472,10 +475,27 @@ def test_geometry_a(M, K, Nc):
     torch.cuda.synchronize()
     want = vo.dequant_a(_np(w), _np(cb))
     assert np.array_equal(_np(dec).view(np.uint16), want.view(np.uint16))
-    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_TWOPASS):
+    fused_ok = K % 64 == 0 and Nc % 16 == 0
+    assert (cabi.select_variant_a(M, K, Nc) == cabi.VARIANT_PREFILL) == (fused_ok and M > 96)
+    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_TWOPASS, cabi.VARIANT_PREFILL):
+        if variant == cabi.VARIANT_PREFILL and not fused_ok:
+            with pytest.raises(cabi.VqGemmError) as ei:
+                cabi.e2e_gemm_a(x, w, cb, variant=variant)
+            assert ei.value.code == -4
+            continue
+        _say("geometry A", cabi.VARIANT_NAMES[variant])
         y = cabi.e2e_gemm_a(x, w, cb, variant=variant)
         torch.cuda.synchronize()
         _check_gemm(y, x, w, cb, geometry=GEOM_A, what=f"A/{cabi.VARIANT_NAMES[variant]}")
+    if fused_ok:
+        # one-hot rows of X read W_dec out through the fused kernel: exact
+        idx = torch.randint(0, K, (M,), generator=torch.Generator().manual_seed(9)).to(DEV)
+        xo = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+        xo[torch.arange(M, device=DEV), idx] = 1
+        _say("geometry A fused one-hot", M, K, Nc)
+        y = cabi.e2e_gemm_a(xo, w, cb, variant=cabi.VARIANT_PREFILL)
+        torch.cuda.synchronize()
+        assert torch.equal(y, dec[idx])
 
 
 # ------------------------------------------------------------------ plain GEMM control and the hipBLASLt baseline

@@ -27,6 +27,7 @@ _SIGNATURES = {
     "vqgemm_encode_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _P]),
     "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
+    "vqgemm_select_variant_a": (ctypes.c_int, [_I64, _I64, _I64, _I32]),
     "vqgemm_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "vqgemm_version": (ctypes.c_int, []),
 }
@@ -196,6 +197,10 @@ def ref_gemm_f16(x, w, w_is_nk=False, out=None):
     if rc != 0:
         raise RuntimeError(f"vqref_gemm_f16 failed with code {rc}: {ref_lib().vqref_error_string(rc).decode()}")
     return out
+
+
+def select_variant_a(M, K, Nc, has_workspace=False) -> int:
+    return lib().vqgemm_select_variant_a(M, K, Nc, 1 if has_workspace else 0)
 
 
 def select_variant_b(M, K, N, vec, entries, n_codebooks, code_bits) -> int:

@@ -118,20 +118,27 @@ torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codeb
     }
     int rc;
     if (g.is_a) {
-        // Reference-native tensors: the tiled fused kernels are K-axis kernels, so this layout is
-        // served as the reference's two-pass strategy does it (strategy_1/src.cu:323-399): the
-        // bit-exact dequant kernel writes W_dec[K, 2*Nc], then a plain GEMM multiplies.  The
-        // second pass is a library GEMM (hipBLASLt, fp32 accumulate) except in the s1 module,
-        // which keeps this library's own MFMA GEMM as the reference's s1 keeps its own.
-        torch::Tensor dec = torch::empty({g.K, g.N}, input.options());
-        rc = vqgemm_dequant_a(c.data_ptr(), cb.data_ptr(), dec.data_ptr(), g.K, g.Nc, cur_stream(input));
-        check_rc(rc, "e2e_gemm (dequant pass)");
-        if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS) {
-            rc = vqgemm_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, cur_stream(input));
+        // Reference-native tensors.  The fused tiled kernel where it is expected to win (the reference's
+        // own scheme: codebooks in shared memory, W dequantised into a tile there).  Otherwise, and in
+        // the s1 module, the reference's two-pass strategy (strategy_1/src.cu:323-399): the bit-exact
+        // dequant kernel writes W_dec[K, 2*Nc], then a plain GEMM multiplies - this library's own in
+        // s1, as the reference's s1 keeps its own, a library GEMM (hipBLASLt) in the other modules.
+        const bool fused = VQ_VARIANT != VQGEMM_VARIANT_TWOPASS &&
+                           vqgemm_select_variant_a(g.M, g.K, g.Nc, 1) == VQGEMM_VARIANT_PREFILL;
+        if (fused) {
+            rc = vqgemm_e2e_gemm_a(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.Nc,
+                                   VQGEMM_VARIANT_PREFILL, nullptr, cur_stream(input));
         } else {
-            const int rrc = vqref_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, 0, cur_stream(input));
-            TORCH_CHECK(rrc == 0, "e2e_gemm (GEMM pass) failed: ", vqref_error_string(rrc), " (code ", rrc, ")");
-            rc = 0;
+            torch::Tensor dec = torch::empty({g.K, g.N}, input.options());
+            rc = vqgemm_dequant_a(c.data_ptr(), cb.data_ptr(), dec.data_ptr(), g.K, g.Nc, cur_stream(input));
+            check_rc(rc, "e2e_gemm (dequant pass)");
+            if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS) {
+                rc = vqgemm_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, cur_stream(input));
+            } else {
+                const int rrc = vqref_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, 0, cur_stream(input));
+                TORCH_CHECK(rrc == 0, "e2e_gemm (GEMM pass) failed: ", vqref_error_string(rrc), " (code ", rrc, ")");
+                rc = 0;
+            }
         }
     } else {
         rc = vqgemm_e2e_gemm_b(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.N, g.vec,

@@ -45,6 +45,18 @@ namespace {
 
 bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+// Whether the automatic choice takes the fused geometry-A kernel.  X shorter than 97 rows leaves its
+// 256-row tile mostly padding.  Its 4-byte gathers keep the LDS busier than the matrix cores, so
+// once there is more than one round of tiles the two-pass route is faster - when the caller brings
+// the scratch for it.
+bool fused_a_preferred(const ProblemA &p, bool has_workspace)
+{
+    if (p.M < 97 || !fused_a_supports(p)) return false;
+    if (!has_workspace) return true;
+    const int64_t tiles = (int64_t)((p.M + 255) / 256) * ((2 * p.Nc + 127) / 128);
+    return tiles <= device_cu_count();
+}
+
 int check_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits)
 {
     if (M < 0 || K < 0 || N < 0 || M > INT_MAX / 2 || K > INT_MAX / 2 || N > INT_MAX / 2) return VQGEMM_E_SHAPE;
@@ -191,12 +203,19 @@ int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *
     p.M = (int)M; p.K = (int)K; p.Nc = (int)Nc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipSuccess;
-    // No tiled fused kernel for this layout yet: with scratch the two-pass route (bit-exact dequant,
-    // then the MFMA GEMM) is the fast one, without it only the scalar kernel remains.
-    if (variant == VQGEMM_VARIANT_AUTO) variant = workspace ? VQGEMM_VARIANT_TWOPASS : VQGEMM_VARIANT_GENERIC;
+    // The fused tiled kernel where it applies and is expected to win; otherwise, with scratch, the
+    // two-pass route (bit-exact dequant, then the MFMA GEMM), and without it the scalar kernel.
+    if (variant == VQGEMM_VARIANT_AUTO) {
+        if (fused_a_preferred(p, workspace != nullptr)) variant = VQGEMM_VARIANT_PREFILL;
+        else variant = workspace ? VQGEMM_VARIANT_TWOPASS : VQGEMM_VARIANT_GENERIC;
+    }
     switch (variant) {
     case VQGEMM_VARIANT_GENERIC:
         e = launch_generic_a(p, s);
+        break;
+    case VQGEMM_VARIANT_PREFILL:
+        if (!fused_a_supports(p)) return aligned(x, 16) && aligned(w, 16) && aligned(codebook, 16) ? VQGEMM_E_VARIANT : VQGEMM_E_ALIGN;
+        e = launch_fused_a(p, s);
         break;
     case VQGEMM_VARIANT_TWOPASS:
         if (!workspace) return VQGEMM_E_NULL;
@@ -206,9 +225,18 @@ int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *
             e = launch_gemm_nn(p.x, static_cast<const half_t *>(workspace), p.y, p.M, p.K, 2 * p.Nc, s);
         break;
     default:
-        return VQGEMM_E_VARIANT;  // the decode/prefill tilings are geometry-B kernels
+        return VQGEMM_E_VARIANT;  // the decode tilings are geometry-B kernels
     }
     return static_cast<int>(e);
+}
+
+int vqgemm_select_variant_a(int64_t M, int64_t K, int64_t Nc, int32_t has_workspace)
+{
+    if (M < 0 || K < 0 || Nc < 0 || M > INT_MAX / 2 || K > INT_MAX / 2 || Nc > INT_MAX / 4 || Nc % 4 != 0) return VQGEMM_E_SHAPE;
+    ProblemA p = {};
+    p.M = (int)M; p.K = (int)K; p.Nc = (int)Nc;
+    if (fused_a_preferred(p, has_workspace != 0)) return VQGEMM_VARIANT_PREFILL;
+    return has_workspace ? VQGEMM_VARIANT_TWOPASS : VQGEMM_VARIANT_GENERIC;
 }
 
 int vqgemm_dequant_b(const void *codes, const void *codebook, void *w_out, int64_t N, int64_t K, int32_t vec,

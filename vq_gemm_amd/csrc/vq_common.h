@@ -89,6 +89,10 @@ bool gemm_tiled_supports(const half_t *x, const half_t *w, int M, int K, int N, 
 hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, bool w_is_kn, hipStream_t s,
                              int tile = 0);
 
+// geometry A, fused: the tiled [K,N] GEMM with its W stages dequantised on the compute unit
+bool fused_a_supports(const ProblemA &p);
+hipError_t launch_fused_a(const ProblemA &p, hipStream_t s);
+
 int device_cu_count();
 
 // Raises a kernel's dynamic-LDS limit when `bytes` needs it; remembers what was granted per

@@ -325,6 +325,299 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *_
     }
 }
 
+// ---- geometry A, fused ---------------------------------------------------------------------------
+// out[M, 2*Nc] = X[M,K] . W_dec with W_dec[k, 2n + r] = codebook[n/4][w[k,n]][r] (reference
+// strategy_2/bsz512/src.cu:163-176, bench.py:46-56): the vector lies along N, so a dequantised
+// row of W is n-contiguous - the [K,N] layout of the kernel above.  This kernel is that kernel with
+// the W part of a stage produced on the compute unit instead of loaded: the tile's codebooks (one
+// per 8 output columns, 1 KB each) and the code bytes of the coming stages sit in the LDS, and while
+// step s multiplies, every thread dequantises two 16-byte chunks of stage s+2 - four code bytes, four
+// 4-byte gathers, one 16-byte write into the k-major W buffer - which the transposing reads of step
+// s+1 then pick up.  This is the reference's own scheme (gather into a shared-memory tile, then
+// fragment loads), with the gather running two steps ahead of the matrix cores instead of between
+// two barriers.
+//
+// 256x128 tile (64 code columns, 16 codebooks), 128x64 per wave.  LDS: six X stages (96 KB), two W
+// buffers (16 KB), the codebooks (16 KB), four code tiles of two stages each (16 KB).
+constexpr int kANP = 4;
+constexpr int kABN = 2 * kANP * 16, kAWN = kANP * 16;       // 128, 64
+constexpr int kANSX = 6;                                     // X stages in the LDS
+constexpr int kAWBytes = kABN * kStepK * 2;                  // one dequantised W stage: 8 KB
+constexpr int kAChunksPerK = kABN / 8;                       // 16
+constexpr int kACbBytes = kAChunksPerK * 1024;               // 16 codebooks of 256 entries x 2 halves
+constexpr int kACodeRow = kABN / 2;                          // code bytes of one k-row of the tile: 64
+constexpr int kACodeTile = 2 * kStepK * kACodeRow;           // the codes of two stages: 4 KB
+constexpr int kANSC = 4;                                     // code tiles in the LDS
+constexpr int kAXBase = 0;
+constexpr int kAWBase = kAXBase + kANSX * kXBytes;
+constexpr int kACbBase = kAWBase + 2 * kAWBytes;
+constexpr int kACodeBase = kACbBase + kACbBytes;
+constexpr size_t kALdsBytes = kACodeBase + kANSC * kACodeTile;
+static_assert(kALdsBytes <= 160 * 1024, "the fused geometry-A kernel fits the LDS");
+
+__global__ __launch_bounds__(kThreads, 1) void gemm_a_fused_kernel(const half_t *__restrict__ x,
+                                                                   const uint8_t *__restrict__ codes,
+                                                                   const half_t *__restrict__ cb,
+                                                                   half_t *__restrict__ y, int M, int K, int Nc,
+                                                                   int tiles_m, int tiles_n)
+{
+    constexpr int NP = kANP, WN = kAWN, BN = kABN;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int N = 2 * Nc;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, kg = lane >> 4;
+
+    int wg = blockIdx.x;
+    const int n_wg = tiles_m * tiles_n;
+    if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+    const int tm = wg / tiles_n, tn = wg % tiles_n;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int n_stage = K / kStepK, n_pair = n_stage / 2;
+
+    // ---- staging: global -> LDS ---------------------------------------------------------------
+    uint32_t x_voff[kXLoads];
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) {
+        const int slot = (4 * i + wave) * 64 + lane;
+        const int bank_row = slot >> 4;
+        const int pos = (slot & 15) ^ (bank_row & 3);
+        const int row = 4 * bank_row + (pos >> 2), cc = pos & 3;
+        x_voff[i] = (uint32_t)(((int64_t)(min(m0 + row, M - 1) - m0) * K + cc * 8) * 2);
+    }
+    // A code tile is 64 k-rows x 64 code bytes, row-major; thread t fetches 16-byte piece t%4 of row
+    // t/4 (columns past Nc: the last 16 columns again).
+    const uint8_t *code_tile = codes + n0 / 2;
+    const uint32_t code_voff = (uint32_t)((int64_t)(tid >> 2) * Nc + (min(n0 / 2 + (tid & 3) * 16, Nc - 16) - n0 / 2));
+    const int64_t pair_step = (int64_t)2 * kStepK * Nc;
+    const half_t *x_tile = x + (int64_t)m0 * K;
+    auto issue_x = [&](int i, int buf, const half_t *xb) {
+        load_to_lds_16(kAXBase + buf * kXBytes + (4 * i + wave) * 1024, x_voff[i], xb);
+    };
+    auto issue_codes = [&](int cbuf, const uint8_t *cbase) {
+        load_to_lds_16(kACodeBase + cbuf * kACodeTile + wave * 1024, code_voff, cbase);
+    };
+    // what the loads issued during the current step read; moved on once per step / pair of steps
+    const half_t *x_ahead = x_tile + min(kANSX, n_stage - 1) * kStepK;
+    const uint8_t *c_ahead = code_tile + min(kANSC, n_pair - 1) * pair_step;
+
+    float4_t acc[NP][MP];
+#pragma unroll
+    for (int j = 0; j < NP; j++)
+#pragma unroll
+        for (int i = 0; i < MP; i++) acc[j][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // ---- operand reads (as in the plain kernel, W from its own two buffers) ----------------------
+    const int x_rd = kAXBase + row_offset(wm * WM + r16, kg);
+    int w_rd[NP];
+    {
+        const int k = kg * 8 + (r16 >> 2);
+#pragma unroll
+        for (int j = 0; j < NP; j++) {
+            const int chunk = (wn * (WN / 8) + 2 * j + ((r16 & 3) >> 1)) ^ kmajor_swizzle(k);
+            w_rd[j] = kAWBase + (k * kAChunksPerK + chunk) * 16 + (r16 & 1) * 8;
+        }
+    }
+    half8_t xs[2][MP];
+    half4_t wlo[2][NP], whi[2][NP];
+    auto load_x = [&](int set, int i, int buf) {
+        xs[set][i] = *reinterpret_cast<const half8_t *>(smem + buf * kXBytes + x_rd + i * 1024);
+    };
+    auto load_w = [&](int set, int j, int h, int wbuf) {
+        typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+        const short4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4_t *)(smem + wbuf * kAWBytes + w_rd[j] + h * (4 * kAChunksPerK * 16)));
+        if (h == 0) wlo[set][j] = __builtin_bit_cast(half4_t, v);
+        else whi[set][j] = __builtin_bit_cast(half4_t, v);
+    };
+
+    // ---- dequantisation: thread t builds chunk c = t%16 of k-rows t/16 and t/16 + 16 of a stage --------
+    // Chunk c (8 output columns = 4 code columns) uses codebook c of the tile.
+    const int dq_c = tid & 15, dq_k = tid >> 4;
+    const uint32_t dq_codes = kACodeBase + dq_k * kACodeRow + dq_c * 4;   // + code tile, + stage parity * 32 rows, + u * 16 rows
+    const uint32_t dq_book = kACbBase + dq_c * 1024;
+    const uint32_t dq_out = kAWBase + (dq_k * kAChunksPerK + (dq_c ^ kmajor_swizzle(dq_k))) * 16;  // + W buffer, + u * 16 rows
+    uint32_t dq_code[2];
+    uint4_t dq_val[2];
+    auto dq_read_codes = [&](int u, int cbuf, int par) {
+        dq_code[u] = *reinterpret_cast<const uint32_t *>(smem + dq_codes + cbuf * kACodeTile + (par * 32 + u * 16) * kACodeRow);
+    };
+    auto dq_gather = [&](int u, int b) {
+        const uint32_t code = (dq_code[u] >> (8 * b)) & 0xffu;
+        dq_val[u][b] = *reinterpret_cast<const uint32_t *>(smem + dq_book + code * 4);
+    };
+    auto dq_write = [&](int u, int wbuf) {
+        *reinterpret_cast<uint4_t *>(smem + dq_out + wbuf * kAWBytes + u * 16 * kAChunksPerK * 16) = dq_val[u];
+    };
+
+    // ---- prologue -----------------------------------------------------------------------------
+    // Loads complete in the order they were issued, so one count serves all of them.  The order is
+    // the one the main loop would have issued them in (X stage s at step s-6, the code tile of
+    // stages 2q, 2q+1 at step 2q-8, behind that step's X loads), with the codebooks in front.
+    {
+        const int g0 = n0 / 8;                       // first codebook of the tile
+        const int avail = (Nc / 4 - g0) * 1024 - 16;  // last valid 16-byte piece behind it
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(cb) + (int64_t)g0 * 1024;
+#pragma unroll
+        for (int i = 0; i < kACbBytes / (kThreads * 16); i++) {
+            const int byte = ((4 * i + wave) * 64 + lane) * 16;
+            load_to_lds_16(kACbBase + (4 * i + wave) * 1024, (uint32_t)min(byte, avail), src);
+        }
+    }
+    auto x_stage = [&](int st) { return x_tile + min(st, n_stage - 1) * kStepK; };
+    auto c_pair = [&](int q) { return code_tile + min(q, n_pair - 1) * pair_step; };
+    issue_codes(0, c_pair(0));
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) issue_x(i, 0, x_stage(0));
+    issue_codes(1, c_pair(1));
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) issue_x(i, 1, x_stage(1));
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) issue_x(i, 2, x_stage(2));
+    issue_codes(2, c_pair(2));
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) issue_x(i, 3, x_stage(3));
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) issue_x(i, 4, x_stage(4));
+    issue_codes(3, c_pair(3));
+#pragma unroll
+    for (int i = 0; i < kXLoads; i++) issue_x(i, 5, x_stage(5));
+    wait_vmcnt<4 * kXLoads + 2>();  // the codebooks, code tiles 0 and 1, X stages 0 and 1 have landed
+    __syncthreads();
+    // W of stages 0 and 1 from code tile 0
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) dq_read_codes(u, 0, st);
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) dq_gather(u, b);
+#pragma unroll
+        for (int u = 0; u < 2; u++) dq_write(u, st);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MP; i++) load_x(0, i, 0);
+#pragma unroll
+    for (int j = 0; j < NP; j++) {
+        load_w(0, j, 0, 0);
+        load_w(0, j, 1, 0);
+    }
+
+    // ---- main loop ----------------------------------------------------------------------------
+    // Step `stage` (parity `set`) multiplies register set `set`, reads the operands of stage+1 (X
+    // buffer xbuf+1, W buffer set^1), dequantises stage+2 into W buffer `set` out of code tile cq
+    // (the tile of stages stage+2 and its partner), and issues the X loads of stage+6 into the X
+    // buffer it multiplies from; even steps also issue the code tile four tiles ahead of cq.
+#define VQ_FENCE __builtin_amdgcn_sched_barrier(0)
+    int xbuf = 0;  // X buffer of the current stage
+    int cq = 1;    // code tile buffer of stage + 2
+    auto step = [&](auto set_const, int stage) {
+        constexpr int set = decltype(set_const)::value;
+        const int xbuf_next = xbuf + 1 == kANSX ? 0 : xbuf + 1;
+        // X of stage+1 and the code tile of stage+2 have landed when only what was issued behind
+        // them is in flight: four X stages and the code tiles of the even steps among them.
+        wait_vmcnt<4 * kXLoads + (set == 0 ? 2 : 3)>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        VQ_FENCE;
+#pragma unroll
+        for (int m = 0; m < NP * MP; m++) {
+            const int q = m >> 4, p = (m >> 2) & 3, f = m & 3;
+            const int j = p, i = q * 4 + f;
+            mfma_in_place(acc[j][i], __builtin_shufflevector(wlo[set][j], whi[set][j], 0, 1, 2, 3, 4, 5, 6, 7),
+                          xs[set][i]);
+            VQ_FENCE;
+            if (m < MP) {
+                load_x(set ^ 1, m, xbuf_next);
+                VQ_FENCE;
+            } else if (m < MP + 2 * NP) {
+                load_w(set ^ 1, (m - MP) >> 1, (m - MP) & 1, set ^ 1);
+                VQ_FENCE;
+            }
+            // the dequantisation of stage+2: code bytes first, the gathers a good LDS latency behind
+            // them, the writes a good LDS latency behind the gathers and ahead of the step's end
+            if (m == 0 || m == 2) {
+                dq_read_codes(m >> 1, cq, set);
+                VQ_FENCE;
+            }
+            if (m >= 9 && m < 17) {
+                dq_gather((m - 9) >> 2, (m - 9) & 3);
+                VQ_FENCE;
+            }
+            if (m == 24 || m == 25) {
+                dq_write(m - 24, set);
+                VQ_FENCE;
+            }
+            if (m % 5 == 1 && m / 5 < kXLoads) {
+                issue_x(m / 5, xbuf, x_ahead);
+                VQ_FENCE;
+            }
+            if (set == 0 && m == 21) {
+                issue_codes(cq == 0 ? kANSC - 1 : cq - 1, c_ahead);
+                VQ_FENCE;
+            }
+        }
+        x_ahead += stage + kANSX + 1 < n_stage ? kStepK : 0;
+        if (set == 1) {
+            c_ahead += (stage >> 1) + kANSC + 1 < n_pair ? pair_step : 0;
+            cq = cq + 1 == kANSC ? 0 : cq + 1;
+        }
+        xbuf = xbuf_next;
+    };
+    for (int stage = 0; stage < n_stage; stage += 2) {
+        step(std::integral_constant<int, 0>{}, stage);
+        step(std::integral_constant<int, 1>{}, stage + 1);
+    }
+#undef VQ_FENCE
+    wait_vmcnt<0>();
+    __syncthreads();
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its wave tile ----------
+    auto round4 = [](const float4_t &a) { return half4_t{(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]}; };
+    if ((reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        constexpr int kPitch = WN * 2 + 16;
+        constexpr int kRowChunks = WN / 8, kRowsPerPass = 64 / kRowChunks;
+        uint8_t *stage_out = smem + wave * (64 * kPitch);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int ii = 0; ii < 4; ii++) {
+                const int i = 4 * h + ii;
+#pragma unroll
+                for (int j = 0; j < NP; j++)
+                    *reinterpret_cast<half4_t *>(stage_out + (ii * 16 + r16) * kPitch + (j * 16 + 4 * kg) * 2) = round4(acc[j][i]);
+            }
+#pragma unroll
+            for (int it = 0; it < 64 / kRowsPerPass; it++) {
+                const int row = it * kRowsPerPass + lane / kRowChunks, c = lane % kRowChunks;
+                const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
+                const int m = m0 + wm * WM + h * 64 + row;
+                const int n = n0 + wn * WN + c * 8;
+                if (m < M && n < N) st_global_16_streaming(y + (int64_t)m * N + n, v);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MP; i++) {
+            const int m = m0 + wm * WM + i * 16 + r16;
+            if (m >= M) continue;
+#pragma unroll
+            for (int j = 0; j < NP; j++) {
+                const int n = n0 + wn * WN + j * 16 + 4 * kg;
+                half_t *dst = y + (int64_t)m * N + n;
+                const half4_t hv = round4(acc[j][i]);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < N) dst[e] = hv[e];
+            }
+        }
+    }
+}
+
 template <bool W_IS_KN, int NP>
 hipError_t launch_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s)
 {
@@ -370,6 +663,27 @@ hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M,
     }
     if (tile == 2) return w_is_kn ? launch_tiled<true, 4>(x, w, y, M, K, N, s) : launch_tiled<false, 4>(x, w, y, M, K, N, s);
     return w_is_kn ? launch_tiled<true, 8>(x, w, y, M, K, N, s) : launch_tiled<false, 8>(x, w, y, M, K, N, s);
+}
+
+// Nc in whole 16-byte pieces of code bytes, K in whole pairs of stages, 16-byte aligned operands.
+bool fused_a_supports(const ProblemA &p)
+{
+    if (p.M < 1 || p.Nc < 16 || p.Nc % 16 != 0 || p.K < 2 * kStepK || p.K % (2 * kStepK) != 0) return false;
+    if ((reinterpret_cast<uintptr_t>(p.x) & 15) != 0 || (reinterpret_cast<uintptr_t>(p.w) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(p.cb) & 15) != 0)
+        return false;
+    return (int64_t)BM * p.K * 2 < (int64_t)1 << 31 && (int64_t)2 * kStepK * p.Nc < (int64_t)1 << 31;
+}
+
+hipError_t launch_fused_a(const ProblemA &p, hipStream_t s)
+{
+    if (!fused_a_supports(p)) return hipErrorInvalidValue;
+    const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (2 * p.Nc + kABN - 1) / kABN;
+    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(gemm_a_fused_kernel), kALdsBytes);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(gemm_a_fused_kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kALdsBytes, s, p.x, p.w, p.cb,
+                       p.y, p.M, p.K, p.Nc, tiles_m, tiles_n);
+    return hipGetLastError();
 }
 
 }  // namespace vq
