@@ -47,7 +47,8 @@ def parse_args():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
     ap.add_argument("--probe", metavar="CONFIG", default=None,
-                    help="profiling aid: launch CONFIG (C1..C5, or a geometry-B shape M,K,N,vec,entries,code_bits) "
+                    help="profiling aid: launch CONFIG (C1..C5, REF = the reference's own shape in its native layout, "
+                         "a geometry-B shape M,K,N,vec,entries,code_bits, or GEMM,M,K,N = the plain fp16 GEMM) "
                          "--steps times, cold-HBM rotation for the decode configs, followed by one 256 MiB "
                          "device copy as a counter yardstick; prints no JSON")
     ap.add_argument("--mfma-ceiling", action="store_true",
@@ -103,13 +104,33 @@ def main():
         torch.cuda.synchronize()
 
     if args.probe:
+        from vq_gemm_amd.problems import GEOM_A, GEOM_B, ProblemSpec
+        if args.probe.startswith("GEMM,"):
+            m, k, n = (int(v) for v in args.probe.split(",")[1:])
+            g = torch.Generator().manual_seed(42)
+            xa = torch.randn(m, k, generator=g).half().to(dev)
+            wa = (torch.randn(k, n, generator=g) * 0.02).half().to(dev)
+            ya = torch.empty(m, n, dtype=torch.float16, device=dev)
+            barrier()
+            for _ in range(args.steps):
+                cabi.gemm_f16(xa, wa, out=ya)
+            barrier()
+            print(f"probe {args.probe}: {args.steps} launches of the plain GEMM", file=sys.stderr)
+            return
         if args.probe in CONFIGS:
             spec = CONFIGS[args.probe]
         else:
-            from vq_gemm_amd.problems import GEOM_B, ProblemSpec
             m, k, n, vec, entries, bits = (int(v) for v in args.probe.split(","))
             spec = ProblemSpec("probe", GEOM_B, m, k, n, vec, entries, 1, bits)
         x, codes, cb = make_problem(spec, seed=42, device=dev)
+        if spec.geometry == GEOM_A:
+            y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
+            barrier()
+            for _ in range(args.steps):
+                cabi.e2e_gemm_a(x, codes, cb, out=y)
+            barrier()
+            print(f"probe {args.probe}: {args.steps} launches, reference-native layout", file=sys.stderr)
+            return
         n_bufs = max(1, min(512, POOL_BYTES // spec.code_bytes)) if spec.M <= 16 else 1
         gen = torch.Generator(device=dev).manual_seed(1234)
         pool = [codes] + [torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev,
