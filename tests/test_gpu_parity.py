@@ -368,6 +368,29 @@ def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
     assert torch.equal(clone(x), layer(x))
 
 
+def test_registered_op_traces_and_matches_eager():
+    """torch.ops.vq_gemm_amd.vq_linear: the fake implementation agrees with the device one (opcheck)
+    and a layer traced by torch.compile (no code generation: the aot_eager backend) gives the eager result."""
+    from vq_gemm_amd.nn import VQLinear
+    from vq_gemm_amd import torch_ops  # noqa: F401
+    spec = ProblemSpec("op", GEOM_B, 24, 512, 384, 8, 256, 3, 8)
+    x, codes, cb = make_problem(spec, seed=13, device=DEV)
+    bias = torch.randn(spec.N, generator=torch.Generator().manual_seed(1)).half().to(DEV)
+    _say("opcheck vq_linear")
+    torch.library.opcheck(torch.ops.vq_gemm_amd.vq_linear.default, (x.view(2, 12, 512), codes, cb, bias),
+                          test_utils=("test_schema", "test_faketensor"))
+    layer = VQLinear(codes, cb, bias)
+    want = layer(x)
+    wq = _np(cabi.dequant_b(codes, cb)).astype(np.float64)
+    e1, _ = vo.rel_err(_np(want), _np(x).astype(np.float64) @ wq.T + _np(bias).astype(np.float64))
+    assert e1 <= TOL, e1
+    _say("aot_eager trace")
+    traced = torch.compile(layer, backend="aot_eager", fullgraph=True)
+    got = traced(x)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
 def test_random_shapes_agree_across_kernels():
     """Seeded random shapes (ragged M and N, rows per codebook that are no multiple of anything, one
     to many K stages, with and without bias): every kernel that accepts a shape agrees with the

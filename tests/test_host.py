@@ -115,3 +115,30 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(ops, "_modules", {})
     with pytest.raises(ImportError, match="no CPU fallback"):
         ops.load_module("s2_128")
+
+
+def test_registered_op_propagates_shapes_and_has_no_cpu_implementation():
+    import torch
+    from vq_gemm_amd import torch_ops  # noqa: F401
+    x = torch.empty(3, 5, 64, dtype=torch.float16, device="meta")
+    codes = torch.empty(32, 8, dtype=torch.uint8, device="meta")
+    cb = torch.empty(2, 256, 8, dtype=torch.float16, device="meta")
+    y = torch.ops.vq_gemm_amd.vq_linear(x, codes, cb)
+    assert y.shape == (3, 5, 32) and y.dtype == torch.float16
+    with pytest.raises(ValueError):   # 64 features against 8 codes x 4
+        torch.ops.vq_gemm_amd.vq_linear(x, codes, torch.empty(256, 4, dtype=torch.float16, device="meta"))
+    with pytest.raises(NotImplementedError):
+        torch.ops.vq_gemm_amd.vq_linear(torch.zeros(2, 64, dtype=torch.float16), torch.zeros(32, 8, dtype=torch.uint8),
+                                        torch.zeros(256, 8, dtype=torch.float16))
+
+
+def test_ctypes_wrappers_refuse_host_tensors():
+    import torch
+    from vq_gemm_amd import cabi
+    x = torch.zeros(2, 64, dtype=torch.float16)
+    codes = torch.zeros(32, 8, dtype=torch.uint8)
+    cb = torch.zeros(256, 8, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x, codes, cb)
+    with pytest.raises(ValueError):
+        cabi.dequant_b(codes, cb)

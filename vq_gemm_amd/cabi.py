@@ -81,7 +81,15 @@ class VqGemmError(RuntimeError):
 
 
 def _ptr(t):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Device address of a tensor (None passes through).  The library dereferences these on the GPU, so
+    anything but a contiguous tensor in device memory is refused here rather than faulting there."""
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("expected a tensor in GPU memory, got one on " + str(t.device))
+    if not t.is_contiguous():
+        raise ValueError("expected a contiguous tensor")
+    return ctypes.c_void_p(t.data_ptr())
 
 
 def _stream():

@@ -2,8 +2,9 @@
 fused VQ GEMM (geometry B), the call site after the path.
 
 Inference only (no gradient flows to codes or codebooks).  The product runs in the HIP library
-through its C ABI, the optional bias is added inside the kernel before the result is rounded.
-Nothing falls back to the CPU.
+through its C ABI, the optional bias is added inside the kernel before the result is rounded; the
+call is registered with `torch.library` (`torch.ops.vq_gemm_amd.vq_linear`) so that a traced graph
+holds it as one node.  Nothing falls back to the CPU.
 """
 from __future__ import annotations
 
@@ -11,6 +12,7 @@ import torch
 
 from . import cabi
 from .quantize import kmeans_quantize
+from .torch_ops import vq_linear
 
 
 class VQLinear(torch.nn.Module):
@@ -44,10 +46,7 @@ class VQLinear(torch.nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.dtype != torch.float16 or x.shape[-1] != self.in_features:
             raise ValueError(f"expected an fp16 input with {self.in_features} features")
-        lead = x.shape[:-1]
-        x2 = x.reshape(-1, self.in_features).contiguous()
-        y = cabi.e2e_gemm_b(x2, self.codes, self.codebook, bias=self.bias)
-        return y.view(*lead, self.out_features)
+        return vq_linear(x, self.codes, self.codebook, self.bias)
 
     def extra_repr(self) -> str:
         g = 1 if self.codebook.dim() == 2 else self.codebook.shape[0]

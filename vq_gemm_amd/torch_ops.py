@@ -1,0 +1,41 @@
+"""`torch.library` registration of the fused VQ GEMM, so that graphs traced by `torch.compile` /
+`torch.export` can hold it as one opaque node:
+
+    torch.ops.vq_gemm_amd.vq_linear(x, codes, codebook, bias=None) -> Tensor
+
+`x` is fp16 [..., K], `codes` [N, K/vec] uint8/uint16, `codebook` fp16 [E, vec] or [G, E, vec],
+`bias` fp16 [N] or None; the result is fp16 [..., N].  The device implementation calls the HIP
+library through its C ABI (the current stream, no synchronisation); the fake implementation only
+propagates shapes.  There is no CPU implementation: CPU tensors are refused.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import cabi
+
+
+def _out_shape(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor):
+    if codes.dim() != 2 or codebook.dim() not in (2, 3) or x.dim() < 1:
+        raise ValueError("vq_linear: x [..., K], codes [N, K/vec], codebook [E, vec] or [G, E, vec]")
+    if x.shape[-1] != codes.shape[1] * codebook.shape[-1]:
+        raise ValueError(f"vq_linear: x has {x.shape[-1]} features, codes x vec give {codes.shape[1] * codebook.shape[-1]}")
+    return (*x.shape[:-1], codes.shape[0])
+
+
+@torch.library.custom_op("vq_gemm_amd::vq_linear", mutates_args=(), device_types="cuda")
+def vq_linear(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor,
+              bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    shape = _out_shape(x, codes, codebook)
+    if x.dtype != torch.float16 or codebook.dtype != torch.float16:
+        raise ValueError("vq_linear: x and codebook must be float16")
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    y = cabi.e2e_gemm_b(x2, codes.contiguous(), codebook.contiguous(), bias=None if bias is None else bias.contiguous())
+    return y.view(shape)
+
+
+@vq_linear.register_fake
+def _vq_linear_fake(x, codes, codebook, bias=None):
+    return x.new_empty(_out_shape(x, codes, codebook))
