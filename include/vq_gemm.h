@@ -43,6 +43,8 @@ extern "C" {
                                      256x128 tiles when those put more compute units to work */
 #define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */
 #define VQGEMM_VARIANT_PREFILL_NARROW 5  /* the prefill kernel with 256x128 tiles, whatever the shape */
+#define VQGEMM_VARIANT_PREFILL_SMALL 6   /* the prefill kernel with 128x128 tiles, two workgroups per compute unit
+                                            (medium M); K a multiple of 64, of 128 for 8-vectors with 8-bit codes */
 
 /*
  * Fused VQ GEMM, geometry B.

@@ -85,13 +85,14 @@ def test_e2e_gemm_b_all_variants(row):
     _say("e2e_gemm_b", spec, "auto ->", cabi.VARIANT_NAMES[auto])
     ran = []
     for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL,
-                    cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_TWOPASS):
+                    cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_PREFILL_SMALL, cabi.VARIANT_TWOPASS):
         _say("  variant", cabi.VARIANT_NAMES[variant])
         try:
             y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
         except cabi.VqGemmError as e:
             assert e.code == -4, e          # "variant cannot serve this shape" is the only accepted refusal
-            assert variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW)
+            assert variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
+                               cabi.VARIANT_PREFILL_SMALL)
             continue
         torch.cuda.synchronize()
         _check_gemm(y, x, codes, cb, what=f"{spec.name}/{cabi.VARIANT_NAMES[variant]}")
@@ -102,7 +103,7 @@ def test_e2e_gemm_b_all_variants(row):
 
 
 @pytest.mark.parametrize("variant", [cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
-                                     cabi.VARIANT_GENERIC])
+                                     cabi.VARIANT_PREFILL_SMALL, cabi.VARIANT_GENERIC])
 @pytest.mark.parametrize("vec,bits,E", [(8, 8, 256), (4, 16, 4096), (4, 8, 256), (8, 16, 512)])
 def test_one_hot_activations_return_weight_columns_bit_exactly(variant, vec, bits, E):
     """X = rows of the identity: Y[m,:] must equal W[:,m] exactly (1.0*w + zeros is exact), which
@@ -201,10 +202,15 @@ PREFILL_B = [
     ("u8v8_many_tiles", 2048, 2048, 4096, 8, 256, 8, 16),
     # more 256x256 tiles than a 256-CU device has units: whole rounds of them, the left-over columns in 256x128 tiles
     ("u8v8_rounds_and_a_narrow_tail", 2048, 256, 8704, 8, 256, 8, 17),
+    # medium M: 128x128 tiles (the automatic choice here); ragged M and N, codebook changes inside a tile
+    ("u8v8_medium_m", 640, 2048, 2048, 8, 256, 8, 1),
+    ("u16v8_medium_m_ragged", 300, 1024, 1000, 8, 1000, 16, 5),
+    ("u8v4_medium_m_24_row_books", 200, 512, 240, 4, 256, 8, 10),
+    ("u8v2_medium_m", 129, 256, 136, 2, 256, 8, 1),
 ]
 
 
-@pytest.mark.parametrize("variant", [cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW])
+@pytest.mark.parametrize("variant", [cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_PREFILL_SMALL])
 @pytest.mark.parametrize("row", PREFILL_B, ids=[r[0] for r in PREFILL_B])
 def test_prefill_kernel_instantiations(row, variant):
     name, M, K, N, v, E, bits, G = row
@@ -214,8 +220,13 @@ def test_prefill_kernel_instantiations(row, variant):
     try:
         y = cabi.e2e_gemm_b(x, codes, cb, variant=variant)
     except cabi.VqGemmError as e:
-        # the 256x128 tile keeps four X buffers and does not take the largest codebooks
-        assert variant == cabi.VARIANT_PREFILL_NARROW and e.code == -4 and E * v * 2 >= 32768
+        assert e.code == -4
+        if variant == cabi.VARIANT_PREFILL_SMALL:
+            # the 128x128 tile wants K in whole code tiles (64 k, 128 k for 8-vectors with 8-bit codes)
+            assert K % (128 if (v, bits) == (8, 8) else 64) != 0
+            pytest.skip("K is not a whole number of code tiles")
+        # the 256x128 tile keeps four X buffers and does not take the largest codebooks (or several large ones)
+        assert variant == cabi.VARIANT_PREFILL_NARROW and E * v * 2 * min(G, 3) >= 32768
         pytest.skip("codebooks too large for the narrow tile")
     torch.cuda.synchronize()
     w = vo.dequant_b(_np(codes), _np(cb))
@@ -320,7 +331,7 @@ def test_bias_is_added_before_the_rounding_in_every_kernel(row):
     ref = _np(x).astype(np.float64) @ w.T + _np(bias).astype(np.float64)
     ran = []
     for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL,
-                    cabi.VARIANT_PREFILL_NARROW):
+                    cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_PREFILL_SMALL):
         _say("bias", name, cabi.VARIANT_NAMES[variant])
         try:
             y = cabi.e2e_gemm_b(x, codes, cb, variant=variant, bias=bias)
@@ -415,7 +426,8 @@ def test_random_shapes_agree_across_kernels():
         _say("random shape", case, spec, "bias" if bias is not None else "")
         ref = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_GENERIC, bias=bias).float()
         scale = max(ref.abs().max().item(), 1e-3)
-        for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW):
+        for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
+                        cabi.VARIANT_PREFILL_SMALL):
             try:
                 y = cabi.e2e_gemm_b(x, codes, cb, variant=variant, bias=bias)
             except cabi.VqGemmError as e:
@@ -442,7 +454,7 @@ def test_every_m_from_1_to_16_on_the_decode_kernel():
 def test_properties_constant_codes_zero_codebook_scaling():
     spec = ProblemSpec("prop", GEOM_B, 16, 1024, 128, 8, 256, 1, 8)
     x, codes, cb = make_problem(spec, seed=4, device=DEV)
-    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW):
+    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_PREFILL_SMALL):
         _say("properties", cabi.VARIANT_NAMES[variant])
         const = torch.full_like(codes, 37)
         y = cabi.e2e_gemm_b(x, const, cb, variant=variant)

@@ -13,8 +13,9 @@ import re
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 _INCLUDE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
 
-VARIANT_AUTO, VARIANT_GENERIC, VARIANT_DECODE, VARIANT_PREFILL, VARIANT_TWOPASS, VARIANT_PREFILL_NARROW = range(6)
-VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass", 5: "prefill_narrow"}
+(VARIANT_AUTO, VARIANT_GENERIC, VARIANT_DECODE, VARIANT_PREFILL, VARIANT_TWOPASS, VARIANT_PREFILL_NARROW,
+ VARIANT_PREFILL_SMALL) = range(7)
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass", 5: "prefill_narrow", 6: "prefill_small"}
 
 _I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
 

@@ -132,7 +132,7 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
 {
     int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
     if (rc != VQGEMM_OK) return rc;
-    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_PREFILL_NARROW) return VQGEMM_E_VARIANT;
+    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_PREFILL_SMALL) return VQGEMM_E_VARIANT;
     if (M == 0 || N == 0) return VQGEMM_OK;
     if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
     const uintptr_t code_align = code_bits / 8;
@@ -163,6 +163,11 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
         if (!a16) return VQGEMM_E_ALIGN;
         if (K == 0 || !prefill_narrow_supports(p)) return VQGEMM_E_VARIANT;
         e = launch_prefill_b(p, s, 2);
+        break;
+    case VQGEMM_VARIANT_PREFILL_SMALL:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !prefill_small_supports(p)) return VQGEMM_E_VARIANT;
+        e = launch_prefill_small_b(p, s);
         break;
     case VQGEMM_VARIANT_TWOPASS:
         if (bias) return VQGEMM_E_VARIANT;  // the plain GEMM of the two-pass route has no bias input

@@ -76,8 +76,14 @@ bool prefill_supports(const ProblemB &p);
 bool prefill_narrow_supports(const ProblemB &p);
 // expected time of the prefill kernel with the tile width it would choose, microseconds
 double prefill_cost_us(const ProblemB &p);
-// tile: 0 = the width expected to be faster, 1 = 256x256, 2 = 256x128
+// tile: 0 = the tile expected to be fastest (256x256, 256x128, a mix of the two, or 128x128),
+// 1 = 256x256, 2 = 256x128
 hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile = 0);
+
+// the prefill kernel with 128x128 tiles (vq_prefill_small.hip), for medium M
+bool prefill_small_supports(const ProblemB &p);
+double prefill_small_cost_us(const ProblemB &p);  // expected time, microseconds (1e30: not supported)
+hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s);
 
 // o[M,N] = x[M,K] . w[K,N]
 hipError_t launch_gemm_nn(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);

@@ -735,10 +735,10 @@ bool decode_supports(const ProblemB &p)
 // the smaller.  Fitted to measurements on a 256-CU MI355X:
 //   decode path   per workgroup a prologue (3), then per codebook and chunk of K its tiles at
 //                 0.75 us per tile and 4096 k (1.25 when K goes in chunks: X is staged again per
-//                 chunk), plus 3.5 per change of codebook or chunk; workgroups beyond those
-//                 resident run in further rounds;
-//   prefill       0.85 + 0.9 * (fraction of the CUs that have a 256x256 tile) us per 64-deep
-//                 stage, one round of tiles per 256 CUs.
+//                 chunk), plus 5 per change of codebook or chunk; workgroups beyond those
+//                 resident run in further rounds.  With K of 2048 or less two workgroups share a
+//                 compute unit: prologue 8, and a tile then costs each of them 1.0 us per 2048 k;
+//   prefill       the prefill kernels' own estimate for the tiles they would choose.
 bool decode_preferred(const ProblemB &p)
 {
     if (!decode_supports(p)) return false;
@@ -747,11 +747,11 @@ bool decode_preferred(const ProblemB &p)
     const int cus = device_cu_count();
     const int per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
     const int rounds_d = (per_slab * g.n_slabs + cus * g.per_cu - 1) / (cus * g.per_cu);
-    const double t_tile = (g.n_chunks == 1 ? 0.75 : 1.25) * g.n_waves / kMaxWaves * g.per_cu;
+    const bool shared = g.per_cu > 1;
+    const double t_tile = (g.n_chunks == 1 ? 0.75 : 1.25) * g.n_waves / kMaxWaves * g.per_cu * (shared ? 1.35 : 1.0);
     const int passes = g.books_per_wg * g.n_chunks;
-    const double t_decode = rounds_d * (3.0 + passes * g.tiles_per_wg * t_tile + (passes - 1) * 3.5);
-    // the prefill kernel's own estimate for the tile width it would choose, plus launch and drain
-    const double t_prefill = prefill_supports(p) ? 3.0 + prefill_cost_us(p) : 1e30;
+    const double t_decode = rounds_d * ((shared ? 8.0 : 3.0) + passes * g.tiles_per_wg * t_tile + (passes - 1) * 5.0);
+    const double t_prefill = prefill_supports(p) ? 1.0 + prefill_cost_us(p) : 1e30;
     return t_decode <= t_prefill;
 }
 

@@ -33,140 +33,13 @@
 // 32 s on, and lane group g (lanes 16g..16g+15) holds the 8 k from 8 g on.  K must be a
 // multiple of the k that 16 bytes of codes cover; a last stage of 32 k runs in the TAIL
 // instantiation, which points the W operands of the missing step at zeros.
-#include "vq_common.h"
+#include "vq_prefill_common.h"
 
 #include <type_traits>
 
 namespace vq {
 
 namespace {
-
-constexpr int BM = 256, BN = 256;     // workgroup tile
-constexpr int WM = 128, WN = 128;     // wave tile
-constexpr int MP = WM / 16, NP = WN / 16;  // 16-row pieces of X and of W per wave
-constexpr int kThreads = 256;
-constexpr int kStageK = 64;           // k per LDS stage (2 MFMA steps)
-constexpr int kStageBytes = BM * kStageK * 2;  // 32 KB
-constexpr int kChunksPerThread = (BM * 8) / kThreads;  // 16-byte chunks of an X stage per thread
-
-template <int VEC, typename CodeT>
-struct PrefillCfg {
-    static constexpr int CSZ = (int)sizeof(CodeT);
-    static constexpr int CPO = 8 / VEC;                 // codes per 8-half operand
-    static constexpr int RB = CPO * CSZ;                // bytes of codes behind one operand (1, 2 or 4)
-    static constexpr int KC = (16 / CSZ) * VEC;         // k covered by 16 bytes of one row's codes
-    static constexpr int K_SUPER = KC > kStageK ? KC : kStageK;  // k per code tile (a "super stage")
-    static constexpr int STAGES = K_SUPER / kStageK;    // LDS stages per super stage (1 or 2)
-    static constexpr int CH = K_SUPER / KC;             // 16-byte chunks per row of a code tile (1 or 2)
-    static constexpr int HALF = 32 / VEC * CSZ;         // bytes of one row's codes per MFMA step
-    static constexpr int kTileBytes = CH * BN * 16;     // code tile in the LDS: [chunk][row][16 bytes]
-    static_assert(RB == 1 || RB == 2 || RB == 4, "unsupported code layout");
-    static_assert(STAGES == 1 || STAGES == 2, "unsupported code layout");
-    // code tiles in flight: the one being read plus those loaded ahead
-    static constexpr int code_bufs(int ns) { return STAGES == 1 ? ns : 3; }
-};
-
-// Byte offset inside a stage buffer of logical 16-byte chunk cc (0..7) of X-tile row `row`.
-__device__ __forceinline__ int x_offset(int row, int cc)
-{
-    const int bank_row = row >> 1;
-    const int pos = (((row & 1) << 3) | cc) ^ (bank_row & 15);
-    return (bank_row * 16 + pos) * 16;
-}
-
-// s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
-// compiler knows nothing about this transfer, so every consumer sits behind an explicit
-// wait_vmcnt + barrier.  `lds_base` must be wave-uniform.
-__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base), "v"(voff), "s"(sbase)
-                 : "memory");
-}
-
-// acc += a . b with the accumulator pinned to one AGPR tuple.  Left to itself the register
-// allocator renames the 64 four-register accumulators from MFMA to MFMA and pays for it with
-// copies at the loop edge and with spills.  The compiler cannot see into the statement, so the
-// callers keep dependent MFMAs (same accumulator) far apart and pad before the accumulators are
-// read back.
-__device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, const half8_t &b)
-{
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-}
-
-// 16-byte store of a result that this kernel does not read again: the non-temporal hint lets the
-// write leave the L2 as it is issued instead of waiting for the write-back at the end of the kernel
-// (all workgroups of a round finish at about the same time).
-__device__ __forceinline__ void st_global_16_streaming(void *p, uint4_t v)
-{
-    __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(p));
-}
-
-// The four fp32 sums of an accumulator rounded to fp16, with the bias of their columns added first.
-template <bool HAS_BIAS>
-__device__ __forceinline__ half4_t round4(const float4_t &a, const float (&b)[4])
-{
-    if constexpr (HAS_BIAS)
-        return half4_t{(half_t)(a[0] + b[0]), (half_t)(a[1] + b[1]), (half_t)(a[2] + b[2]), (half_t)(a[3] + b[3])};
-    else
-        return half4_t{(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]};
-}
-
-// floor(x / d) for 0 <= x and a quotient small enough that float rounding stays within one
-// (here: x < d + 256); `rcp` = 1.0f / d.
-__device__ __forceinline__ int small_div(int x, int d, float rcp)
-{
-    int qt = (int)((float)x * rcp);
-    const int rem = x - qt * d;
-    qt += rem >= d ? 1 : 0;
-    qt -= rem < 0 ? 1 : 0;
-    return qt;
-}
-
-// The RB bytes of codes behind one operand, zero-extended.
-template <int RB>
-__device__ __forceinline__ uint32_t read_codes(const uint8_t *p)
-{
-    if constexpr (RB == 1) return *p;
-    else if constexpr (RB == 2) return *reinterpret_cast<const uint16_t *>(p);
-    else return *reinterpret_cast<const uint32_t *>(p);
-}
-
-// Gathers half `h` (4 halves) of one MFMA operand: the codes packed in `cr` select codewords of
-// the codebook at LDS byte offset `book`.  With `zero` set the reads go to the 16 zero bytes at
-// `zero_off` instead (a step past the end of K).  An operand is fetched in two halves because a
-// 16-byte gather with its bank conflicts holds the wave's issue longer than the gap between two
-// MFMAs.
-template <int VEC, typename CodeT, bool TAIL>
-__device__ __forceinline__ half4_t gather4(const uint8_t *lds, uint32_t book, uint32_t cr, int h, bool zero, uint32_t zero_off)
-{
-    constexpr int CPO = 8 / VEC, BITS = 8 * (int)sizeof(CodeT);
-    auto at = [&](int c, int byte_off) {
-        const uint32_t code = CPO == 1 ? cr : (cr >> (BITS * c)) & ((1u << BITS) - 1u);
-        uint32_t a = book + code * (uint32_t)(VEC * 2);
-        if (TAIL) a = zero ? zero_off : a;
-        return lds + a + byte_off;
-    };
-    if constexpr (VEC == 8) {
-        return *reinterpret_cast<const half4_t *>(at(0, 8 * h));
-    } else if constexpr (VEC == 4) {
-        return *reinterpret_cast<const half4_t *>(at(h, 0));
-    } else {
-        static_assert(VEC == 2, "vector length must be 2, 4 or 8");
-        const half2_t q0 = *reinterpret_cast<const half2_t *>(at(2 * h, 0));
-        const half2_t q1 = *reinterpret_cast<const half2_t *>(at(2 * h + 1, 0));
-        return __builtin_shufflevector(q0, q1, 0, 1, 2, 3);
-    }
-}
 
 template <int VEC, typename CodeT, bool TAIL, int NS>
 __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__restrict__ x,
@@ -903,25 +776,6 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
     else epilogue(std::false_type{});
 }
 
-constexpr size_t kLdsLimit = 160 * 1024;
-
-int codebooks_per_tile(const ProblemB &p, int bn)
-{
-    // Worst case number of codebooks a band of `bn` rows of W touches.
-    int n;
-    if (p.n_codebooks == 1) n = 1;
-    else if (p.rows_per_cb >= bn && p.rows_per_cb % bn == 0) n = 1;
-    else if (bn % p.rows_per_cb == 0) n = bn / p.rows_per_cb;
-    else n = (bn + p.rows_per_cb - 1) / p.rows_per_cb + 1;
-    return n < p.n_codebooks ? n : p.n_codebooks;
-}
-
-// codebooks of a tile, padded to the 1 KB steps they are copied in, plus 16 zero bytes
-size_t books_bytes(const ProblemB &p, int bn)
-{
-    return (((size_t)codebooks_per_tile(p, bn) * p.entries * p.vec * 2 + 1023) & ~(size_t)1023) + 16;
-}
-
 template <int VEC, typename CodeT>
 size_t lds_bytes(const ProblemB &p, int n_stages)
 {
@@ -1077,16 +931,26 @@ bool prefill_narrow_supports(const ProblemB &p)
     return what.narrow;
 }
 
+// 128x128 tiles are taken when they are expected to be clearly faster than the best cut into large tiles
+constexpr double kSmallTileMargin = 0.95;
+
 double prefill_cost_us(const ProblemB &p)
 {
     PrefillQuery what;
     prefill_query(p, what);
-    return what.cost_us;
+    if (!what.wide) return what.cost_us;
+    const double small = prefill_small_cost_us(p);
+    return small < kSmallTileMargin * what.cost_us ? small : what.cost_us;
 }
 
 hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile)
 {
     if (!prefill_supports(p)) return hipErrorInvalidValue;
+    if (tile == 0) {
+        PrefillQuery what;
+        prefill_query(p, what);
+        if (prefill_small_cost_us(p) < kSmallTileMargin * what.cost_us) return launch_prefill_small_b(p, s);
+    }
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
     case 8: return u8 ? launch_prefill_typed<8, uint8_t>(p, s, tile) : launch_prefill_typed<8, uint16_t>(p, s, tile);
