@@ -554,6 +554,22 @@ def test_plain_gemm_and_hipblaslt_baseline(M, K, N):
         assert e1 <= TOL, e1
 
 
+@pytest.mark.parametrize("kernel", ["s1", "s2_128", "s3_wasp"])
+def test_harness_with_the_reference_controls(kernel):
+    """vq_gemm_amd.harness: the reference harness's three calls on its own tensor layout, with its checks
+    made assertions; the full reference shape through the fused module, small shapes through the others."""
+    from vq_gemm_amd import harness
+    full = kernel == "s2_128"
+    _say("harness", kernel, "vq gemm")
+    r = harness.run(kernel, M=2048 if full else 300, K=4096 if full else 256, N=640 if full else 80, timing=False)
+    assert r["deterministic"] and r["dequant_bit_exact"] and r["rel_err"] <= TOL
+    _say("harness", kernel, "plain gemm")
+    r = harness.run(kernel, test_gemm=True, M=200, K=128, N=136, timing=False)
+    assert r["deterministic"] and r["rel_err"] <= TOL
+    _say("harness", kernel, "profiling launch")
+    harness.run(kernel, profiling=True, M=128, K=64, N=32)
+
+
 # shapes the tiled kernel takes (K a multiple of 64, N of 8, X taller than 96 rows): few tiles -> 256x128
 # tiles, a full device -> 256x256 tiles; ragged M and N
 TILED_GEMM = [(300, 128, 520), (512, 192, 1288), (1024, 256, 136), (1024, 128, 16384), (2048, 4096, 1280),
