@@ -51,6 +51,8 @@ def parse_args():
                          "a geometry-B shape M,K,N,vec,entries,code_bits, or GEMM,M,K,N = the plain fp16 GEMM) "
                          "--steps times, cold-HBM rotation for the decode configs, followed by one 256 MiB "
                          "device copy as a counter yardstick; prints no JSON")
+    ap.add_argument("--probe-variant", type=int, default=0,
+                    help="with --probe on a geometry-B shape: the VQGEMM_VARIANT_* value to launch (0 = automatic choice)")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="run the register-only MFMA loop (vq_gemm_amd/lib/mfma_ceiling): what the matrix cores "
                          "sustain on this device with random and with zero operands; prints no JSON")
@@ -140,7 +142,7 @@ def main():
         dst = torch.empty_like(src)
         barrier()
         for i in range(args.steps):
-            cabi.e2e_gemm_b(x, pool[i % n_bufs], cb, out=y)
+            cabi.e2e_gemm_b(x, pool[i % n_bufs], cb, out=y, variant=args.probe_variant)
         barrier()
         dst.copy_(src)   # yardstick: reads 256 MiB, writes 256 MiB
         barrier()

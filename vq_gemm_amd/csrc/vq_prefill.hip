@@ -41,7 +41,12 @@ namespace vq {
 
 namespace {
 
-template <int VEC, typename CodeT, bool TAIL, int NS>
+// The prologue of the 256x256 kernel puts up to three X loads of stage D into buffer D: 12 KB from its
+// start on are taken, the rest is free until the main loop.
+constexpr int kWideSplitSkip = 12 * 1024;
+
+// SPLIT: the codebooks lie in the LDS in the split layout (vq_prefill_common.h).
+template <int VEC, typename CodeT, bool TAIL, int NS, bool SPLIT>
 __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__restrict__ x,
                                                               const CodeT *__restrict__ codes,
                                                               const half_t *__restrict__ cb,
@@ -59,6 +64,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int kCodeBase = NS * kStageBytes;
     constexpr int kCbBase = kCodeBase + NC * C::kTileBytes;
+    constexpr int kSplitTemp = D * kStageBytes + kWideSplitSkip;  // where the plain copy of the codebooks waits
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int wm = wave >> 1, wn = wave & 1;
@@ -164,10 +170,10 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
     };
     // the two halves of W piece j from the codes read before
     auto load_w1 = [&](int set, int j, bool zero) {
-        wlo[j] = gather4<VEC, CodeT, TAIL>(smem, book[j], cr[set][j & 3], 0, zero, zero_off);
+        wlo[j] = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[set][j & 3], 0, zero, zero_off);
     };
     auto load_w2 = [&](int set, int j, bool zero) {
-        whi[j] = gather4<VEC, CodeT, TAIL>(smem, book[j], cr[set][j & 3], 1, zero, zero_off);
+        whi[j] = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[set][j & 3], 1, zero, zero_off);
     };
     // MFMA f of group p of the 4x4 quadrant (jh, ih): a group is W piece p against the four X
     // pieces, or (x_outer) X piece p against the four W pieces
@@ -186,9 +192,11 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         const uint8_t *src = reinterpret_cast<const uint8_t *>(cb + (int64_t)g_first * entries * VEC);
         const int n16 = cb_lds_count * cb_bytes / 16;
         const int g_total_16 = (int)(((int64_t)((ldn + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
-        // past the last codebook: read its last 16 bytes again
+        // past the last codebook: read its last 16 bytes again.  SPLIT: a plain copy first, into the
+        // part of X buffer D that the prologue's loads of stage D leave alone, re-laid below.
+        const int dst = SPLIT ? kSplitTemp : kCbBase;
         for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
-            load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
+            load_to_lds_16(dst + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
     }
 #pragma unroll
     for (int d = 0; d < D; d++) {
@@ -218,6 +226,10 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         else wait_vmcnt<in_flight>();
     }
     __syncthreads();
+    if constexpr (SPLIT) {
+        split_codebooks(smem, kSplitTemp, kCbBase, cb_lds_count, tid, kThreads);
+        __syncthreads();
+    }
     int buf = 0;   // X buffer of the current stage; stage+j lives in (buf + j) % NS
     int cbuf = 0;  // code buffer of the current super stage; super+j lives in (cbuf + j) % NC
 #pragma unroll
@@ -486,7 +498,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
 constexpr int NPN = 4;                 // W pieces per wave in the narrow tile
 constexpr int WNN = NPN * 16, BNN = 2 * WNN;
 
-template <int VEC, typename CodeT, bool TAIL>
+template <int VEC, typename CodeT, bool TAIL, bool SPLIT>
 __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_t *__restrict__ x,
                                                                      const CodeT *__restrict__ codes,
                                                                      const half_t *__restrict__ cb,
@@ -590,7 +602,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
         cr[cset][j & 1] = read_codes<C::RB>(smem + code_rd + cbuf * kTile + (pos / 16) * (BNN * 16) + j * 256 + pos % 16);
     };
     auto load_w_half = [&](int set, int cset, int j, int h, bool zero) {
-        const half4_t v = gather4<VEC, CodeT, TAIL>(smem, book[j], cr[cset][j & 1], h, zero, zero_off);
+        const half4_t v = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[cset][j & 1], h, zero, zero_off);
         if (h == 0) wlo[set][j] = v;
         else whi[set][j] = v;
     };
@@ -604,8 +616,10 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
         const uint8_t *src = reinterpret_cast<const uint8_t *>(cb + (int64_t)g_first * entries * VEC);
         const int n16 = cb_lds_count * cb_bytes / 16;
         const int g_total_16 = (int)(((int64_t)((ldn + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
+        // SPLIT: a plain copy first, into X buffer D (nothing is loaded into it before the main loop), re-laid below
+        const int dst = SPLIT ? D * kStageBytes : kCbBase;
         for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
-            load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
+            load_to_lds_16(dst + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
     }
 #pragma unroll
     for (int d = 0; d < D; d++) {
@@ -623,6 +637,10 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
         wait_vmcnt<in_flight>();
     }
     __syncthreads();
+    if constexpr (SPLIT) {
+        split_codebooks(smem, D * kStageBytes, kCbBase, cb_lds_count, tid, kThreads);
+        __syncthreads();
+    }
 
     int buf = 0, cbuf = 0;
     // step 0 of stage 0: all of its operands; and the codes of the first W pair of step 1
@@ -850,9 +868,19 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         // waits for its own loads) only so that very large codebooks still run.
         const int ns = lds_bytes<VEC, CodeT>(p, 4) <= kLdsLimit ? 4 : lds_bytes<VEC, CodeT>(p, 3) <= kLdsLimit ? 3 : 2;
         const size_t smem = lds_bytes<VEC, CodeT>(p, ns);
-        auto kern = ns == 4   ? (tail ? prefill_kernel<VEC, CodeT, true, 4> : prefill_kernel<VEC, CodeT, false, 4>)
-                    : ns == 3 ? (tail ? prefill_kernel<VEC, CodeT, true, 3> : prefill_kernel<VEC, CodeT, false, 3>)
-                              : (tail ? prefill_kernel<VEC, CodeT, true, 2> : prefill_kernel<VEC, CodeT, false, 2>);
+        // the split codebook layout (8-vectors, 8-bit codes, 256 entries) is built out of a plain copy
+        // that waits in the unused part of an X buffer
+        constexpr bool can_split = VEC == 8 && sizeof(CodeT) == 1;
+        const bool split = can_split && split_layout_applies(p, n_cb, kStageBytes - kWideSplitSkip);
+        auto pick = [&](auto tail_c, auto ns_c) {
+            constexpr bool T = decltype(tail_c)::value;
+            constexpr int S = decltype(ns_c)::value;
+            return split ? prefill_kernel<VEC, CodeT, T, S, can_split> : prefill_kernel<VEC, CodeT, T, S, false>;
+        };
+        using std::integral_constant;
+        auto kern = ns == 4   ? (tail ? pick(std::true_type{}, integral_constant<int, 4>{}) : pick(std::false_type{}, integral_constant<int, 4>{}))
+                    : ns == 3 ? (tail ? pick(std::true_type{}, integral_constant<int, 3>{}) : pick(std::false_type{}, integral_constant<int, 3>{}))
+                              : (tail ? pick(std::true_type{}, integral_constant<int, 2>{}) : pick(std::false_type{}, integral_constant<int, 2>{}));
         hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
@@ -865,7 +893,10 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return hipErrorInvalidValue;
         const int tiles_n = (p.N - n_split + BNN - 1) / BNN;
         const size_t smem = lds_bytes_narrow<VEC, CodeT>(p);
-        auto kern = tail ? prefill_narrow_kernel<VEC, CodeT, true> : prefill_narrow_kernel<VEC, CodeT, false>;
+        constexpr bool can_split = VEC == 8 && sizeof(CodeT) == 1;
+        const bool split = can_split && split_layout_applies(p, codebooks_per_tile(p, BNN), kStageBytes);
+        auto kern = split ? (tail ? prefill_narrow_kernel<VEC, CodeT, true, can_split> : prefill_narrow_kernel<VEC, CodeT, false, can_split>)
+                          : (tail ? prefill_narrow_kernel<VEC, CodeT, true, false> : prefill_narrow_kernel<VEC, CodeT, false, false>);
         hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,

@@ -113,10 +113,22 @@ __device__ __forceinline__ uint32_t read_codes(const uint8_t *p)
 // `zero_off` instead (a step past the end of K).  An operand is fetched in two halves because a
 // 16-byte gather with its bank conflicts holds the wave's issue longer than the gap between two
 // MFMAs.
-template <int VEC, typename CodeT, bool TAIL>
+// SPLIT (8-vectors, 256 entries): a codebook lies in the LDS as two tables, the first 8 bytes of
+// every entry and, kSplitHi bytes on, the second 8 bytes.  A half gather at a 16-byte stride reaches
+// only every other pair of the 64 banks; at an 8-byte stride it spreads over all of them, and
+// random codewords collide less often.
+constexpr uint32_t kSplitEntries = 256, kSplitHi = kSplitEntries * 8;
+
+template <int VEC, typename CodeT, bool TAIL, bool SPLIT = false>
 __device__ __forceinline__ half4_t gather4(const uint8_t *lds, uint32_t book, uint32_t cr, int h, bool zero, uint32_t zero_off)
 {
     constexpr int CPO = 8 / VEC, BITS = 8 * (int)sizeof(CodeT);
+    static_assert(!SPLIT || VEC == 8, "the split layout is for 16-byte entries");
+    if constexpr (SPLIT) {
+        uint32_t a = book + cr * 8u + (h ? kSplitHi : 0u);
+        if (TAIL) a = zero ? zero_off : a;
+        return *reinterpret_cast<const half4_t *>(lds + a);
+    }
     auto at = [&](int c, int byte_off) {
         const uint32_t code = CPO == 1 ? cr : (cr >> (BITS * c)) & ((1u << BITS) - 1u);
         uint32_t a = book + code * (uint32_t)(VEC * 2);
@@ -133,6 +145,27 @@ __device__ __forceinline__ half4_t gather4(const uint8_t *lds, uint32_t book, ui
         const half2_t q1 = *reinterpret_cast<const half2_t *>(at(2 * h + 1, 0));
         return __builtin_shufflevector(q0, q1, 0, 1, 2, 3);
     }
+}
+
+// Re-lays `count` codebooks of 256 16-byte entries from a plain copy at LDS offset `src` into the
+// split layout at `dst` (all threads of the workgroup; the caller synchronises before and after).
+__device__ __forceinline__ void split_codebooks(uint8_t *lds, uint32_t src, uint32_t dst, int count, int tid, int n_threads)
+{
+    for (int i = tid; i < count * (int)kSplitEntries; i += n_threads) {
+        const int g = i / (int)kSplitEntries, e = i % (int)kSplitEntries;
+        const uint4_t v = *reinterpret_cast<const uint4_t *>(lds + src + i * 16);
+        *reinterpret_cast<uint2_t *>(lds + dst + g * (2 * kSplitHi) + e * 8) = uint2_t{v[0], v[1]};
+        *reinterpret_cast<uint2_t *>(lds + dst + g * (2 * kSplitHi) + kSplitHi + e * 8) = uint2_t{v[2], v[3]};
+    }
+}
+
+// whether a tile's codebooks can take the split layout, given the bytes free for the plain copy
+inline bool split_layout_applies(const ProblemB &p, int codebooks, size_t temp_bytes)
+{
+#ifdef VQ_NO_SPLIT
+    return false;
+#endif
+    return p.vec == 8 && p.code_bits == 8 && p.entries == (int)kSplitEntries && (size_t)codebooks * 2 * kSplitHi <= temp_bytes;
 }
 
 constexpr size_t kLdsLimit = 160 * 1024;

@@ -38,7 +38,8 @@ constexpr int small_code_bufs(int ns)
     return PrefillCfg<VEC, CodeT>::STAGES == 1 ? ns : (ns - 1) / 2 + 2;
 }
 
-template <int VEC, typename CodeT, int NS>
+// SPLIT: the codebooks lie in the LDS in the split layout (vq_prefill_common.h).
+template <int VEC, typename CodeT, int NS, bool SPLIT>
 __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t *__restrict__ x,
                                                                     const CodeT *__restrict__ codes,
                                                                     const half_t *__restrict__ cb,
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
         cr[j] = read_codes<C::RB>(smem + code_rd + cbuf * kTile + (pos / 16) * (SBN * 16) + j * 256 + pos % 16);
     };
     auto load_w_half = [&](int set, int j, int h) {
-        const half4_t v = gather4<VEC, CodeT, false>(smem, book[j], cr[j], h, false, 0);
+        const half4_t v = gather4<VEC, CodeT, false, SPLIT>(smem, book[j], cr[j], h, false, 0);
         if (h == 0) wlo[set][j] = v;
         else whi[set][j] = v;
     };
@@ -160,8 +161,10 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
         const int n16 = cb_lds_count * cb_bytes / 16;
         const int g_total_16 = (int)(((int64_t)((N + rows_per_cb - 1) / rows_per_cb - g_first) * cb_bytes) / 16);
         // past the last codebook: read its last 16 bytes again
+        // SPLIT: into the last X buffer first (free until stage 0 issues the loads of stage D), re-laid below
+        const int dst = SPLIT ? D * kSmallStage : kCbBase;
         for (int i0 = wave * 64; i0 < n16; i0 += kThreads)
-            load_to_lds_16(kCbBase + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
+            load_to_lds_16(dst + i0 * 16, (uint32_t)min(i0 + lane, g_total_16 - 1) * 16u, src);
     }
 #pragma unroll
     for (int d = 0; d < D; d++) {
@@ -183,6 +186,10 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
         wait_vmcnt<in_flight>();
     }
     __syncthreads();
+    if constexpr (SPLIT) {
+        split_codebooks(smem, D * kSmallStage, kCbBase, cb_lds_count, tid, kThreads);
+        __syncthreads();
+    }
 
     int buf = 0, cbuf = 0;
     // step 0 of stage 0: all of its operands; then the codes of step 1
@@ -349,7 +356,10 @@ hipError_t launch_small_typed(const ProblemB &p, hipStream_t s)
     if (!small_cfg_supports<VEC, CodeT>(p)) return hipErrorInvalidValue;
     const int tiles_m = (p.M + SBM - 1) / SBM, tiles_n = (p.N + SBN - 1) / SBN;
     const size_t smem = lds_bytes_small<VEC, CodeT>(p, 4);
-    auto kern = prefill_small_kernel<VEC, CodeT, 4>;
+    // the split codebook layout is built out of a copy in the last X buffer
+    constexpr bool can_split = VEC == 8 && sizeof(CodeT) == 1;
+    const bool split = can_split && split_layout_applies(p, codebooks_per_tile(p, SBN), kSmallStage);
+    auto kern = split ? prefill_small_kernel<VEC, CodeT, 4, can_split> : prefill_small_kernel<VEC, CodeT, 4, false>;
     const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), smem, s, p.x,
