@@ -16,6 +16,15 @@ run:
 
 try:;$(MAKE) compile;$(MAKE) run
 
+# the reference's harness flow (its bench.py) with its environment controls KERNELS / TEST_GEMM / PROFILING
+harness:
+	KERNELS=$(if $(filter all,$(KERNELS)),s2_128,$(KERNELS)) $(PYTHON) -m vq_gemm_amd.harness
+
+# every kernel variant timed on one shape, next to the automatic choice: make tune SHAPE="512 4096 4096"
+SHAPE ?= 512 4096 4096 8 256 32 8
+tune:
+	$(PYTHON) -m vq_gemm_amd.tune $(SHAPE)
+
 test:
 	$(PYTHON) -m pytest tests -x -q -m "not gpu"
 
@@ -30,4 +39,4 @@ profile:
 clean:
 	@rm -rf build vq_gemm_amd/lib oracle/libvq_oracle.so
 
-.PHONY: setup compile run try test test-gpu profile clean
+.PHONY: setup compile run try harness tune test test-gpu profile clean

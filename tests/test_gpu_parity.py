@@ -570,6 +570,16 @@ def test_harness_with_the_reference_controls(kernel):
     harness.run(kernel, profiling=True, M=128, K=64, N=32)
 
 
+def test_tune_reports_every_variant_and_the_automatic_choice():
+    from vq_gemm_amd import tune
+    _say("tune 300 512 520")
+    r = tune.tune(300, 512, 520, 8, 256, 4, 8, verbose=False)
+    assert {"prefill", "prefill_small", "twopass", "auto"} <= set(r["times_us"])
+    assert r["auto_picks"] in r["times_us"] and r["hipblaslt_us"] > 0
+    # the automatic choice is never far from the best forced variant on a shape this small
+    assert r["auto_over_fastest"] < 1.5
+
+
 # shapes the tiled kernel takes (K a multiple of 64, N of 8, X taller than 96 rows): few tiles -> 256x128
 # tiles, a full device -> 256x256 tiles; ragged M and N
 TILED_GEMM = [(300, 128, 520), (512, 192, 1288), (1024, 256, 136), (1024, 128, 16384), (2048, 4096, 1280),
