@@ -116,6 +116,15 @@ int vqgemm_encode_b(const void *w, const void *codebook, void *codes_out,
                     int32_t n_codebooks, int32_t code_bits, void *stream);
 
 /*
+ * Element-wise pass behind a gate/up projection pair (the MLP shapes among the measured
+ * configurations): out[m, n] = silu(gate_up[m, n]) * gate_up[m, N + n], gate_up [M, 2N] fp16 being
+ * one fused VQ GEMM over the gate rows of W stacked on its up rows; silu(g) = g / (1 + exp(-g)),
+ * fp32 arithmetic, one rounding to fp16.  No counterpart in the reference (its e2e_gemm has no
+ * epilogue); for call sites that hold a gated MLP (vq_gemm_amd.nn.VQGatedMLP).
+ */
+int vqgemm_silu_mul(const void *gate_up, void *out, int64_t M, int64_t N, void *stream);
+
+/*
  * Plain fp16 GEMM o[M,N] = input[M,K] . w[K,N] (fp32 accumulate), the no-dequant control.
  * Replaces: torch::Tensor gemm(input, w) — reference bind.cpp:4,8, strategy_1/src.cu:171-265.
  */

@@ -149,3 +149,15 @@ def encode_b_distances(w: np.ndarray, codebook: np.ndarray) -> np.ndarray:
     g = np.arange(N, dtype=np.int64) // (N // G)
     books = cb.astype(np.float64)[g][:, None, :, :]      # [N,1,E,v]
     return ((wv - books) ** 2).sum(axis=-1)
+
+
+def silu_mul(gate_up: np.ndarray) -> np.ndarray:
+    """out[m, n] = silu(a[m, n]) * a[m, N + n] for a [M, 2N] fp16, silu(g) = g / (1 + exp(-g)), in
+    float64 with one rounding to fp16 (the element-wise pass behind a gate/up projection pair; no
+    counterpart in the reference).  Pinned in tests/test_oracle.py by known values and identities."""
+    a = np.asarray(gate_up)
+    n = a.shape[1] // 2
+    g = a[:, :n].astype(np.float64)
+    u = a[:, n:].astype(np.float64)
+    with np.errstate(over="ignore"):
+        return (g / (1.0 + np.exp(-g)) * u).astype(np.float16)

@@ -570,6 +570,51 @@ def test_harness_with_the_reference_controls(kernel):
     harness.run(kernel, profiling=True, M=128, K=64, N=32)
 
 
+@pytest.mark.parametrize("M,N", [(1, 8), (16, 11008), (33, 50), (300, 1000), (2048, 4096)])
+def test_silu_mul_kernel_against_the_oracle(M, N):
+    g = torch.Generator().manual_seed(21)
+    a = (torch.randn(M, 2 * N, generator=g) * 3).half().to(DEV)
+    a[0, 0] = 0.0
+    a[M - 1, N - 1] = 30.0
+    a[M - 1, 0] = -30.0
+    _say("silu_mul", M, N)
+    out = cabi.silu_mul(a)
+    torch.cuda.synchronize()
+    want = vo.silu_mul(_np(a))
+    # exp differs in the last fp32 bits between the device and the host: at most one fp16 step apart
+    def ordered(h):   # fp16 bit patterns on one monotonic integer scale, -0 and +0 together
+        b = h.view(np.uint16).astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7fff), b)
+    steps = np.abs(ordered(_np(out)) - ordered(want))
+    assert steps.max() <= 1, steps.max()
+    assert (steps == 0).mean() > 0.99
+
+
+def test_gated_mlp_module():
+    from vq_gemm_amd.nn import VQGatedMLP, VQLinear
+    K, H = 512, 768
+    s_gu = ProblemSpec("gu", GEOM_B, 1, K, 2 * H, 8, 256, 2, 8, codebook_3d=True, codebook_std=0.05)
+    s_d = ProblemSpec("d", GEOM_B, 1, H, K, 8, 256, 1, 8, codebook_std=0.05)
+    _, c_gu, cb_gu = make_problem(s_gu, seed=31, device=DEV)
+    _, c_d, cb_d = make_problem(s_d, seed=32, device=DEV)
+    mlp = VQGatedMLP(VQLinear(c_gu, cb_gu), VQLinear(c_d, cb_d))
+    w_gu = vo.dequant_b(_np(c_gu), _np(cb_gu)).astype(np.float64)
+    w_d = vo.dequant_b(_np(c_d), _np(cb_d)).astype(np.float64)
+    for M in (3, 200):
+        x = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).half().to(DEV)
+        _say("gated mlp", M)
+        y = mlp(x)
+        torch.cuda.synchronize()
+        # the same chain with the same rounding points: fp16 after the first product, after the gate, at the end
+        h = (_np(x).astype(np.float64) @ w_gu.T).astype(np.float16)
+        ref = vo.silu_mul(h).astype(np.float64) @ w_d.T
+        # the device's intermediate results sit one fp16 step off the host's here and there (fp32 against
+        # float64 sums at rounding boundaries), so the chain is held to the bound on the largest output
+        e1, e2 = vo.rel_err(_np(y), ref)
+        _say(f"  gated mlp M={M}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+        assert e2 <= TOL and e1 <= 0.1, (e1, e2)
+
+
 def test_tune_reports_every_variant_and_the_automatic_choice():
     from vq_gemm_amd import tune
     _say("tune 300 512 520")

@@ -339,3 +339,20 @@ def test_encoder_inverts_the_dequantiser():
     # a NaN vector keeps entry 0, whatever the codebook
     w[3, 4:8] = np.nan
     assert c_oracle.encode_b(w, cb, 8)[3, 1] == 0
+
+
+def test_silu_mul_known_values_and_an_independent_formula():
+    a = np.array([[0.0, 20.0, -20.0, 1.0, 3.0, 2.0, 5.0, 4.0]], dtype=np.float16)
+    got = vo.silu_mul(a)
+    # silu(0) = 0; silu(20) = 20 to fp16 precision; silu(-20) * 5 = -100 / (1 + e^20); silu(1) = 0.731058...
+    want = np.array([[0.0, 40.0, -100.0 / (1.0 + np.exp(20.0)), 4.0 / (1.0 + np.exp(-1.0))]]).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    rng = np.random.default_rng(3)
+    a = (rng.standard_normal((7, 26)) * 3).astype(np.float16)
+    g, u = a[:, :13].astype(np.float64), a[:, 13:].astype(np.float64)
+    other = (g * 0.5 * (1.0 + np.tanh(g / 2.0)) * u).astype(np.float16)   # silu(g) = g (1 + tanh(g/2)) / 2
+    got = vo.silu_mul(a)
+    # the two formulas round differently in the last float64 bit at most: the fp16 results agree
+    # except where the product sits on a rounding boundary
+    assert np.max(np.abs(got.view(np.int16).astype(np.int32) - other.view(np.int16).astype(np.int32))) <= 1
+    assert np.array_equal(vo.silu_mul(np.zeros((2, 6), dtype=np.float16)), np.zeros((2, 3), dtype=np.float16))

@@ -27,6 +27,7 @@ _SIGNATURES = {
     "vqgemm_dequant_a": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "vqgemm_encode_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _P]),
+    "vqgemm_silu_mul": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
     "vqgemm_select_variant_a": (ctypes.c_int, [_I64, _I64, _I64, _I32]),
     "vqgemm_error_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -192,6 +193,20 @@ def gemm_f16(x, w, out=None):
     rc = lib().vqgemm_gemm_f16(_ptr(x), _ptr(w), _ptr(out), M, K, N, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_gemm_f16")
+    return out
+
+
+def silu_mul(gate_up, out=None):
+    """out[M,N] = silu(gate_up[:, :N]) * gate_up[:, N:] for a contiguous fp16 [M, 2N] device tensor."""
+    import torch
+    M, N2 = gate_up.shape
+    if N2 % 2 != 0 or gate_up.dtype != torch.float16:
+        raise ValueError("expected an fp16 [M, 2N] tensor")
+    if out is None:
+        out = torch.empty((M, N2 // 2), dtype=torch.float16, device=gate_up.device)
+    rc = lib().vqgemm_silu_mul(_ptr(gate_up), _ptr(out), M, N2 // 2, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_silu_mul")
     return out
 
 

@@ -269,6 +269,16 @@ int vqgemm_encode_b(const void *w, const void *codebook, void *codes_out, int64_
     return static_cast<int>(launch_encode_b(static_cast<const half_t *>(w), p, codes_out, static_cast<hipStream_t>(stream)));
 }
 
+int vqgemm_silu_mul(const void *gate_up, void *out, int64_t M, int64_t N, void *stream)
+{
+    if (M < 0 || N < 0 || M > INT_MAX / 2 || N > INT_MAX / 4) return VQGEMM_E_SHAPE;
+    if (M == 0 || N == 0) return VQGEMM_OK;
+    if (!gate_up || !out) return VQGEMM_E_NULL;
+    if (!aligned(gate_up, 2) || !aligned(out, 2)) return VQGEMM_E_ALIGN;
+    return static_cast<int>(launch_silu_mul(static_cast<const half_t *>(gate_up), static_cast<half_t *>(out), M, N,
+                                            static_cast<hipStream_t>(stream)));
+}
+
 int vqgemm_dequant_a(const void *w, const void *codebook, void *w_out, int64_t K, int64_t Nc, void *stream)
 {
     if (K < 0 || Nc < 0 || K > INT_MAX / 2 || Nc > INT_MAX / 4 || Nc % 4 != 0) return VQGEMM_E_SHAPE;

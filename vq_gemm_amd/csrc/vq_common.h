@@ -99,6 +99,9 @@ hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M,
 bool fused_a_supports(const ProblemA &p);
 hipError_t launch_fused_a(const ProblemA &p, hipStream_t s);
 
+// out[M,N] = silu(a[:, :N]) * a[:, N:] for a [M, 2N]
+hipError_t launch_silu_mul(const half_t *a, half_t *out, int64_t M, int64_t N, hipStream_t s);
+
 int device_cu_count();
 
 // Raises a kernel's dynamic-LDS limit when `bytes` needs it; remembers what was granted per

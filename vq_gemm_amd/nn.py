@@ -12,7 +12,7 @@ import torch
 
 from . import cabi
 from .quantize import kmeans_quantize
-from .torch_ops import vq_linear
+from .torch_ops import silu_mul, vq_linear
 
 
 class VQLinear(torch.nn.Module):
@@ -52,3 +52,22 @@ class VQLinear(torch.nn.Module):
         g = 1 if self.codebook.dim() == 2 else self.codebook.shape[0]
         return (f"in_features={self.in_features}, out_features={self.out_features}, vec={self.codebook.shape[-1]}, "
                 f"entries={self.codebook.shape[-2]}, codebooks={g}, bias={self.bias is not None}")
+
+
+class VQGatedMLP(torch.nn.Module):
+    """down(silu(x @ Wg.T) * (x @ Wu.T)) with all three weights vector-quantised.
+
+    `gate_up` holds the gate rows of W stacked on the up rows ([2*H, K] as codes): one fused VQ GEMM
+    gives both products, an element-wise kernel applies silu(gate) * up, `down` ([K_out, H]) follows.
+    """
+
+    def __init__(self, gate_up: VQLinear, down: VQLinear):
+        super().__init__()
+        if gate_up.out_features % 2 != 0 or gate_up.out_features // 2 != down.in_features:
+            raise ValueError("gate_up must have twice as many output features as down has input features")
+        self.gate_up = gate_up
+        self.down = down
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down(silu_mul(self.gate_up(x)))

@@ -39,3 +39,19 @@ def vq_linear(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor,
 @vq_linear.register_fake
 def _vq_linear_fake(x, codes, codebook, bias=None):
     return x.new_empty(_out_shape(x, codes, codebook))
+
+
+@torch.library.custom_op("vq_gemm_amd::silu_mul", mutates_args=(), device_types="cuda")
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(gate_up[..., :N]) * gate_up[..., N:] for fp16 gate_up [..., 2N]."""
+    if gate_up.dtype != torch.float16 or gate_up.shape[-1] % 2 != 0:
+        raise ValueError("silu_mul: expected an fp16 tensor with an even last dimension")
+    a = gate_up.reshape(-1, gate_up.shape[-1]).contiguous()
+    return cabi.silu_mul(a).view(*gate_up.shape[:-1], gate_up.shape[-1] // 2)
+
+
+@silu_mul.register_fake
+def _silu_mul_fake(gate_up):
+    if gate_up.shape[-1] % 2 != 0:
+        raise ValueError("silu_mul: expected an even last dimension")
+    return gate_up.new_empty((*gate_up.shape[:-1], gate_up.shape[-1] // 2))
