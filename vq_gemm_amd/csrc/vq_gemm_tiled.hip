@@ -29,7 +29,7 @@
 //
 // K must be a multiple of 64 (and N a multiple of 8 in the NN layout); other shapes stay on the
 // simple kernel of vq_gemm_plain.hip.
-#include "vq_common.h"
+#include "vq_tile_helpers.h"
 
 #include <type_traits>
 
@@ -60,38 +60,6 @@ struct TileCfg {
 };
 
 typedef short short4_t __attribute__((__vector_size__(4 * sizeof(short))));
-
-// s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
-// compiler knows nothing about this transfer, so every consumer sits behind an explicit
-// wait_vmcnt + barrier.  `lds_base` must be wave-uniform.
-__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base), "v"(voff), "s"(sbase)
-                 : "memory");
-}
-
-// acc += a . b with the accumulator pinned to one AGPR tuple (the register allocator otherwise
-// renames the 64 accumulators from MFMA to MFMA and fills the loop with copies).  The callers keep
-// MFMAs on one accumulator 64 MFMAs apart and pad before the accumulators are read back.
-__device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, const half8_t &b)
-{
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-}
-
-__device__ __forceinline__ void st_global_16_streaming(void *p, uint4_t v)
-{
-    __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(p));
-}
 
 // Row-major part (X, or W in the NT layout): byte offset of 16-byte chunk cc (0..3) of row `row`.
 __device__ __forceinline__ int row_offset(int row, int cc)

@@ -2,7 +2,7 @@
 // 256x128 tiles; vq_prefill_small.hip: 128x128 tiles).
 #pragma once
 
-#include "vq_common.h"
+#include "vq_tile_helpers.h"
 
 namespace vq {
 
@@ -39,43 +39,6 @@ __device__ __forceinline__ int x_offset(int row, int cc)
     const int bank_row = row >> 1;
     const int pos = (((row & 1) << 3) | cc) ^ (bank_row & 15);
     return (bank_row * 16 + pos) * 16;
-}
-
-// s_waitcnt for the vector-memory counter only (gfx9 encoding: vmcnt = simm16[15:14]:[3:0]).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
-// compiler knows nothing about this transfer, so every consumer sits behind an explicit
-// wait_vmcnt + barrier.  `lds_base` must be wave-uniform.
-__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base), "v"(voff), "s"(sbase)
-                 : "memory");
-}
-
-// acc += a . b with the accumulator pinned to one AGPR tuple.  Left to itself the register
-// allocator renames the 64 four-register accumulators from MFMA to MFMA and pays for it with
-// copies at the loop edge and with spills.  The compiler cannot see into the statement, so the
-// callers keep dependent MFMAs (same accumulator) far apart and pad before the accumulators are
-// read back.
-__device__ __forceinline__ void mfma_in_place(float4_t &acc, const half8_t &a, const half8_t &b)
-{
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-}
-
-// 16-byte store of a result that this kernel does not read again: the non-temporal hint lets the
-// write leave the L2 as it is issued instead of waiting for the write-back at the end of the kernel
-// (all workgroups of a round finish at about the same time).
-__device__ __forceinline__ void st_global_16_streaming(void *p, uint4_t v)
-{
-    __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(p));
 }
 
 // The four fp32 sums of an accumulator rounded to fp16, with the bias of their columns added first.
