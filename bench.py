@@ -231,6 +231,34 @@ def main():
         others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
         others["C5"], _ = bench_config("C5", 10, 3, cold_pool=False)
 
+    # ---- the reference's own shape in its native layout, and the plain GEMM control ---------------
+    native = None
+    if not args.only_main:
+        rspec = CONFIGS["REF"]
+        xr_, wr_, cbr_ = make_problem(rspec, seed=42, device=dev)
+        yr_ = torch.empty(rspec.M, rspec.N, dtype=torch.float16, device=dev)
+        dec_ = torch.empty(rspec.K, rspec.N, dtype=torch.float16, device=dev)
+        t_fused = time_launches(lambda i: cabi.e2e_gemm_a(xr_, wr_, cbr_, out=yr_), 1, 100, 50)
+        t_two = time_launches(lambda i: cabi.e2e_gemm_a(xr_, wr_, cbr_, variant=cabi.VARIANT_TWOPASS, out=yr_,
+                                                        workspace=dec_), 1, 100, 50)
+        t_lib = time_launches(lambda i: (cabi.dequant_a(wr_, cbr_, out=dec_), cabi.ref_gemm_f16(xr_, dec_, out=yr_)), 1, 100, 50)
+        g = torch.Generator().manual_seed(7)
+        xa = torch.randn(4096, 4096, generator=g).half().to(dev)
+        wa = (torch.randn(4096, 4096, generator=g) * 0.02).half().to(dev)
+        ya = torch.empty(4096, 4096, dtype=torch.float16, device=dev)
+        t_gemm = time_launches(lambda i: cabi.gemm_f16(xa, wa, out=ya), 1, 40, 10)
+        t_gemm_lib = time_launches(lambda i: cabi.ref_gemm_f16(xa, wa, out=ya), 1, 40, 10)
+        native = {
+            "reference_shape": {"M": rspec.M, "K": rspec.K, "code_columns": rspec.N // 2, "layout": "w[K,Nc] uint8, codebook[Nc/4,256,2]",
+                                "variant": cabi.VARIANT_NAMES[cabi.select_variant_a(rspec.M, rspec.K, rspec.N // 2)],
+                                "us": t_fused * 1e6, "tflops": rspec.flops / t_fused / 1e12,
+                                "two_pass_us": t_two * 1e6, "dequant_plus_hipblaslt_us": t_lib * 1e6},
+            "plain_gemm_4096": {"us": t_gemm * 1e6, "tflops": 2 * 4096 ** 3 / t_gemm / 1e12,
+                                "hipblaslt_us": t_gemm_lib * 1e6, "hipblaslt_tflops": 2 * 4096 ** 3 / t_gemm_lib / 1e12},
+        }
+        del xr_, wr_, cbr_, yr_, dec_, xa, wa, ya
+        torch.cuda.empty_cache()
+
     # ---- CPU baseline: the reference math (gather + fp32 matmul) on the host cores -------------
     cpu = None
     if not args.skip_cpu:
@@ -289,6 +317,7 @@ def main():
                       "speedup_vs_hipblaslt": main_res["speedup_vs_hipblaslt"]},
         "deterministic_5_runs": main_res["deterministic_5_runs"],
         "other_configs": others,
+        "reference_layout_and_control": native,
     }
     if others:
         # what the matrix cores sustain on this device with random operands (register-only MFMA loop):
