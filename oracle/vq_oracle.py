@@ -27,6 +27,8 @@ Pinning status (no golden vectors exist in the reference; see tests/test_oracle.
                           indexing written the way `bench.py:46-55` writes it.
   vq_gemm_a, vq_gemm_b, gemm — pinned: integer-valued known answers computed by hand,
                           one-hot identities, fp64 cross-accumulation, the C restatement.
+  silu_mul              — pinned: closed-form values at 0, 1 and +-20, the tanh form of the
+                          same function.
 """
 from __future__ import annotations
 
