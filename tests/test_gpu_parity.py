@@ -662,6 +662,46 @@ def test_plain_gemm_tiled_kernel(M, K, N):
         assert e1 <= TOL, e1
 
 
+def test_random_shapes_plain_gemm_and_reference_layout_against_the_library_gemm():
+    """Seeded random shapes through the tiled plain GEMM ([K,N] and, by the two-pass route, [N,K]) and the
+    fused kernel for the reference's layout, each against hipBLASLt on the same (dequantised) operands."""
+    import random
+    rnd = random.Random(77)
+
+    def close(y, ref, what):
+        scale = max(ref.float().abs().max().item(), 1e-3)
+        err = ((y.float() - ref.float()).abs().max() / scale).item()
+        assert err <= TOL, (what, err)
+
+    for case in range(12):
+        M = rnd.choice([97, 130, 256, 257, 300, 513, 777, 1024])
+        K = 64 * rnd.randint(1, 24)
+        N = 8 * rnd.randint(1, 300)
+        g = torch.Generator().manual_seed(case)
+        x = torch.randn(M, K, generator=g).half().to(DEV)
+        w = (torch.randn(K, N, generator=g) * 0.05).half().to(DEV)
+        _say("random plain gemm", M, K, N)
+        close(cabi.gemm_f16(x, w), cabi.ref_gemm_f16(x, w), ("gemm", M, K, N))
+    for case in range(10):
+        M = rnd.choice([16, 97, 130, 256, 257, 300, 513, 777])
+        K = 64 * rnd.randint(1, 24)
+        Nc = 16 * rnd.randint(1, 60)
+        spec = ProblemSpec("A", GEOM_A, M, K, 2 * Nc, 2, 256, Nc // 4, 8, codebook_std=0.05)
+        x, w, cb = make_problem(spec, seed=case, device=DEV)
+        _say("random reference layout", M, K, Nc)
+        y = cabi.e2e_gemm_a(x, w, cb, variant=cabi.VARIANT_PREFILL)
+        close(y, cabi.ref_gemm_f16(x, cabi.dequant_a(w, cb)), ("A", M, K, Nc))
+    for case in range(8):
+        M = rnd.choice([97, 130, 256, 300, 513])
+        K = 64 * rnd.randint(1, 24)
+        N = rnd.randint(1, 1500)
+        spec = ProblemSpec("B", GEOM_B, M, K, N, 8, 256, 1, 8)
+        x, codes, cb = make_problem(spec, seed=case, device=DEV)
+        _say("random two-pass", M, K, N)
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_TWOPASS)
+        close(y, cabi.ref_gemm_f16(x, cabi.dequant_b(codes, cb), w_is_nk=True), ("two-pass", M, K, N))
+
+
 # ------------------------------------------------------------------ the measured configurations at full size
 def test_config_c1_full_against_golden_and_oracle():
     import json, os
