@@ -385,16 +385,17 @@ bool prefill_small_supports(const ProblemB &p)
 
 // Microseconds the kernel is expected to take, fitted to measurements: the tiles go over the
 // compute units in rounds (a second workgroup on a unit shares its LDS bandwidth, which is what
-// bounds this tile, and gains nothing); a tile costs 4 us plus K/64 stages of 0.46 us on an idle
-// device, 0.56 us when every unit works.
+// bounds this tile, and gains nothing in the main loop; it does overlap its prologue and epilogue
+// with the other's work); a tile costs 4 us plus K/64 stages of 0.46 us on an idle device, 0.56 us
+// when every unit works.
 double prefill_small_cost_us(const ProblemB &p)
 {
     if (!prefill_small_supports(p)) return 1e30;
     const int cus = device_cu_count();
     const int64_t tiles = (int64_t)((p.M + SBM - 1) / SBM) * ((p.N + SBN - 1) / SBN);
-    const int64_t rounds = (tiles + cus - 1) / cus;
+    const int64_t rounds = (tiles + cus - 1) / cus, resident_rounds = (tiles + 2 * cus - 1) / (2 * cus);
     const double busy = tiles >= cus ? 1.0 : (double)tiles / cus;
-    return (double)rounds * (4.0 + p.K / 64.0 * (0.46 + 0.10 * busy));
+    return (double)resident_rounds * 4.0 + (double)rounds * (p.K / 64.0 * (0.46 + 0.10 * busy));
 }
 
 hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s)
