@@ -305,8 +305,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *_
 // fragment loads), with the gather running two steps ahead of the matrix cores instead of between
 // two barriers.
 //
-// 256x128 tile (64 code columns, 16 codebooks), 128x64 per wave.  LDS: six X stages (96 KB), two W
-// buffers (16 KB), the codebooks (16 KB), four code tiles of two stages each (16 KB).
+// 256x128 tile (64 code columns, 16 codebooks), 128x64 per wave; or 128x128, 64x64 per wave, when
+// the taller tiles are fewer than the compute units.  LDS: six X stages (96 or 48 KB), two W buffers
+// (16 KB), the codebooks (16 KB), four code tiles of two stages each (16 KB).
 constexpr int kANP = 4;
 constexpr int kABN = 2 * kANP * 16, kAWN = kANP * 16;       // 128, 64
 constexpr int kANSX = 6;                                     // X stages in the LDS
@@ -317,19 +318,41 @@ constexpr int kACodeRow = kABN / 2;                          // code bytes of on
 constexpr int kACodeTile = 2 * kStepK * kACodeRow;           // the codes of two stages: 4 KB
 constexpr int kANSC = 4;                                     // code tiles in the LDS
 constexpr int kAXBase = 0;
-constexpr int kAWBase = kAXBase + kANSX * kXBytes;
-constexpr int kACbBase = kAWBase + 2 * kAWBytes;
-constexpr int kACodeBase = kACbBase + kACbBytes;
-constexpr size_t kALdsBytes = kACodeBase + kANSC * kACodeTile;
-static_assert(kALdsBytes <= 160 * 1024, "the fused geometry-A kernel fits the LDS");
 
+// Tile height and, with it, the LDS layout and where in a step of 4*MPA MFMAs the other work goes.
+template <int MPA>
+struct FusedACfg {
+    static constexpr int WM = MPA * 16, BM = 2 * WM;
+    static constexpr int kXBytes = BM * kStepK * 2;              // X part of a stage: 16 or 8 KB
+    static constexpr int kXLoads = kXBytes / (kThreads * 16);    // 4 or 2
+    static constexpr int kWBase = kAXBase + kANSX * kXBytes;
+    static constexpr int kCbBase = kWBase + 2 * kAWBytes;
+    static constexpr int kCodeBase = kCbBase + kACbBytes;
+    static constexpr size_t kLdsBytes = kCodeBase + kANSC * kACodeTile;
+    // MFMA slots (an MFMA index m of the step; the instruction goes behind that MFMA)
+    static constexpr int kCodeRead1 = MPA == 8 ? 2 : 1;          // second code read (the first is at 0)
+    static constexpr int kGather0 = MPA == 8 ? 9 : 3;            // eight gathers from here on
+    static constexpr int kWrite0 = MPA == 8 ? 24 : 12;           // two writes
+    static constexpr int kXIssue0 = MPA == 8 ? 1 : 13, kXIssueGap = MPA == 8 ? 5 : 2;   // global loads of X
+    static constexpr int kCodeIssue = MPA == 8 ? 21 : 14;        // the code tile load of even steps
+    static_assert(kLdsBytes <= 160 * 1024, "the fused geometry-A kernel fits the LDS");
+};
+
+template <int MPA>
 __global__ __launch_bounds__(kThreads, 1) void gemm_a_fused_kernel(const half_t *__restrict__ x,
                                                                    const uint8_t *__restrict__ codes,
                                                                    const half_t *__restrict__ cb,
                                                                    half_t *__restrict__ y, int M, int K, int Nc,
                                                                    int tiles_m, int tiles_n)
 {
+    // MPA 16-row pieces of X per wave: 8 makes the 256x128 tile, 4 a 128x128 tile for problems whose
+    // larger tiles are fewer than the compute units (every thread then dequantises as much per half
+    // as many MFMAs, and twice as many units work).
+    static_assert(MPA == 8 || MPA == 4, "8 or 4 pieces of X per wave");
+    typedef FusedACfg<MPA> A;
     constexpr int NP = kANP, WN = kAWN, BN = kABN;
+    constexpr int MP = MPA, WM = A::WM, BM = A::BM, kXBytes = A::kXBytes, kXLoads = A::kXLoads;
+    constexpr int kAWBase = A::kWBase, kACbBase = A::kCbBase, kACodeBase = A::kCodeBase;
     extern __shared__ __align__(16) uint8_t smem[];
     const int N = 2 * Nc;
     const int tid = threadIdx.x;
@@ -498,6 +521,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_a_fused_kernel(const half_t 
             mfma_in_place(acc[j][i], __builtin_shufflevector(wlo[set][j], whi[set][j], 0, 1, 2, 3, 4, 5, 6, 7),
                           xs[set][i]);
             VQ_FENCE;
+            // Between the MFMAs: the operand reads of stage+1 (X, then W in halves), the dequantisation
+            // of stage+2 (code bytes first, the gathers a good LDS latency behind them, the writes a
+            // good LDS latency behind the gathers and ahead of the step's end), the global loads.
             if (m < MP) {
                 load_x(set ^ 1, m, xbuf_next);
                 VQ_FENCE;
@@ -505,25 +531,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_a_fused_kernel(const half_t 
                 load_w(set ^ 1, (m - MP) >> 1, (m - MP) & 1, set ^ 1);
                 VQ_FENCE;
             }
-            // the dequantisation of stage+2: code bytes first, the gathers a good LDS latency behind
-            // them, the writes a good LDS latency behind the gathers and ahead of the step's end
-            if (m == 0 || m == 2) {
-                dq_read_codes(m >> 1, cq, set);
+            if (m == 0 || m == A::kCodeRead1) {
+                dq_read_codes(m == 0 ? 0 : 1, cq, set);
                 VQ_FENCE;
             }
-            if (m >= 9 && m < 17) {
-                dq_gather((m - 9) >> 2, (m - 9) & 3);
+            if (m >= A::kGather0 && m < A::kGather0 + 8) {
+                dq_gather((m - A::kGather0) >> 2, (m - A::kGather0) & 3);
                 VQ_FENCE;
             }
-            if (m == 24 || m == 25) {
-                dq_write(m - 24, set);
+            if (m == A::kWrite0 || m == A::kWrite0 + 1) {
+                dq_write(m - A::kWrite0, set);
                 VQ_FENCE;
             }
-            if (m % 5 == 1 && m / 5 < kXLoads) {
-                issue_x(m / 5, xbuf, x_ahead);
+            if (m >= A::kXIssue0 && (m - A::kXIssue0) % A::kXIssueGap == 0 && (m - A::kXIssue0) / A::kXIssueGap < kXLoads) {
+                issue_x((m - A::kXIssue0) / A::kXIssueGap, xbuf, x_ahead);
                 VQ_FENCE;
             }
-            if (set == 0 && m == 21) {
+            if (set == 0 && m == A::kCodeIssue) {
                 issue_codes(cq == 0 ? kANSC - 1 : cq - 1, c_ahead);
                 VQ_FENCE;
             }
@@ -551,7 +575,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_a_fused_kernel(const half_t 
         constexpr int kRowChunks = WN / 8, kRowsPerPass = 64 / kRowChunks;
         uint8_t *stage_out = smem + wave * (64 * kPitch);
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
+        for (int h = 0; h < MP / 4; h++) {
 #pragma unroll
             for (int ii = 0; ii < 4; ii++) {
                 const int i = 4 * h + ii;
@@ -646,12 +670,21 @@ bool fused_a_supports(const ProblemA &p)
 hipError_t launch_fused_a(const ProblemA &p, hipStream_t s)
 {
     if (!fused_a_supports(p)) return hipErrorInvalidValue;
-    const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (2 * p.Nc + kABN - 1) / kABN;
-    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(gemm_a_fused_kernel), kALdsBytes);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(gemm_a_fused_kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kALdsBytes, s, p.x, p.w, p.cb,
-                       p.y, p.M, p.K, p.Nc, tiles_m, tiles_n);
-    return hipGetLastError();
+    const int tiles_n = (2 * p.Nc + kABN - 1) / kABN;
+    // 256x128 tiles, or 128x128 where those go over the compute units in fewer rounds at four fifths of the
+    // time per round (measured at one round each: 48 against 60 us per 4096 k)
+    const int cus = device_cu_count();
+    const int64_t n_tall = (int64_t)((p.M + 255) / 256) * tiles_n, n_short = (int64_t)((p.M + 127) / 128) * tiles_n;
+    const bool tall = (double)((n_tall + cus - 1) / cus) <= 0.8 * (double)((n_short + cus - 1) / cus);
+    auto launch = [&](auto kern, int bm, size_t lds) {
+        const int tiles_m = (p.M + bm - 1) / bm;
+        const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), lds, s, p.x, p.w, p.cb, p.y, p.M, p.K,
+                           p.Nc, tiles_m, tiles_n);
+        return hipGetLastError();
+    };
+    return tall ? launch(gemm_a_fused_kernel<8>, 256, FusedACfg<8>::kLdsBytes) : launch(gemm_a_fused_kernel<4>, 128, FusedACfg<4>::kLdsBytes);
 }
 
 }  // namespace vq
