@@ -498,10 +498,10 @@ def test_empty_problems_and_rejections_on_device():
 
 
 # ------------------------------------------------------------------ geometry A (reference-native tensors)
-# the last four are shapes the fused tiled kernel takes (K % 64 == 0, Nc % 16 == 0, M > 96): ragged M and N,
-# K of two stages only, a single 16-column piece of codes
+# all but the second and the third are shapes the fused tiled kernel takes (K % 64 == 0, Nc % 16 == 0): a
+# single row, ragged M and N, K of two stages only, a single 16-column piece of codes
 @pytest.mark.parametrize("M,K,Nc", [(32, 256, 64), (5, 96, 8), (130, 512, 132), (300, 128, 80), (257, 64, 16),
-                                    (1000, 1024, 400), (520, 2048, 640)])
+                                    (1000, 1024, 400), (520, 2048, 640), (1, 64, 16), (16, 1024, 640)])
 def test_geometry_a(M, K, Nc):
     spec = ProblemSpec("A", GEOM_A, M, K, 2 * Nc, 2, 256, Nc // 4, 8, codebook_std=1.0)
     x, w, cb = make_problem(spec, seed=5, device=DEV)
@@ -511,7 +511,7 @@ def test_geometry_a(M, K, Nc):
     want = vo.dequant_a(_np(w), _np(cb))
     assert np.array_equal(_np(dec).view(np.uint16), want.view(np.uint16))
     fused_ok = K % 64 == 0 and Nc % 16 == 0
-    assert (cabi.select_variant_a(M, K, Nc) == cabi.VARIANT_PREFILL) == (fused_ok and M > 96)
+    assert (cabi.select_variant_a(M, K, Nc) == cabi.VARIANT_PREFILL) == fused_ok
     for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_TWOPASS, cabi.VARIANT_PREFILL):
         if variant == cabi.VARIANT_PREFILL and not fused_ok:
             with pytest.raises(cabi.VqGemmError) as ei:
@@ -625,10 +625,11 @@ def test_tune_reports_every_variant_and_the_automatic_choice():
     assert r["auto_over_fastest"] < 1.5
 
 
-# shapes the tiled kernel takes (K a multiple of 64, N of 8, X taller than 96 rows): few tiles -> 256x128
-# tiles, a full device -> 256x256 tiles; ragged M and N
+# shapes the tiled kernel takes (K a multiple of 64, N of 8): few tiles -> 128x128
+# tiles (the first three and the fifth), about one 256x128 tile per compute unit -> those (the seventh and eighth),
+# more -> 256x256 tiles (the fourth and the sixth); ragged M and N
 TILED_GEMM = [(300, 128, 520), (512, 192, 1288), (1024, 256, 136), (1024, 128, 16384), (2048, 4096, 1280),
-              (700, 64, 16392)]
+              (700, 64, 16392), (2000, 256, 4088), (1024, 192, 8192), (1, 64, 8), (16, 128, 520), (96, 256, 136)]
 
 
 @pytest.mark.parametrize("M,K,N", TILED_GEMM)
@@ -651,7 +652,7 @@ def test_plain_gemm_tiled_kernel(M, K, N):
     e1, _ = vo.rel_err(_np(y), ref)
     assert e1 <= TOL, e1
     # and the [N,K] layout, through the two-pass route of the VQ entry point
-    if K % 8 == 0 and M <= 1024:
+    if K % 8 == 0 and M * K <= 1024 * 1024:
         spec = ProblemSpec("t", GEOM_B, M, K, N, 8, 256, 1, 8)
         x, codes, cb = make_problem(spec, seed=8, device=DEV)
         _say("tiled gemm two-pass", M, K, N)

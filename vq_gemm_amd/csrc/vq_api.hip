@@ -45,13 +45,13 @@ namespace {
 
 bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
-// Whether the automatic choice takes the fused geometry-A kernel.  X shorter than 97 rows leaves its
-// 256-row tile mostly padding.  Its 4-byte gathers keep the LDS busier than the matrix cores, so
-// once there is more than one round of tiles the two-pass route is faster - when the caller brings
-// the scratch for it.
+// Whether the automatic choice takes the fused geometry-A kernel: at every height (a short X
+// leaves its 128-row tile mostly padding, and the kernel is still an order of magnitude ahead of the
+// scalar one).  Its 4-byte gathers keep the LDS busier than the matrix cores, so once there is more
+// than one round of tiles the two-pass route is faster - when the caller brings the scratch for it.
 bool fused_a_preferred(const ProblemA &p, bool has_workspace)
 {
-    if (p.M < 97 || !fused_a_supports(p)) return false;
+    if (p.M < 1 || !fused_a_supports(p)) return false;
     if (!has_workspace) return true;
     const int64_t tiles = (int64_t)((p.M + 255) / 256) * ((2 * p.Nc + 127) / 128);
     return tiles <= device_cu_count();

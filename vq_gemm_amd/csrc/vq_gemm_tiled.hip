@@ -37,23 +37,23 @@ namespace vq {
 
 namespace {
 
-constexpr int BM = 256;
-constexpr int WM = 128;
-constexpr int MP = WM / 16;
+constexpr int BM = 256;                              // rows of the tallest tile
 constexpr int kThreads = 256;
 constexpr int kStepK = 32;                           // k per stage
-constexpr int kXBytes = BM * kStepK * 2;             // the X part of a stage: 16 KB
-constexpr int kXLoads = kXBytes / (kThreads * 16);   // 16-byte chunks per thread: 4
 
-// The tile: NP 16-row pieces of W per wave (8: 256x256 tile, 4: 256x128).
-template <int NP>
+// The tile: MPW 16-row pieces of X and NP 16-row pieces of W per wave
+// (8, 8: 256x256 tile; 8, 4: 256x128; 4, 4: 128x128).
+template <int NP, int MPW>
 struct TileCfg {
-    static_assert(NP == 8 || NP == 4, "8 or 4 pieces of W per wave");
+    static_assert((NP == 8 || NP == 4) && (MPW == 8 || MPW == 4) && MPW >= NP, "256x256, 256x128 or 128x128 tiles");
+    static constexpr int WM = MPW * 16, BM = 2 * WM;
     static constexpr int WN = NP * 16, BN = 2 * WN;
+    static constexpr int kXBytes = BM * kStepK * 2;                // the X part of a stage: 16 or 8 KB
+    static constexpr int kXLoads = kXBytes / (kThreads * 16);      // 4 or 2
     static constexpr int kWBytes = BN * kStepK * 2;                // the W part of a stage
     static constexpr int kWLoads = kWBytes / (kThreads * 16);      // 4 or 2
-    static constexpr int kStageBytes = kXBytes + kWBytes;          // 32 or 24 KB
-    static constexpr int NS = NP == 8 ? 5 : 6;                     // stages in the LDS
+    static constexpr int kStageBytes = kXBytes + kWBytes;          // 32, 24 or 16 KB
+    static constexpr int NS = NP == 8 ? 5 : (MPW == 8 ? 6 : 8);    // stages in the LDS
     static constexpr int kLoads = kXLoads + kWLoads;               // loads per thread and stage
     static constexpr int kChunksPerK = BN / 8;                     // 16-byte chunks of a k-row (NN layout)
     static constexpr size_t kLdsBytes = (size_t)NS * kStageBytes;
@@ -72,14 +72,15 @@ __device__ __forceinline__ int row_offset(int row, int cc)
 // k-major part (W in the NN layout): the XOR applied to the chunk index of k-row `k` (below 16).
 __device__ __forceinline__ int kmajor_swizzle(int k) { return 2 * ((k & 3) | (((k >> 3) & 1) << 2)); }
 
-template <bool W_IS_KN, int NP>
+template <bool W_IS_KN, int NP, int MPW>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *__restrict__ x,
                                                                  const half_t *__restrict__ w,
                                                                  half_t *__restrict__ y, int M, int K, int N,
                                                                  int tiles_m, int tiles_n)
 {
-    typedef TileCfg<NP> C;
+    typedef TileCfg<NP, MPW> C;
     constexpr int NS = C::NS, WN = C::WN, BN = C::BN, kStageBytes = C::kStageBytes;
+    constexpr int MP = MPW, WM = C::WM, BM = C::BM, kXBytes = C::kXBytes, kXLoads = C::kXLoads;
     extern __shared__ __align__(16) uint8_t smem[];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -196,8 +197,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *_
     // sixteen: at most three other instructions fit between two MFMAs.
     constexpr int kReads = MP + (W_IS_KN ? 2 * NP : NP);
     constexpr int kReadGap = NP == 8 ? 2 : 1;   // MFMAs from one operand read to the next
-    constexpr int kLoadGap = NP == 8 ? 8 : 5;   // MFMAs from one global load to the next
-    static_assert(kReads * kReadGap <= NP * MP - 14, "the reads of a step end well ahead of its last MFMA");
+    constexpr int kLoadGap = NP == 8 ? 8 : (MP == 8 ? 5 : 4);   // MFMAs from one global load to the next
+    static_assert(kReads * kReadGap <= NP * MP - 4, "the reads of a step end ahead of its last MFMAs");
     static_assert(1 + (C::kLoads - 1) * kLoadGap < NP * MP, "the loads of a stage fit into a step");
 #define VQ_FENCE __builtin_amdgcn_sched_barrier(0)
     int buf = 0;  // buffer of the current stage
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *_
             // 4x4 quadrants of the pieces: (0,0) (1,0) (1,1) (0,1) for 8 pieces of W, (0,0) (0,1) for 4
             const int q = m >> 4, p = (m >> 2) & 3, f = m & 3;
             const int jh = NP == 8 ? ((q == 1 || q == 2) ? 1 : 0) : 0;
-            const int ih = NP == 8 ? q >> 1 : q;
+            const int ih = NP == 8 ? q >> 1 : q;   // (one quadrant only with 4 x 4 pieces)
             const int j = jh * 4 + p, i = ih * 4 + f;
             mfma_in_place(acc[j][i], __builtin_shufflevector(wlo[set][j], whi[set][j], 0, 1, 2, 3, 4, 5, 6, 7),
                           xs[set][i]);
@@ -258,7 +259,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_kernel(const half_t *_
         constexpr int kRowChunks = WN / 8, kRowsPerPass = 64 / kRowChunks;
         uint8_t *stage_out = smem + wave * (64 * kPitch);
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
+        for (int h = 0; h < MP / 4; h++) {
 #pragma unroll
             for (int ii = 0; ii < 4; ii++) {
                 const int i = 4 * h + ii;
@@ -610,12 +611,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_a_fused_kernel(const half_t 
     }
 }
 
-template <bool W_IS_KN, int NP>
+template <bool W_IS_KN, int NP, int MPW>
 hipError_t launch_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s)
 {
-    typedef TileCfg<NP> C;
-    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + C::BN - 1) / C::BN;
-    auto kern = gemm_tiled_kernel<W_IS_KN, NP>;
+    typedef TileCfg<NP, MPW> C;
+    const int tiles_m = (M + C::BM - 1) / C::BM, tiles_n = (N + C::BN - 1) / C::BN;
+    auto kern = gemm_tiled_kernel<W_IS_KN, NP, MPW>;
     const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), C::kLdsBytes);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), C::kLdsBytes, s, x, w, y, M, K, N,
@@ -634,27 +635,32 @@ bool gemm_tiled_supports(const half_t *x, const half_t *w, int M, int K, int N, 
     return (int64_t)BM * K * 2 < (int64_t)1 << 31;
 }
 
-// tile: 0 = the width expected to be faster, 1 = 256x256, 2 = 256x128
+// tile: 0 = the tile expected to be fastest, 1 = 256x256, 2 = 256x128, 3 = 128x128
 hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, bool w_is_kn, hipStream_t s,
                              int tile)
 {
     if (!gemm_tiled_supports(x, w, M, K, N, w_is_kn)) return hipErrorInvalidValue;
+#ifdef VQ_FORCE_TILE
+    tile = VQ_FORCE_TILE;   // measurement builds only
+#endif
     if (tile == 0) {
         // Rounds of tiles over the compute units.  A tile costs K/64 times a per-stage time that
         // grows with the share of the units at work (the clock drops under load): fitted to
-        // measurements, 1.2 us for the wide tile and 0.68 us for the narrow one on an idle device,
-        // 1.6 times that on a full one.
+        // measurements, 1.2 us for the 256x256 tile, 0.68 us for 256x128 and 0.40 us for 128x128 on
+        // an idle device, 1.6 times that on a full one.
         const int cus = device_cu_count();
-        const int64_t tiles_m = (M + BM - 1) / BM;
-        auto cost = [&](int64_t tiles, double per_stage) {
+        auto cost = [&](int bm, int bn, double per_stage) {
+            const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             const int64_t rounds = (tiles + cus - 1) / cus;
             const double busy = (double)tiles / (double)(rounds * cus);
             return (double)rounds * (5.0 + K / 64.0 * per_stage * (1.0 + 0.6 * busy));
         };
-        tile = cost(tiles_m * ((N + 127) / 128), 0.68) < cost(tiles_m * ((N + 255) / 256), 1.2) ? 2 : 1;
+        const double t1 = cost(256, 256, 1.2), t2 = cost(256, 128, 0.68), t3 = cost(128, 128, 0.40);
+        tile = t3 < t2 && t3 < t1 ? 3 : (t2 < t1 ? 2 : 1);
     }
-    if (tile == 2) return w_is_kn ? launch_tiled<true, 4>(x, w, y, M, K, N, s) : launch_tiled<false, 4>(x, w, y, M, K, N, s);
-    return w_is_kn ? launch_tiled<true, 8>(x, w, y, M, K, N, s) : launch_tiled<false, 8>(x, w, y, M, K, N, s);
+    if (tile == 3) return w_is_kn ? launch_tiled<true, 4, 4>(x, w, y, M, K, N, s) : launch_tiled<false, 4, 4>(x, w, y, M, K, N, s);
+    if (tile == 2) return w_is_kn ? launch_tiled<true, 4, 8>(x, w, y, M, K, N, s) : launch_tiled<false, 4, 8>(x, w, y, M, K, N, s);
+    return w_is_kn ? launch_tiled<true, 8, 8>(x, w, y, M, K, N, s) : launch_tiled<false, 8, 8>(x, w, y, M, K, N, s);
 }
 
 // Nc in whole 16-byte pieces of code bytes, K in whole pairs of stages, 16-byte aligned operands.
