@@ -379,6 +379,45 @@ def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
     assert torch.equal(clone(x), layer(x))
 
 
+def test_residual_stages_accumulate_in_one_fused_gemm():
+    """Additive quantisation: every stage lowers the error, the merged codes index the merged codebook
+    stage by stage, and the layer's one GEMM over [X, X] equals X times the sum of the stage weights."""
+    from vq_gemm_amd.nn import VQLinear
+    from vq_gemm_amd.quantize import residual_quantize
+    g = torch.Generator(device="cpu").manual_seed(21)
+    N, K, v = 512, 1024, 8
+    w = (torch.randn(N, K, generator=g) * 0.05).half().to(DEV)
+    for entries, stages, G, dtype in ((128, 2, 2, torch.uint8), (256, 3, 1, torch.uint16)):
+        _say("residual quantiser", entries, stages, G)
+        codes, cb, hist = residual_quantize(w, v, entries, stages=stages, n_codebooks=G, iters=3, seed=3)
+        _say("    mse per element after each stage:", ["%.3e" % h for h in hist])
+        J = K // v
+        assert codes.shape == (N, stages * J) and codes.dtype == dtype and cb.shape == (G, stages * entries, v)
+        assert all(hist[s + 1] < 0.9 * hist[s] for s in range(stages - 1))
+        c = _np(codes).astype(np.int64)
+        for s in range(stages):
+            blk = c[:, s * J:(s + 1) * J]
+            assert blk.min() >= s * entries and blk.max() < (s + 1) * entries
+        # the weight: sum over the stages of the oracle's dequantisation of each stage's block
+        wd = vo.dequant_b(_np(codes), _np(cb)).astype(np.float64)          # [N, stages*K]
+        w_sum = wd.reshape(N, stages, K).sum(axis=1)
+        assert float(((w_sum - _np(w).astype(np.float64)) ** 2).mean()) == pytest.approx(hist[-1], rel=1e-3)
+        layer = VQLinear(codes, cb, k_repeat=stages)
+        assert layer.in_features == K and layer.out_features == N
+        assert np.array_equal(_np(layer.dequantized_weight()), w_sum.astype(np.float32).astype(np.float16))
+        for M in (1, 16, 300):
+            x = torch.randn(M, K, generator=g).half().to(DEV)
+            _say("residual layer", entries, stages, M)
+            y = layer(x)
+            torch.cuda.synchronize()
+            e1, _ = vo.rel_err(_np(y), _np(x).astype(np.float64) @ w_sum.T)
+            assert e1 <= TOL, (entries, stages, M, e1)
+    layer = VQLinear.from_float(w, vec=v, entries=128, iters=2, residual_stages=2)
+    assert layer.k_repeat == 2 and layer.codes.shape == (N, 2 * K // v)
+    with pytest.raises(ValueError):
+        VQLinear(layer.codes, layer.codebook, k_repeat=3)
+
+
 def test_registered_op_traces_and_matches_eager():
     """torch.ops.vq_gemm_amd.vq_linear: the fake implementation agrees with the device one (opcheck)
     and a layer traced by torch.compile (no code generation: the aot_eager backend) gives the eager result."""

@@ -356,3 +356,20 @@ def test_silu_mul_known_values_and_an_independent_formula():
     # except where the product sits on a rounding boundary
     assert np.max(np.abs(got.view(np.int16).astype(np.int32) - other.view(np.int16).astype(np.int32))) <= 1
     assert np.array_equal(vo.silu_mul(np.zeros((2, 6), dtype=np.float16)), np.zeros((2, 3), dtype=np.float16))
+
+
+def test_additive_stages_side_by_side_along_k_known_answer():
+    """The residual mode's identity, pinned by hand: stages laid side by side along K with their
+    indices offset into a merged codebook, multiplied against [X, X], give X times the sum of the
+    stage weights."""
+    # stage 0 entries 0..1, stage 1 entries 2..3 (vectors of two)
+    cb = np.array([[1, 2], [3, 4], [10, 20], [30, 40]], dtype=np.float16)
+    stage0 = np.array([[0, 1], [1, 1]], dtype=np.uint8)          # W0 rows: [1 2 3 4], [3 4 3 4]
+    stage1 = np.array([[1, 0], [0, 0]], dtype=np.uint8) + 2      # W1 rows: [30 40 10 20], [10 20 10 20]
+    codes = np.concatenate([stage0, stage1], axis=1)
+    x = np.array([[1, 0, 0, 0], [1, 1, 1, 1], [2, -1, 0, 3]], dtype=np.float16)
+    # W0 + W1 rows: [31 42 13 24], [13 24 13 24]
+    want = np.array([[31, 13], [110, 74], [62 - 42 + 72, 26 - 24 + 72]], dtype=np.float16)
+    xx = np.concatenate([x, x], axis=1)
+    for fn in (vo.vq_gemm_b, c_oracle.vq_gemm_b):
+        assert np.array_equal(fn(xx, codes, cb), want), fn

@@ -11,14 +11,20 @@ from __future__ import annotations
 import torch
 
 from . import cabi
-from .quantize import kmeans_quantize
+from .quantize import kmeans_quantize, residual_quantize
 from .torch_ops import silu_mul, vq_linear
 
 
 class VQLinear(torch.nn.Module):
-    """y = x @ W.T + bias with W[n, j*vec + t] = codebook[n // (N/G)][codes[n, j]][t]."""
+    """y = x @ W.T + bias with W[n, j*vec + t] = codebook[n // (N/G)][codes[n, j]][t].
 
-    def __init__(self, codes: torch.Tensor, codebook: torch.Tensor, bias: torch.Tensor | None = None):
+    With `k_repeat` = S > 1 the codes hold S additive stages side by side along K (see
+    `vq_gemm_amd.quantize.residual_quantize`): the layer's weight is the sum of the S [N, K] blocks of
+    the dequantised [N, S*K] matrix, and the input is repeated S times along K before the one fused
+    GEMM, so that all stages accumulate in the same fp32 sums.
+    """
+
+    def __init__(self, codes: torch.Tensor, codebook: torch.Tensor, bias: torch.Tensor | None = None, k_repeat: int = 1):
         super().__init__()
         if codes.dtype not in (torch.uint8, torch.uint16) or codes.dim() != 2:
             raise ValueError("codes must be a [N, K/vec] uint8 or uint16 tensor")
@@ -27,31 +33,45 @@ class VQLinear(torch.nn.Module):
         self.register_buffer("codes", codes.contiguous())
         self.register_buffer("codebook", codebook.contiguous())
         self.register_buffer("bias", None if bias is None else bias.to(torch.float16).contiguous())
+        if k_repeat < 1 or (codes.shape[1] * codebook.shape[-1]) % k_repeat != 0:
+            raise ValueError("k_repeat must divide the dequantised row length")
+        self.k_repeat = k_repeat
         self.out_features = codes.shape[0]
-        self.in_features = codes.shape[1] * codebook.shape[-1]
+        self.in_features = codes.shape[1] * codebook.shape[-1] // k_repeat
         if self.bias is not None and self.bias.shape != (self.out_features,):
             raise ValueError("bias must have one entry per output feature")
 
     @classmethod
     def from_float(cls, weight: torch.Tensor, vec: int = 8, entries: int = 256, n_codebooks: int = 1,
-                   bias: torch.Tensor | None = None, iters: int = 10, seed: int = 0) -> "VQLinear":
-        """Quantise an fp16 weight [N, K] on the GPU (Lloyd iterations around the HIP encoder)."""
+                   bias: torch.Tensor | None = None, iters: int = 10, seed: int = 0, residual_stages: int = 1) -> "VQLinear":
+        """Quantise an fp16 weight [N, K] on the GPU (Lloyd iterations around the HIP encoder), in
+        `residual_stages` additive stages of `entries` vectors each."""
+        if residual_stages > 1:
+            codes, codebook, _ = residual_quantize(weight.to(torch.float16), vec, entries, residual_stages, n_codebooks,
+                                                   iters, seed)
+            return cls(codes, codebook, bias, k_repeat=residual_stages)
         codes, codebook, _ = kmeans_quantize(weight.to(torch.float16), vec, entries, n_codebooks, iters, seed)
         return cls(codes, codebook, bias)
 
     def dequantized_weight(self) -> torch.Tensor:
-        return cabi.dequant_b(self.codes, self.codebook)
+        """The weight the layer multiplies by, [N, K] fp16 (the fp32 sum of the stages, rounded once)."""
+        w = cabi.dequant_b(self.codes, self.codebook)
+        if self.k_repeat == 1:
+            return w
+        return w.view(self.out_features, self.k_repeat, self.in_features).float().sum(dim=1).half()
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.dtype != torch.float16 or x.shape[-1] != self.in_features:
             raise ValueError(f"expected an fp16 input with {self.in_features} features")
+        if self.k_repeat > 1:
+            x = x.repeat(*([1] * (x.dim() - 1)), self.k_repeat)
         return vq_linear(x, self.codes, self.codebook, self.bias)
 
     def extra_repr(self) -> str:
         g = 1 if self.codebook.dim() == 2 else self.codebook.shape[0]
         return (f"in_features={self.in_features}, out_features={self.out_features}, vec={self.codebook.shape[-1]}, "
-                f"entries={self.codebook.shape[-2]}, codebooks={g}, bias={self.bias is not None}")
+                f"entries={self.codebook.shape[-2]}, codebooks={g}, stages={self.k_repeat}, bias={self.bias is not None}")
 
 
 class VQGatedMLP(torch.nn.Module):

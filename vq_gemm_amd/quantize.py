@@ -5,6 +5,14 @@ the step before the path for real weights.  Plain Lloyd iterations per codebook 
 assignment step (by far the heaviest: every vector against every entry) runs in the library's HIP
 encoder (vqgemm_encode_b), the centroid update is a handful of torch reductions on the device.
 Nothing here runs on the CPU and nothing falls back to it.
+
+`residual_quantize` is the additive ("residual") mode the reference names in an unused macro
+(`RESIDUAL`, strategy_1/src.cu:18-19) and never implements: W ~ sum over stages s of
+codebook_s[codes_s], stage s quantising what the stages before it left.  It needs no kernel of its
+own: X.(W_0 + W_1).T = [X, X].[W_0, W_1].T, so the stages are laid side by side along K - codes
+[N, S*K/vec] with stage s's indices offset by s*entries into one merged codebook of S*entries
+vectors - and the fused GEMM multiplies them against X repeated S times along K, all stages
+accumulating in the same fp32 sums.
 """
 from __future__ import annotations
 
@@ -57,3 +65,38 @@ def kmeans_quantize(w, vec: int, entries: int, n_codebooks: int = 1, iters: int 
         # an entry nothing was assigned to keeps its value
         codebook = torch.where(counts[:, :, None] > 0, mean, codebook.float()).half().contiguous()
     return codes, codebook, history
+
+
+def residual_quantize(w, vec: int, entries: int, stages: int = 2, n_codebooks: int = 1, iters: int = 10, seed: int = 0):
+    """Additive quantisation of W [N,K] (fp16, on the GPU) in `stages` rounds of `kmeans_quantize`,
+    each on the residual of the rounds before it.
+
+    Returns (codes [N, stages*K/vec], codebook [G, stages*entries, vec] fp16, history): columns
+    [s*K/vec, (s+1)*K/vec) of the codes belong to stage s and index rows [s*entries, (s+1)*entries)
+    of the merged codebook; uint8 while stages*entries <= 256, else uint16.  history[s] is the mean
+    squared error per element of the sum of stages 0..s against W.  The layer multiplies them against
+    X repeated `stages` times along K (`vq_gemm_amd.nn.VQLinear(..., k_repeat=stages)`).
+    """
+    import torch
+
+    if stages < 1:
+        raise ValueError("stages must be at least 1")
+    if stages * entries > 65536:
+        raise ValueError("stages * entries must fit 16-bit codes")
+    if w.dtype != torch.float16 or w.dim() != 2 or not w.is_cuda:
+        raise ValueError("w must be a 2-D fp16 tensor on the GPU")
+    target = w.float()
+    approx = torch.zeros_like(target)
+    wide = stages * entries > 256
+    all_codes, all_books, history = [], [], []
+    for s in range(stages):
+        residual = (target - approx).half().contiguous()
+        codes, codebook, _ = kmeans_quantize(residual, vec, entries, n_codebooks, iters, seed + s)
+        approx += cabi.dequant_b(codes, codebook).float()
+        history.append(float(((approx - target) ** 2).mean()))
+        all_codes.append(codes.to(torch.int32) + s * entries)
+        all_books.append(codebook)
+    merged = torch.cat(all_codes, dim=1)
+    # (not every build converts to uint16 directly: narrow to int16, same bits)
+    merged = merged.to(torch.int16).view(torch.uint16) if wide else merged.to(torch.uint8)
+    return merged.contiguous(), torch.cat(all_books, dim=1).contiguous(), history
