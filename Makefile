@@ -36,7 +36,23 @@ profile:
 	mkdir -p build/prof
 	cd /tmp && TMPDIR=/tmp rocprofv3 --kernel-trace --stats --output-format csv -d $(CURDIR)/build/prof -o bench -- python3 $(CURDIR)/bench.py
 
-clean:
-	@rm -rf build vq_gemm_amd/lib oracle/libvq_oracle.so
+# one launch of one module under the profiler: the reference's per-variant targets (reference Makefile:24-28,53-57)
+prof-harness:
+	mkdir -p build/prof
+	cd /tmp && TMPDIR=/tmp PROFILING=TRUE KERNELS=$(KERNELS) PYTHONPATH=$(CURDIR) rocprofv3 --kernel-trace --stats --output-format csv -d $(CURDIR)/build/prof -o $(KERNELS) -- python3 -m vq_gemm_amd.harness
 
-.PHONY: setup compile run try harness tune test test-gpu profile clean
+# per-variant shorthands with the reference's names (reference Makefile:36-61)
+VARIANTS := s1 s2_128 s2_512 s3_naive s3_wasp
+define variant_targets
+try-$(subst _,-,$(1)):;$$(MAKE) compile KERNELS=$(1) && $$(MAKE) harness KERNELS=$(1)
+run-$(subst _,-,$(1)):;$$(MAKE) harness KERNELS=$(1)
+prof-$(subst _,-,$(1)):;$$(MAKE) prof-harness KERNELS=$(1)
+endef
+$(foreach v,$(VARIANTS),$(eval $(call variant_targets,$(v))))
+run-gemm-128:;TEST_GEMM=TRUE $(MAKE) harness KERNELS=s1
+run-gemm-s2:;TEST_GEMM=TRUE $(MAKE) harness KERNELS=s2_128
+
+clean:
+	@rm -rf build vq_gemm_amd/lib oracle/libvq_oracle.so figures
+
+.PHONY: setup compile run try harness tune test test-gpu profile prof-harness clean run-gemm-128 run-gemm-s2

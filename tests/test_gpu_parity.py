@@ -594,14 +594,18 @@ def test_plain_gemm_and_hipblaslt_baseline(M, K, N):
 
 
 @pytest.mark.parametrize("kernel", ["s1", "s2_128", "s3_wasp"])
-def test_harness_with_the_reference_controls(kernel):
+def test_harness_with_the_reference_controls(kernel, tmp_path):
     """vq_gemm_amd.harness: the reference harness's three calls on its own tensor layout, with its checks
     made assertions; the full reference shape through the fused module, small shapes through the others."""
     from vq_gemm_amd import harness
     full = kernel == "s2_128"
     _say("harness", kernel, "vq gemm")
-    r = harness.run(kernel, M=2048 if full else 300, K=4096 if full else 256, N=640 if full else 80, timing=False)
+    r = harness.run(kernel, M=2048 if full else 300, K=4096 if full else 256, N=640 if full else 80, timing=False,
+                    figures=None if full else str(tmp_path))
     assert r["deterministic"] and r["dequant_bit_exact"] and r["rel_err"] <= TOL
+    if not full:   # the error picture (reference bench.py:105-116) is written where asked
+        import os
+        assert r["figure"] == os.path.join(str(tmp_path), "M=300_N=80_K=256_err.png") and os.path.getsize(r["figure"]) > 1000
     _say("harness", kernel, "plain gemm")
     r = harness.run(kernel, test_gemm=True, M=200, K=128, N=136, timing=False)
     assert r["deterministic"] and r["rel_err"] <= TOL

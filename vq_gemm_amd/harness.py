@@ -13,8 +13,9 @@ position, and whether five runs give identical bits (bench.py:97-103,118-132).  
 reference it also checks: the maximum error against the fp32-accumulated reference must stay within
 2e-3 of the largest output, and the runs must be identical.  Latency and TFLOP/s come from the
 reference's protocol, 50 warm-up and 100 timed launches (strategy_1/src.cu:330-331), measured here
-around the call instead of inside it.  The error heat-map of the reference (bench.py:105-116) is
-not produced.
+around the call instead of inside it.  The picture of the absolute error over the output matrix
+(bench.py:105-116) is written to `$FIGURES/M=.._N=.._K=.._err.png` (default `./figures`; an empty
+FIGURES switches it off).
 """
 from __future__ import annotations
 
@@ -47,6 +48,27 @@ def _report(out: torch.Tensor, ref: torch.Tensor, what: str) -> float:
     return diff.max().item() / max(scale, 1e-30)
 
 
+def save_error_map(out: torch.Tensor, ref: torch.Tensor, path: str, mark_above: float = 1.0) -> str:
+    """|out - ref| over the output matrix as an image, entries above `mark_above` marked in white
+    (the reference's error picture, bench.py:105-116)."""
+    import matplotlib
+    matplotlib.use("Agg")
+    from matplotlib import pyplot as plt
+    err = (out.float() - ref.float()).abs().cpu().numpy()
+    os.makedirs(os.path.dirname(path) or ".", exist_ok=True)
+    fig, ax = plt.subplots(figsize=(8, 6))
+    image = ax.imshow(err, aspect="auto", cmap="viridis", interpolation="nearest")
+    fig.colorbar(image, ax=ax)
+    rows, cols = (err > mark_above).nonzero()
+    if rows.size:
+        ax.scatter(cols, rows, color="white", s=1)
+    ax.set_title(f"absolute error, max {err.max():.4g}, {rows.size} entries above {mark_above:g}")
+    fig.savefig(path, dpi=100)
+    plt.close(fig)
+    print(f"figure saved to {path}")
+    return path
+
+
 def _time(fn, flops: float) -> float:
     for _ in range(50):
         fn()
@@ -64,8 +86,10 @@ def _time(fn, flops: float) -> float:
 
 
 def run(kernel: str = "s2_128", test_gemm: bool = False, profiling: bool = False, M: int | None = None,
-        K: int | None = None, N: int | None = None, seed: int = 42, timing: bool = True) -> dict:
-    """One pass of the harness; returns the figures it printed.  N counts code columns (the output has 2*N)."""
+        K: int | None = None, N: int | None = None, seed: int = 42, timing: bool = True,
+        figures: str | None = None) -> dict:
+    """One pass of the harness; returns the figures it printed.  N counts code columns (the output has 2*N).
+    With `figures` (a directory) the error picture of the VQ GEMM against the library GEMM is saved there."""
     if not torch.cuda.is_available():
         raise RuntimeError("the harness needs a GPU")
     if test_gemm:
@@ -99,6 +123,8 @@ def run(kernel: str = "s2_128", test_gemm: bool = False, profiling: bool = False
         torch.cuda.synchronize()
         print(f"VQ GEMM output shape: {tuple(out.shape)}")
         result["rel_err_vs_library_gemm"] = _report(out, ref, kernel)
+        if figures:
+            result["figure"] = save_error_map(out, ref, os.path.join(figures, f"M={M}_N={N}_K={K}_err.png"))
         # the fp32-accumulated product of the same dequantised weights is the stated truth
         truth = x.float() @ w_decoded.float()
         result["rel_err"] = _report(out, truth, kernel + " (against fp32 matmul)")
@@ -132,7 +158,8 @@ def main() -> int:
     kernel = os.getenv("KERNELS", "all")
     if kernel == "all":   # the reference needs one key here (bench.py:28); take the fused default
         kernel = ops.DEFAULT_VARIANT
-    run(kernel, test_gemm=os.getenv("TEST_GEMM", "FALSE") == "TRUE", profiling=os.getenv("PROFILING", "FALSE") == "TRUE")
+    run(kernel, test_gemm=os.getenv("TEST_GEMM", "FALSE") == "TRUE", profiling=os.getenv("PROFILING", "FALSE") == "TRUE",
+        figures=os.getenv("FIGURES", "figures") or None)
     return 0
 
 
