@@ -45,6 +45,9 @@ extern "C" {
 #define VQGEMM_VARIANT_PREFILL_NARROW 5  /* the prefill kernel with 256x128 tiles, whatever the shape */
 #define VQGEMM_VARIANT_PREFILL_SMALL 6   /* the prefill kernel with 128x128 tiles, two workgroups per compute unit
                                             (medium M); K a multiple of 64, of 128 for 8-vectors with 8-bit codes */
+#define VQGEMM_VARIANT_DECODE_PACKED 7   /* VQGEMM_VARIANT_DECODE on a code matrix that vqgemm_pack_codes_b has put
+                                            in the order the kernel's lanes load it (never chosen by AUTO: the
+                                            layout is a property of the caller's data); same results bit for bit */
 
 /*
  * Fused VQ GEMM, geometry B.
@@ -123,6 +126,29 @@ int vqgemm_encode_b(const void *w, const void *codebook, void *codes_out,
  * epilogue); for call sites that hold a gated MLP (vq_gemm_amd.nn.VQGatedMLP).
  */
 int vqgemm_silu_mul(const void *gate_up, void *out, int64_t M, int64_t N, void *stream);
+
+/*
+ * Offline re-layout of a geometry-B code matrix for VQGEMM_VARIANT_DECODE_PACKED (the step before
+ * the path; the reference keeps its w tensor as generated, bench.py:84, and has no counterpart).
+ * The decode kernel's waves each own 256 k of 16 rows of W; in the plain [N, K/vec] matrix one wave
+ * load is 16 pieces of 32 or 64 bytes in 16 different rows.  The packed matrix holds the same pieces
+ * in the order the lanes ask for them,
+ *     packed[n/16][s][t][q][n%16][c] = codes[n][(s*256 + t*kw)/vec + q*cpl + c],
+ *     cpl = codes per lane load (16 bytes; 8 bytes for 8-vectors with 8-bit codes), c < cpl,
+ *     kw = 4*cpl*vec (k per wave load), s < K/256, t < 256/kw, q < 4,
+ * so that a wave load is one run of 512 or 1024 consecutive bytes.  Same size, codes unchanged.
+ * inverse != 0 turns a packed matrix back into the plain one.  K % 256 == 0, N % 16 == 0, vec 2, 4
+ * or 8, else VQGEMM_E_VARIANT; not in place.
+ */
+int vqgemm_pack_codes_b(const void *codes, void *codes_out, int64_t N, int64_t K, int32_t vec,
+                        int32_t code_bits, int32_t inverse, void *stream);
+
+/*
+ * 1 when VQGEMM_VARIANT_DECODE_PACKED serves the shape (host only, no GPU call), 0 when it does
+ * not, or a negative error for an invalid shape.
+ */
+int vqgemm_decode_packed_supports(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                                  int32_t n_codebooks, int32_t code_bits);
 
 /*
  * Plain fp16 GEMM o[M,N] = input[M,K] . w[K,N] (fp32 accumulate), the no-dequant control.

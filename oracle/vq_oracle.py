@@ -29,6 +29,11 @@ Pinning status (no golden vectors exist in the reference; see tests/test_oracle.
                           one-hot identities, fp64 cross-accumulation, the C restatement.
   silu_mul              — pinned: closed-form values at 0, 1 and +-20, the tanh form of the
                           same function.
+  pack_codes_b          — no counterpart in the reference (its w tensor is used as generated,
+                          `bench.py:84`); a permutation defined by the library's header, pinned
+                          by a hand-written known answer, by an element-by-element loop over the
+                          header's formula, by pack/unpack round trips and - on the GPU - by the
+                          fused GEMM reading W back bit-exactly through the packed matrix.
 """
 from __future__ import annotations
 
@@ -163,3 +168,29 @@ def silu_mul(gate_up: np.ndarray) -> np.ndarray:
     u = a[:, n:].astype(np.float64)
     with np.errstate(over="ignore"):
         return (g / (1.0 + np.exp(-g)) * u).astype(np.float16)
+
+
+def pack_lane_bytes(vec: int, code_bytes: int) -> int:
+    """Bytes of codes one lane of the decode kernel loads at a time: 16, or 8 where four lanes'
+    16 bytes would cover more than the 256 k a wave owns (8-vectors with 8-bit codes)."""
+    return 8 if (16 // code_bytes) * vec * 4 > 256 else 16
+
+
+def pack_codes_b(codes: np.ndarray, vec: int, inverse: bool = False) -> np.ndarray:
+    """The decode kernel's packed code layout (include/vq_gemm.h, vqgemm_pack_codes_b).
+
+    packed[n//16][s][t][q][n%16][c] = codes[n][(s*256 + t*kw)//vec + q*cpl + c], flattened in that
+    order and returned with the shape of `codes`; cpl = codes per lane load, kw = 4*cpl*vec.
+    """
+    codes = np.asarray(codes)
+    N, J = codes.shape
+    K = J * vec
+    if K % 256 != 0 or N % 16 != 0 or vec not in (2, 4, 8):
+        raise ValueError("packed layout needs K % 256 == 0, N % 16 == 0 and vec in (2, 4, 8)")
+    cpl = pack_lane_bytes(vec, codes.dtype.itemsize) // codes.dtype.itemsize
+    kw = 4 * cpl * vec
+    T, S, L = N // 16, K // 256, 256 // kw
+    if not inverse:
+        # plain [tile, r, s, t, q, c] -> packed [tile, s, t, q, r, c]
+        return np.ascontiguousarray(codes.reshape(T, 16, S, L, 4, cpl).transpose(0, 2, 3, 4, 1, 5)).reshape(N, J)
+    return np.ascontiguousarray(codes.reshape(T, S, L, 4, 16, cpl).transpose(0, 4, 1, 2, 3, 5)).reshape(N, J)

@@ -179,6 +179,52 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
     yw = cabi.e2e_gemm_b(eye, codes, cb)
     assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
     assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)
+    # The same through the packed code matrix: the re-layout against the oracle's, the GEMM bit for
+    # bit the plain layout's (same arithmetic in the same order), W read back through a one-hot X.
+    assert cabi.decode_packed_supports(M, K, N, v, E, G, bits)
+    packed = cabi.pack_codes_b(codes, v)
+    assert np.array_equal(_np(packed), vo.pack_codes_b(_np(codes), v))
+    assert torch.equal(cabi.pack_codes_b(packed, v, inverse=True), codes)
+    yp = cabi.e2e_gemm_b(x, packed, cb, variant=cabi.VARIANT_DECODE_PACKED)
+    assert torch.equal(yp, y)
+    ywp = cabi.e2e_gemm_b(eye, packed, cb, variant=cabi.VARIANT_DECODE_PACKED)
+    assert np.array_equal(_np(ywp).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+
+
+def test_packed_codes_small_shapes_bias_and_rejections():
+    for (M, K, N, v, E, G, bits) in [(1, 256, 16, 8, 256, 1, 8), (5, 512, 48, 4, 4096, 1, 16), (16, 256, 32, 2, 256, 2, 8),
+                                     (33, 1024, 64, 8, 300, 4, 16), (3, 768, 32, 2, 1000, 1, 16), (16, 4096, 4096, 8, 256, 1, 8)]:
+        spec = ProblemSpec("packed", GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+        x, codes, cb = make_problem(spec, seed=5, device=DEV)
+        _say("packed decode", spec)
+        packed = cabi.pack_codes_b(codes, v)
+        assert np.array_equal(_np(packed), vo.pack_codes_b(_np(codes), v))
+        bias = torch.randn(N, device=DEV).half()
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE, bias=bias)
+        yp = cabi.e2e_gemm_b(x, packed, cb, variant=cabi.VARIANT_DECODE_PACKED, bias=bias)
+        assert torch.equal(yp, y)
+        # the unrounded product in float64 (the oracle's own GEMM returns it rounded to fp16)
+        ref = _np(x).astype(np.float64) @ vo.dequant_b(_np(codes), _np(cb)).astype(np.float64).T + _np(bias).astype(np.float64)
+        e1, _ = vo.rel_err(_np(yp), ref)
+        assert e1 <= TOL
+    # shapes outside the batched kernel: no packed layout, and the packed variant refuses them
+    codes = torch.zeros(16, 40, dtype=torch.uint8, device=DEV)          # K = 320
+    with pytest.raises(cabi.VqGemmError) as ei:
+        cabi.pack_codes_b(codes, 8)
+    assert ei.value.code == -4
+    assert not cabi.decode_packed_supports(4, 320, 16, 8, 256, 1, 8)
+    assert not cabi.decode_packed_supports(4, 512, 24, 8, 256, 1, 8)    # N not a multiple of 16
+    x = torch.zeros(4, 320, dtype=torch.float16, device=DEV)
+    cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
+    with pytest.raises(cabi.VqGemmError) as ei:
+        cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_PACKED)
+    assert ei.value.code == -4
+    with pytest.raises(cabi.VqGemmError):                                # not in place
+        c2 = torch.zeros(16, 32, dtype=torch.uint8, device=DEV)
+        cabi.pack_codes_b(c2, 8, out=c2)
+    # the automatic choice never takes the packed variant
+    assert cabi.select_variant_b(1, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.pack_codes_b(torch.zeros(0, 64, dtype=torch.uint8, device=DEV), 8).shape == (0, 64)
 
 
 # Shapes that walk the prefill kernel through each of its instantiations: both super-stage
@@ -377,6 +423,14 @@ def test_vqlinear_module_matches_a_dense_layer_on_its_dequantised_weight():
     clone.load_state_dict(layer.state_dict())
     x = torch.randn(4, K, generator=g).half().to(DEV)
     assert torch.equal(clone(x), layer(x))
+    # a second copy of the codes in the decode kernel's order: short inputs read it, same bits out
+    packed = VQLinear(layer.codes, layer.codebook, bias).prepack_for_decode()
+    assert packed.codes_packed is not None and "codes_packed" not in packed.state_dict()
+    for shape in ((1, K), (2, 7, K), (300, K)):
+        x = torch.randn(*shape, generator=g).half().to(DEV)
+        assert torch.equal(packed(x), layer(x))
+    with pytest.raises(ValueError):
+        VQLinear(layer.codes[:, :40], layer.codebook).prepack_for_decode()    # K = 320
 
 
 def test_residual_stages_accumulate_in_one_fused_gemm():

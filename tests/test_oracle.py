@@ -373,3 +373,48 @@ def test_additive_stages_side_by_side_along_k_known_answer():
     xx = np.concatenate([x, x], axis=1)
     for fn in (vo.vq_gemm_b, c_oracle.vq_gemm_b):
         assert np.array_equal(fn(xx, codes, cb), want), fn
+
+
+# ---- packed code layout of the decode kernel -------------------------------------------------
+def test_pack_codes_known_answer():
+    # 8-vectors, 8-bit codes: 8 codes per lane load, one wave load per 256 k.  16 rows x 32 codes
+    # holding code[n][j] = n*32 + j (mod 256): the packed order is k-group, then row, then the lane's
+    # 8 codes, so the first 16 pieces are codes 0..7 of rows 0..15, the next 16 codes 8..15, ...
+    N, J = 16, 32
+    codes = ((np.arange(N)[:, None] * J + np.arange(J)[None, :]) % 256).astype(np.uint8)
+    flat = vo.pack_codes_b(codes, 8).reshape(-1)
+    assert flat[:8].tolist() == codes[0, :8].tolist()
+    assert flat[8:16].tolist() == codes[1, :8].tolist()
+    assert flat[15 * 8:16 * 8].tolist() == codes[15, :8].tolist()
+    assert flat[16 * 8:17 * 8].tolist() == codes[0, 8:16].tolist()
+    assert flat[(3 * 16 + 5) * 8:(3 * 16 + 5) * 8 + 8].tolist() == codes[5, 24:32].tolist()
+
+
+@pytest.mark.parametrize("N,K,v,bits", [(32, 512, 8, 8), (16, 256, 4, 16), (48, 768, 4, 8), (16, 512, 2, 8),
+                                        (32, 256, 2, 16), (16, 1024, 8, 16)])
+def test_pack_codes_follows_the_header_formula_element_by_element(N, K, v, bits):
+    rng = np.random.default_rng(N + K + v + bits)
+    dt = np.uint8 if bits == 8 else np.uint16
+    codes = rng.integers(0, 1 << bits, size=(N, K // v)).astype(dt)
+    packed = vo.pack_codes_b(codes, v).reshape(-1)
+    cpl = (8 if (16 // (bits // 8)) * v * 4 > 256 else 16) // (bits // 8)
+    kw = 4 * cpl * v
+    i = 0
+    for tile in range(N // 16):
+        for s in range(K // 256):
+            for t in range(256 // kw):
+                for q in range(4):
+                    for r in range(16):
+                        for c in range(cpl):
+                            assert packed[i] == codes[tile * 16 + r][(s * 256 + t * kw) // v + q * cpl + c]
+                            i += 1
+    assert i == packed.size
+    assert np.array_equal(vo.pack_codes_b(vo.pack_codes_b(codes, v), v, inverse=True), codes)
+    assert sorted(packed.tolist()) == sorted(codes.reshape(-1).tolist())
+
+
+def test_pack_codes_rejects_shapes_the_kernel_does_not_take():
+    with pytest.raises(ValueError):
+        vo.pack_codes_b(np.zeros((16, 31), np.uint8), 8)
+    with pytest.raises(ValueError):
+        vo.pack_codes_b(np.zeros((8, 32), np.uint8), 8)

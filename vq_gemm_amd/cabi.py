@@ -14,8 +14,9 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 _INCLUDE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
 
 (VARIANT_AUTO, VARIANT_GENERIC, VARIANT_DECODE, VARIANT_PREFILL, VARIANT_TWOPASS, VARIANT_PREFILL_NARROW,
- VARIANT_PREFILL_SMALL) = range(7)
-VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass", 5: "prefill_narrow", 6: "prefill_small"}
+ VARIANT_PREFILL_SMALL, VARIANT_DECODE_PACKED) = range(8)
+VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass", 5: "prefill_narrow", 6: "prefill_small",
+                 7: "decode_packed"}
 
 _I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
 
@@ -26,6 +27,8 @@ _SIGNATURES = {
     "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_dequant_a": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "vqgemm_encode_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
+    "vqgemm_pack_codes_b": (ctypes.c_int, [_P, _P, _I64, _I64, _I32, _I32, _I32, _P]),
+    "vqgemm_decode_packed_supports": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
     "vqgemm_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _P]),
     "vqgemm_silu_mul": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
     "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
@@ -171,6 +174,24 @@ def encode_b(w, codebook, code_bits=None, out=None):
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_encode_b")
     return out
+
+
+def pack_codes_b(codes, vec, inverse=False, out=None):
+    """The code matrix [N, K/vec] re-laid for VARIANT_DECODE_PACKED (same shape and dtype; `inverse`
+    restores the plain matrix)."""
+    import torch
+    N, J = codes.shape
+    bits = 8 if codes.dtype == torch.uint8 else 16
+    if out is None:
+        out = torch.empty_like(codes)
+    rc = lib().vqgemm_pack_codes_b(_ptr(codes), _ptr(out), N, J * vec, vec, bits, 1 if inverse else 0, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_pack_codes_b")
+    return out
+
+
+def decode_packed_supports(M, K, N, vec, entries, n_codebooks, code_bits) -> bool:
+    return lib().vqgemm_decode_packed_supports(M, K, N, vec, entries, n_codebooks, code_bits) == 1
 
 
 def dequant_a(w, codebook, out=None):

@@ -81,6 +81,7 @@ ProblemB make_b(const void *x, const void *codes, const void *codebook, void *y,
     p.vec = vec; p.entries = entries; p.n_codebooks = n_codebooks; p.code_bits = code_bits;
     p.rows_per_cb = N > 0 ? (int)(N / n_codebooks) : 1;
     if (p.rows_per_cb < 1) p.rows_per_cb = 1;
+    p.packed = false;
     return p;
 }
 
@@ -132,7 +133,7 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
 {
     int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
     if (rc != VQGEMM_OK) return rc;
-    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_PREFILL_SMALL) return VQGEMM_E_VARIANT;
+    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_DECODE_PACKED) return VQGEMM_E_VARIANT;
     if (M == 0 || N == 0) return VQGEMM_OK;
     if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
     const uintptr_t code_align = code_bits / 8;
@@ -152,6 +153,12 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
     case VQGEMM_VARIANT_DECODE:
         if (!a16) return VQGEMM_E_ALIGN;
         if (K == 0 || !decode_supports(p)) return VQGEMM_E_VARIANT;
+        e = launch_decode_b(p, s);
+        break;
+    case VQGEMM_VARIANT_DECODE_PACKED:
+        if (!a16) return VQGEMM_E_ALIGN;
+        p.packed = true;
+        if (K == 0 || !decode_packed_supports(p)) return VQGEMM_E_VARIANT;
         e = launch_decode_b(p, s);
         break;
     case VQGEMM_VARIANT_PREFILL:
@@ -254,6 +261,32 @@ int vqgemm_dequant_b(const void *codes, const void *codebook, void *w_out, int64
     if (!aligned(w_out, 2) || !aligned(codebook, 2) || !aligned(codes, code_bits / 8)) return VQGEMM_E_ALIGN;
     const ProblemB p = make_b(nullptr, codes, codebook, nullptr, 0, K, N, vec, entries, n_codebooks, code_bits);
     return static_cast<int>(launch_dequant_b(p, static_cast<half_t *>(w_out), static_cast<hipStream_t>(stream)));
+}
+
+int vqgemm_pack_codes_b(const void *codes, void *codes_out, int64_t N, int64_t K, int32_t vec, int32_t code_bits,
+                        int32_t inverse, void *stream)
+{
+    if (N < 0 || K < 0 || N > INT_MAX / 2 || K > INT_MAX / 2) return VQGEMM_E_SHAPE;
+    if (code_bits != 8 && code_bits != 16) return VQGEMM_E_CODEBITS;
+    if (vec < 1 || K % vec != 0) return VQGEMM_E_SHAPE;
+    if (!pack_codes_supports(N, K, vec, code_bits)) return VQGEMM_E_VARIANT;
+    if (N == 0 || K == 0) return VQGEMM_OK;
+    if (!codes || !codes_out) return VQGEMM_E_NULL;
+    if (codes == codes_out) return VQGEMM_E_NULL;  // not in place: a permutation of the whole matrix
+    if (!aligned(codes, 16) || !aligned(codes_out, 16)) return VQGEMM_E_ALIGN;
+    return static_cast<int>(launch_pack_codes(codes, codes_out, N, K, vec, code_bits, inverse != 0,
+                                              static_cast<hipStream_t>(stream)));
+}
+
+int vqgemm_decode_packed_supports(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks,
+                                  int32_t code_bits)
+{
+    const int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (M == 0 || N == 0 || K == 0) return 0;
+    ProblemB p = make_b(nullptr, nullptr, nullptr, nullptr, M, K, N, vec, entries, n_codebooks, code_bits);
+    p.packed = true;
+    return decode_packed_supports(p) ? 1 : 0;
 }
 
 int vqgemm_encode_b(const void *w, const void *codebook, void *codes_out, int64_t N, int64_t K, int32_t vec,

@@ -27,6 +27,7 @@ struct ProblemB {
     int M, K, N;
     int vec, entries, n_codebooks, code_bits;
     int rows_per_cb;      // N / G
+    bool packed;          // codes are in the packed layout of the batched decode kernel (launch_pack_codes)
 };
 
 struct ProblemA {
@@ -67,6 +68,13 @@ bool decode_supports(const ProblemB &p);
 // whether the decode path is expected to beat the prefill kernel on a shape it supports
 bool decode_preferred(const ProblemB &p);
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s);
+// The packed code layout of the batched decode kernel: the pieces of the code matrix in the order
+// the kernel's lanes load them (same size, codes unchanged).  `inverse` restores the plain matrix.
+bool pack_codes_supports(int64_t N, int64_t K, int vec, int code_bits);
+hipError_t launch_pack_codes(const void *src, void *dst, int64_t N, int64_t K, int vec, int code_bits, bool inverse,
+                             hipStream_t s);
+// whether launch_decode_b takes the shape with p.packed set (the batched kernel only)
+bool decode_packed_supports(const ProblemB &p);
 // the general kernel behind launch_decode_b: one slab of at most 16 rows of X
 bool decode_general_supports(const ProblemB &p);
 hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);

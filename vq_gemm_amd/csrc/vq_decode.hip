@@ -243,7 +243,7 @@ constexpr int kStageOverTable = 1, kStageOverSlots = 2;
 __device__ __forceinline__ const half_t *bias_of() { return nullptr; }
 __device__ __forceinline__ const half_t *bias_of(const half_t *b) { return b; }
 
-template <int VEC, typename CodeT, bool REPL, int TB, typename... Bias>
+template <int VEC, typename CodeT, bool REPL, int TB, bool PACKED, typename... Bias>
 __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
                                                                const CodeT *__restrict__ codes,
                                                                const half_t *__restrict__ cb,
@@ -307,9 +307,15 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
 
     // Codes: lane offset inside a tile and chunk, scalar base per tile and chunk.  The last unit
     // may hold fewer than TB tiles.
-    const uint32_t voff = (uint32_t)((r16 * J + (w * kSliceK + kq * C::K_LANE) / VEC) * (int)sizeof(CodeT));
+    // Plain layout [N, K/VEC]: a lane load is LB bytes of row r16, the four k-groups of a wave load
+    // lie 4*LB bytes apart in each of 16 rows.  Packed layout (pack_codes_kernel below): the 64 lane
+    // loads of a wave load are contiguous, [tile][slice][load][lane], so that a wave instruction
+    // reads 64*LB consecutive bytes instead of 16 pieces of 4*LB.
+    constexpr int kLoadPitch = PACKED ? 64 * C::LB : 4 * C::LB;  // bytes between the loads of a slice
+    const uint32_t voff = PACKED ? (uint32_t)((w * C::LPT * 64 + lane) * C::LB)
+                                 : (uint32_t)((r16 * J + (w * kSliceK + kq * C::K_LANE) / VEC) * (int)sizeof(CodeT));
     const int64_t tile_bytes = (int64_t)kTileN * J * (int)sizeof(CodeT);
-    const int chunk_bytes = n_waves * kSliceK / VEC * (int)sizeof(CodeT);
+    const int chunk_bytes = n_waves * kSliceK / VEC * (int)sizeof(CodeT) * (PACKED ? kTileN : 1);
     auto load_unit = [&](int q, Codes (&cw)[TB]) {
 #pragma unroll
         for (int j = 0; j < TB; j++) {
@@ -317,9 +323,9 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
             if (tile >= tile_end) break;
             const uint8_t *sbase = reinterpret_cast<const uint8_t *>(codes) + tile * tile_bytes + chunk * chunk_bytes;
             if constexpr (C::LPT >= 1) cw[j].template load_async_s<0>(0, voff, sbase);
-            if constexpr (C::LPT >= 2) cw[j].template load_async_s<4 * C::LB>(1, voff, sbase);
-            if constexpr (C::LPT >= 3) cw[j].template load_async_s<8 * C::LB>(2, voff, sbase);
-            if constexpr (C::LPT >= 4) cw[j].template load_async_s<12 * C::LB>(3, voff, sbase);
+            if constexpr (C::LPT >= 2) cw[j].template load_async_s<kLoadPitch>(1, voff, sbase);
+            if constexpr (C::LPT >= 3) cw[j].template load_async_s<2 * kLoadPitch>(2, voff, sbase);
+            if constexpr (C::LPT >= 4) cw[j].template load_async_s<3 * kLoadPitch>(3, voff, sbase);
             static_assert(C::LPT <= 4, "at most four lane loads per slice");
         }
     };
@@ -689,7 +695,7 @@ BatchedPlan plan_batched(const ProblemB &p)
     }
 }
 
-template <int VEC, typename CodeT>
+template <int VEC, typename CodeT, bool PACKED>
 hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
 {
     typedef DecodeCfg<VEC, CodeT> C;
@@ -711,19 +717,82 @@ hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
     // a full batch of one tile is the only case with a replicated table and TB = 1
     const int tb = g.full ? C::TB : 1;
     if (p.bias) {
-        if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, const half_t *>, p.bias)
-                                   : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, const half_t *>, p.bias);
-        return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, const half_t *>, p.bias)
-                       : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, const half_t *>, p.bias);
+        if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, PACKED, const half_t *>, p.bias)
+                                   : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, PACKED, const half_t *>, p.bias);
+        return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, PACKED, const half_t *>, p.bias)
+                       : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, PACKED, const half_t *>, p.bias);
     }
-    if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1>)
-                               : launch(decode_batched_kernel<VEC, CodeT, true, C::TB>);
-    return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1>) : launch(decode_batched_kernel<VEC, CodeT, false, C::TB>);
+    if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, PACKED>)
+                               : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, PACKED>);
+    return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, PACKED>)
+                   : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, PACKED>);
+}
+
+// ---- packed code layout ---------------------------------------------------------------------
+// The batched kernel's lane (k-group kq, row r) of the wave that owns slice s loads, for load t of
+// the slice, LB bytes of row r starting at code (s*256 + t*K_WAVE + kq*K_LANE)/VEC.  The packed
+// layout stores exactly these pieces in the order the lanes ask for them:
+//     packed[tile][s][t][kq][r][LB bytes],   tile = n / 16, r = n % 16,
+// so that a wave load is one contiguous run of 64*LB bytes.  Same size as the plain matrix; the
+// permutation moves whole pieces, codes keep their values.  One thread moves one piece.
+template <int LB>
+__global__ __launch_bounds__(256) void pack_codes_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                        int64_t n_pieces, int row_bytes, bool inverse)
+{
+    typedef uint32_t piece_t __attribute__((ext_vector_type(LB / 4)));
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // index in the packed order
+    if (i >= n_pieces) return;
+    const int r = (int)(i & 15), kq = (int)((i >> 4) & 3);
+    const int64_t rest = i >> 6;  // (tile * slices + s) * lpt + t
+    const int per_tile = row_bytes / (4 * LB);  // slices * lpt
+    const int64_t tile = rest / per_tile;
+    const int st = (int)(rest - tile * per_tile);  // s * lpt + t: wave loads follow each other along the row
+    const int64_t plain = ((tile * kTileN + r) * (int64_t)row_bytes + (int64_t)st * 4 * LB + kq * LB) / LB;
+    const piece_t *s = reinterpret_cast<const piece_t *>(src);
+    piece_t *d = reinterpret_cast<piece_t *>(dst);
+    if (inverse) d[plain] = s[i];
+    else d[i] = s[plain];
+}
+
+template <int VEC, typename CodeT>
+hipError_t launch_pack(const void *src, void *dst, int64_t N, int64_t K, bool inverse, hipStream_t s)
+{
+    typedef DecodeCfg<VEC, CodeT> C;
+    static_assert(C::LPT * C::K_WAVE == kSliceK, "a slice is a whole number of wave loads");
+    const int row_bytes = (int)(K / VEC) * (int)sizeof(CodeT);
+    const int64_t n_pieces = N * row_bytes / C::LB;
+    if (n_pieces == 0) return hipSuccess;
+    const unsigned blocks = (unsigned)((n_pieces + 255) / 256);
+    hipLaunchKernelGGL(pack_codes_kernel<C::LB>, dim3(blocks), dim3(256), 0, s, static_cast<const uint8_t *>(src),
+                       static_cast<uint8_t *>(dst), n_pieces, row_bytes, inverse);
+    return hipGetLastError();
 }
 
 bool batched_supports(const ProblemB &p) { return plan_batched(p).ok; }
 
 }  // namespace
+
+bool decode_packed_supports(const ProblemB &p)
+{
+    return p.M >= 1 && p.M <= kBatchedMaxM && decode_general_supports(p) && batched_supports(p);
+}
+
+bool pack_codes_supports(int64_t N, int64_t K, int vec, int code_bits)
+{
+    return (vec == 2 || vec == 4 || vec == 8) && (code_bits == 8 || code_bits == 16) && K % kSliceK == 0 && N % kTileN == 0;
+}
+
+hipError_t launch_pack_codes(const void *src, void *dst, int64_t N, int64_t K, int vec, int code_bits, bool inverse,
+                             hipStream_t s)
+{
+    if (!pack_codes_supports(N, K, vec, code_bits)) return hipErrorInvalidValue;
+    const bool u8 = code_bits == 8;
+    switch (vec) {
+    case 8: return u8 ? launch_pack<8, uint8_t>(src, dst, N, K, inverse, s) : launch_pack<8, uint16_t>(src, dst, N, K, inverse, s);
+    case 4: return u8 ? launch_pack<4, uint8_t>(src, dst, N, K, inverse, s) : launch_pack<4, uint16_t>(src, dst, N, K, inverse, s);
+    default: return u8 ? launch_pack<2, uint8_t>(src, dst, N, K, inverse, s) : launch_pack<2, uint16_t>(src, dst, N, K, inverse, s);
+    }
+}
 
 bool decode_supports(const ProblemB &p)
 {
@@ -761,12 +830,20 @@ hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
     const bool u8 = p.code_bits == 8;
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension
+        if (p.packed) {
+            switch (p.vec) {
+            case 8: return u8 ? launch_decode_batched<8, uint8_t, true>(p, s) : launch_decode_batched<8, uint16_t, true>(p, s);
+            case 4: return u8 ? launch_decode_batched<4, uint8_t, true>(p, s) : launch_decode_batched<4, uint16_t, true>(p, s);
+            default: return u8 ? launch_decode_batched<2, uint8_t, true>(p, s) : launch_decode_batched<2, uint16_t, true>(p, s);
+            }
+        }
         switch (p.vec) {
-        case 8: return u8 ? launch_decode_batched<8, uint8_t>(p, s) : launch_decode_batched<8, uint16_t>(p, s);
-        case 4: return u8 ? launch_decode_batched<4, uint8_t>(p, s) : launch_decode_batched<4, uint16_t>(p, s);
-        default: return u8 ? launch_decode_batched<2, uint8_t>(p, s) : launch_decode_batched<2, uint16_t>(p, s);
+        case 8: return u8 ? launch_decode_batched<8, uint8_t, false>(p, s) : launch_decode_batched<8, uint16_t, false>(p, s);
+        case 4: return u8 ? launch_decode_batched<4, uint8_t, false>(p, s) : launch_decode_batched<4, uint16_t, false>(p, s);
+        default: return u8 ? launch_decode_batched<2, uint8_t, false>(p, s) : launch_decode_batched<2, uint16_t, false>(p, s);
         }
     }
+    if (p.packed) return hipErrorInvalidValue;  // only the batched kernel reads the packed layout
     // The general kernel multiplies 16 rows of X per launch; taller X goes in slabs, one launch
     // each: still far better than a 256-row MFMA tile that is mostly padding and fills only
     // N/256 compute units.

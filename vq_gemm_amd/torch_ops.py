@@ -41,6 +41,25 @@ def _vq_linear_fake(x, codes, codebook, bias=None):
     return x.new_empty(_out_shape(x, codes, codebook))
 
 
+@torch.library.custom_op("vq_gemm_amd::vq_linear_packed", mutates_args=(), device_types="cuda")
+def vq_linear_packed(x: torch.Tensor, codes_packed: torch.Tensor, codebook: torch.Tensor,
+                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`vq_linear` on a code matrix in the decode kernel's packed layout (`cabi.pack_codes_b`):
+    the decode kernel only, for the shapes `cabi.decode_packed_supports` accepts."""
+    shape = _out_shape(x, codes_packed, codebook)
+    if x.dtype != torch.float16 or codebook.dtype != torch.float16:
+        raise ValueError("vq_linear_packed: x and codebook must be float16")
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    y = cabi.e2e_gemm_b(x2, codes_packed.contiguous(), codebook.contiguous(), variant=cabi.VARIANT_DECODE_PACKED,
+                        bias=None if bias is None else bias.contiguous())
+    return y.view(shape)
+
+
+@vq_linear_packed.register_fake
+def _vq_linear_packed_fake(x, codes_packed, codebook, bias=None):
+    return x.new_empty(_out_shape(x, codes_packed, codebook))
+
+
 @torch.library.custom_op("vq_gemm_amd::silu_mul", mutates_args=(), device_types="cuda")
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     """silu(gate_up[..., :N]) * gate_up[..., N:] for fp16 gate_up [..., 2N]."""
