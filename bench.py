@@ -92,7 +92,7 @@ def main():
     import torch
 
     from vq_gemm_amd import cabi
-    from vq_gemm_amd.problems import CONFIGS, make_problem
+    from vq_gemm_amd.problems import CONFIGS, GEOM_B, ProblemSpec, make_problem
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -137,6 +137,8 @@ def main():
         gen = torch.Generator(device=dev).manual_seed(1234)
         pool = [codes] + [torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev,
                                         dtype=torch.int32).to(spec.code_dtype) for _ in range(n_bufs - 1)]
+        if args.probe_variant == cabi.VARIANT_DECODE_PACKED:   # that variant reads code matrices re-laid offline
+            pool = [cabi.pack_codes_b(c, spec.vec) for c in pool]
         y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
@@ -181,7 +183,7 @@ def main():
             return e0.elapsed_time(e1) * 1e-3 / steps
 
     def bench_config(name, steps, warmup, cold_pool):
-        spec = CONFIGS[name]
+        spec = CONFIGS[name] if isinstance(name, str) else name
         x, codes, cb = make_problem(spec, seed=42, device=dev)
         n_bufs = max(1, min(512, POOL_BYTES // max(spec.code_bytes, 1))) if cold_pool else 1
         pool = [codes]
@@ -212,6 +214,24 @@ def main():
             "speedup_vs_hipblaslt": t_blas / t_cold,
             "code_buffers_rotated": n_bufs, "steps": steps,
         }
+        # The same launches on code matrices re-laid offline in the order the decode kernel's lanes
+        # load them (vqgemm_pack_codes_b): beside the figures above, which stay on the plain
+        # [N, K/vec] tensor of the reference's call.
+        dims = (spec.M, spec.K, spec.N, spec.vec, spec.entries, spec.n_codebooks, spec.code_bits)
+        if cold_pool and cabi.decode_packed_supports(*dims):
+            ppool = [cabi.pack_codes_b(c, spec.vec) for c in pool]
+            launch_p = lambda i: cabi.e2e_gemm_b(x, ppool[i], cb, out=y, variant=cabi.VARIANT_DECODE_PACKED)
+            tp_cold = time_launches(launch_p, n_bufs, steps, warmup)
+            tp_warm = time_launches(lambda i: launch_p(0), 1, steps, warmup)
+            y_plain = cabi.e2e_gemm_b(x, pool[0], cb, variant=cabi.VARIANT_DECODE).clone()
+            res["prepacked_codes"] = {
+                "us": tp_cold * 1e6, "us_warm_cache": tp_warm * 1e6,
+                "algorithmic_gbps": spec.algorithmic_bytes / tp_cold / 1e9,
+                "hbm_roofline_frac": spec.algorithmic_bytes / tp_cold / 1e9 / HBM_PEAK_GBPS,
+                "speedup_vs_hipblaslt": t_blas / tp_cold,
+                "bit_identical_to_plain_layout": bool(torch.equal(launch_p(0), y_plain)),
+            }
+            del ppool
         # run-to-run determinism, as the reference harness reports it (bench.py:118-132)
         y0 = cabi.e2e_gemm_b(x, codes, cb).clone()
         res["deterministic_5_runs"] = all(torch.equal(cabi.e2e_gemm_b(x, codes, cb), y0) for _ in range(4))
@@ -227,6 +247,10 @@ def main():
     others = {}
     if not args.only_main:
         others["C3"], _ = bench_config("C3", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        # a long run of tiles per workgroup: one token through a 70B-class MLP up-projection
+        others["decode_m1_k8192_n28672"], _ = bench_config(
+            ProblemSpec("decode_m1_k8192_n28672", GEOM_B, 1, 8192, 28672, 8, 256, 1, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         others["C1"], _ = bench_config("C1", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=False)
         others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
         others["C5"], _ = bench_config("C5", 10, 3, cold_pool=False)
@@ -316,6 +340,7 @@ def main():
         "hipblaslt": {"us": main_res["hipblaslt_us"], "tflops": main_res["hipblaslt_tflops"],
                       "speedup_vs_hipblaslt": main_res["speedup_vs_hipblaslt"]},
         "deterministic_5_runs": main_res["deterministic_5_runs"],
+        "prepacked_codes": main_res.get("prepacked_codes"),
         "other_configs": others,
         "reference_layout_and_control": native,
     }
