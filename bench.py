@@ -216,9 +216,10 @@ def main():
         }
         # The same launches on code matrices re-laid offline in the order the decode kernel's lanes
         # load them (vqgemm_pack_codes_b): beside the figures above, which stay on the plain
-        # [N, K/vec] tensor of the reference's call.
+        # [N, K/vec] tensor of the reference's call.  (Where the K-sliced MFMA kernel is the one that
+        # runs: the GEMV kernel of short single-row launches reads the plain matrix in whole runs.)
         dims = (spec.M, spec.K, spec.N, spec.vec, spec.entries, spec.n_codebooks, spec.code_bits)
-        if cold_pool and cabi.decode_packed_supports(*dims):
+        if cold_pool and res["variant"] == "decode" and cabi.decode_packed_supports(*dims):
             ppool = [cabi.pack_codes_b(c, spec.vec) for c in pool]
             launch_p = lambda i: cabi.e2e_gemm_b(x, ppool[i], cb, out=y, variant=cabi.VARIANT_DECODE_PACKED)
             tp_cold = time_launches(launch_p, n_bufs, steps, warmup)

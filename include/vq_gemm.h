@@ -47,7 +47,13 @@ extern "C" {
                                             (medium M); K a multiple of 64, of 128 for 8-vectors with 8-bit codes */
 #define VQGEMM_VARIANT_DECODE_PACKED 7   /* VQGEMM_VARIANT_DECODE on a code matrix that vqgemm_pack_codes_b has put
                                             in the order the kernel's lanes load it (never chosen by AUTO: the
-                                            layout is a property of the caller's data); same results bit for bit */
+                                            layout is a property of the caller's data); the K-sliced MFMA kernel
+                                            whatever the shape, same results as on the plain matrix bit for bit */
+#define VQGEMM_VARIANT_DECODE_GEMV 8     /* the GEMV kernel: M == 1, 8-vectors, 8-bit codes, at most 256 entries, K a
+                                            multiple of 2048 up to 8192, N and N / n_codebooks multiples of 16; whole
+                                            rows of W per wave, no matrix core.  VQGEMM_VARIANT_DECODE and AUTO take it
+                                            for short launches (K <= 6144, at most 4 tiles of 16 rows per compute
+                                            unit) and the K-sliced MFMA kernel otherwise */
 
 /*
  * Fused VQ GEMM, geometry B.

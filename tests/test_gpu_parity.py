@@ -223,8 +223,61 @@ def test_packed_codes_small_shapes_bias_and_rejections():
         c2 = torch.zeros(16, 32, dtype=torch.uint8, device=DEV)
         cabi.pack_codes_b(c2, 8, out=c2)
     # the automatic choice never takes the packed variant
-    assert cabi.select_variant_b(1, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(1, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
+    assert cabi.select_variant_b(16, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.pack_codes_b(torch.zeros(0, 64, dtype=torch.uint8, device=DEV), 8).shape == (0, 64)
+
+
+GEMV_B = [
+    # name, K, N, E, G
+    ("one_run", 2048, 64, 256, 1),
+    ("c2", 4096, 4096, 256, 1),
+    ("few_entries_4_books", 4096, 4096, 100, 4),
+    ("three_runs_2_books", 6144, 1024, 256, 2),
+    ("four_runs", 8192, 2048, 256, 1),
+    ("16_row_books", 2048, 256, 256, 16),
+    ("many_tiles", 4096, 32768, 256, 1),
+]
+
+
+@pytest.mark.parametrize("row", GEMV_B, ids=[r[0] for r in GEMV_B])
+def test_gemv_kernel_one_row_of_x(row):
+    name, K, N, E, G = row
+    spec = ProblemSpec(name, GEOM_B, 1, K, N, 8, E, G, 8, codebook_3d=(G > 1))
+    x, codes, cb = make_problem(spec, seed=31, device=DEV)
+    _say("gemv", spec)
+    y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+    torch.cuda.synchronize()
+    _check_gemm(y, x, codes, cb, what=name)
+    # one-hot x reads a column of W out bit for bit (fp16 subnormals included: nothing is flushed)
+    w = vo.dequant_b(_np(codes), _np(cb))
+    for col in (0, 7, K // 2 + 3, K - 1):
+        eye = torch.zeros(1, K, dtype=torch.float16, device=DEV)
+        eye[0, col] = 1.0
+        yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+        assert np.array_equal(_np(yw).view(np.uint16)[0], w[:, col].copy().view(np.uint16))
+    bias = torch.randn(N, device=DEV).half()
+    yb = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV, bias=bias)
+    ref = _np(x).astype(np.float64) @ w.astype(np.float64).T + _np(bias).astype(np.float64)
+    e1, _ = vo.rel_err(_np(yb), ref)
+    assert e1 <= TOL
+    for _ in range(4):
+        assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), y)
+    # the decode variant takes this kernel for short launches and the batched kernel for long ones:
+    # same product within the bar either way
+    _check_gemm(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE), x, codes, cb, what=name + " (decode)")
+
+
+def test_gemv_kernel_refuses_other_shapes():
+    cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
+    for (M, K, N, v, bits) in [(2, 2048, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 10240, 64, 8, 8), (1, 2048, 24, 8, 8),
+                               (1, 2048, 64, 4, 8), (1, 2048, 64, 8, 16)]:
+        x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+        codes = torch.zeros(N, K // v, dtype=torch.uint8 if bits == 8 else torch.uint16, device=DEV)
+        c = cb if v == 8 else torch.zeros(256, v, dtype=torch.float16, device=DEV)
+        with pytest.raises(cabi.VqGemmError) as ei:
+            cabi.e2e_gemm_b(x, codes, c, variant=cabi.VARIANT_DECODE_GEMV)
+        assert ei.value.code == -4
 
 
 # Shapes that walk the prefill kernel through each of its instantiations: both super-stage

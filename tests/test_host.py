@@ -54,7 +54,7 @@ def test_argument_validation_happens_before_any_gpu_call():
 
 
 def test_variant_selection_for_the_measured_configurations():
-    want = {"C1": cabi.VARIANT_DECODE, "C2": cabi.VARIANT_DECODE, "C3": cabi.VARIANT_DECODE,
+    want = {"C1": cabi.VARIANT_DECODE, "C2": cabi.VARIANT_DECODE_GEMV, "C3": cabi.VARIANT_DECODE,
             "C4": cabi.VARIANT_PREFILL, "C5": cabi.VARIANT_PREFILL}
     for name, v in want.items():
         s = CONFIGS[name]

@@ -14,9 +14,9 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 _INCLUDE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
 
 (VARIANT_AUTO, VARIANT_GENERIC, VARIANT_DECODE, VARIANT_PREFILL, VARIANT_TWOPASS, VARIANT_PREFILL_NARROW,
- VARIANT_PREFILL_SMALL, VARIANT_DECODE_PACKED) = range(8)
+ VARIANT_PREFILL_SMALL, VARIANT_DECODE_PACKED, VARIANT_DECODE_GEMV) = range(9)
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass", 5: "prefill_narrow", 6: "prefill_small",
-                 7: "decode_packed"}
+                 7: "decode_packed", 8: "decode_gemv"}
 
 _I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
 

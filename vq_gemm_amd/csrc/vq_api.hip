@@ -89,7 +89,8 @@ int select_b(const ProblemB &p, bool all_aligned16)
 {
     if (p.K == 0 || !all_aligned16) return VQGEMM_VARIANT_GENERIC;
     const bool prefill_ok = prefill_supports(p);
-    if (decode_supports(p) && (!prefill_ok || decode_preferred(p))) return VQGEMM_VARIANT_DECODE;
+    if (decode_supports(p) && (!prefill_ok || decode_preferred(p)))
+        return decode_gemv_preferred(p) ? VQGEMM_VARIANT_DECODE_GEMV : VQGEMM_VARIANT_DECODE;
     if (prefill_ok) return VQGEMM_VARIANT_PREFILL;
     return VQGEMM_VARIANT_GENERIC;
 }
@@ -133,7 +134,7 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
 {
     int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
     if (rc != VQGEMM_OK) return rc;
-    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_DECODE_PACKED) return VQGEMM_E_VARIANT;
+    if (variant < VQGEMM_VARIANT_AUTO || variant > VQGEMM_VARIANT_DECODE_GEMV) return VQGEMM_E_VARIANT;
     if (M == 0 || N == 0) return VQGEMM_OK;
     if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
     const uintptr_t code_align = code_bits / 8;
@@ -154,6 +155,11 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
         if (!a16) return VQGEMM_E_ALIGN;
         if (K == 0 || !decode_supports(p)) return VQGEMM_E_VARIANT;
         e = launch_decode_b(p, s);
+        break;
+    case VQGEMM_VARIANT_DECODE_GEMV:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !decode_gemv_supports(p)) return VQGEMM_E_VARIANT;
+        e = launch_decode_gemv(p, s);
         break;
     case VQGEMM_VARIANT_DECODE_PACKED:
         if (!a16) return VQGEMM_E_ALIGN;

@@ -75,6 +75,12 @@ hipError_t launch_pack_codes(const void *src, void *dst, int64_t N, int64_t K, i
                              hipStream_t s);
 // whether launch_decode_b takes the shape with p.packed set (the batched kernel only)
 bool decode_packed_supports(const ProblemB &p);
+// the GEMV kernel behind launch_decode_b (vq_decode_gemv.hip): one row of X, 8-vectors, 8-bit codes,
+// whole rows of W per wave; launch_decode_b takes it while a compute unit has few rows to do
+bool decode_gemv_supports(const ProblemB &p);
+hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s);
+// whether launch_decode_b takes the GEMV kernel for the shape
+bool decode_gemv_preferred(const ProblemB &p);
 // the general kernel behind launch_decode_b: one slab of at most 16 rows of X
 bool decode_general_supports(const ProblemB &p);
 hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);

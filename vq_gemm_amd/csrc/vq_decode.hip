@@ -824,9 +824,25 @@ bool decode_preferred(const ProblemB &p)
     return t_decode <= t_prefill;
 }
 
+// The GEMV kernel has no work shared between its waves and a short chain of latencies; the batched
+// kernel streams long runs of tiles better.  Measured on a 256-CU MI355X at K = 4096 (us, batched ->
+// GEMV, cold HBM): 1 tile of 16 rows per compute unit 4.96 -> 3.85, 2 tiles 6.0 -> 4.8, 4 tiles
+// 7.5 -> 6.6, 8 tiles 11.1 -> 11.1; K = 8192 (x takes 64 registers, two waves per SIMD) is a tie
+// already at 2 tiles.
+#ifndef VQ_GEMV_MAX_TILES_PER_CU
+#define VQ_GEMV_MAX_TILES_PER_CU 4
+#endif
+constexpr int kGemvAutoMaxK = 6144;
+
+bool decode_gemv_preferred(const ProblemB &p)
+{
+    return decode_gemv_supports(p) && p.K <= kGemvAutoMaxK && p.N / kTileN <= VQ_GEMV_MAX_TILES_PER_CU * device_cu_count();
+}
+
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
+    if (decode_gemv_preferred(p)) return launch_decode_gemv(p, s);
     const bool u8 = p.code_bits == 8;
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension

@@ -1,0 +1,148 @@
+// Decode GEMV proper (one row of X): y[n] = sum_k x[k] W[n,k], W given as 8-bit codes of 8-vectors
+// and a codebook of at most 256 entries.  A short launch of this path is a chain of latencies, not
+// a stream, so the kernel is built to keep the chain short rather than to share work:
+//
+//   * A wave owns whole rows of W (four of them), so nothing is summed across waves: no partial
+//     sums in the LDS, no barrier behind the multiply.  A row's sum is folded inside the wave with
+//     DPP adds and four lane reads.
+//   * No matrix core: with one row of X fifteen of an MFMA's sixteen columns would be padding, and
+//     feeding it means laying X out in operand order through the LDS first.  Here a lane keeps
+//     its share of x (the 8-vectors its codes meet) in registers, loaded straight from global
+//     memory while the codes are on their way, and multiplies with v_dot2_f32_f16: four per code.
+//   * Lane l takes the codes 4l..4l+3 of every run of 256 codes: one dword load per row and run
+//     (a wave reads 256 contiguous bytes), x in 64-byte pieces per lane.
+//   * The only barrier publishes the codebook (4 KB, one 16-byte entry per thread) in the LDS; the
+//     gathers are 16-byte reads at code*16.
+//
+// Four waves per workgroup, 16 rows of W: as many workgroups as the batched kernel has tiles.  It
+// wins while a compute unit has a tile or two; for long runs of tiles the batched kernel, whose
+// waves share X and the table over many tiles, is the better stream.
+#include "vq_common.h"
+
+namespace vq {
+
+namespace {
+
+constexpr int kGemvWaves = 4;
+constexpr int kGemvRows = 4;                                // rows of W per wave
+constexpr int kGemvTile = kGemvWaves * kGemvRows;           // rows of W per workgroup
+constexpr int kRunCodes = 256;                              // codes of a row one wave load covers
+constexpr int kRunK = kRunCodes * 8;                        // 2048 k
+constexpr int kGemvMaxRuns = 4;                             // x stays in registers: 16 per run
+
+__device__ __forceinline__ float dpp_add_quad_perm_1032(float v)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dpp_add_quad_perm_2301(float v)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dpp_add_row_half_mirror(float v)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dpp_add_row_mirror(float v)
+{
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));
+}
+
+// Sum of v over the 64 lanes, the same value in every lane: four DPP steps leave each row of 16
+// lanes with its own sum, the four row sums are read out by lane and added in a fixed order.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = dpp_add_quad_perm_1032(v);
+    v = dpp_add_quad_perm_2301(v);
+    v = dpp_add_row_half_mirror(v);
+    v = dpp_add_row_mirror(v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+template <int RUNS>
+__global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half_t *__restrict__ x,
+                                                                       const uint8_t *__restrict__ codes,
+                                                                       const half_t *__restrict__ cb,
+                                                                       half_t *__restrict__ y,
+                                                                       const half_t *__restrict__ bias, int N,
+                                                                       int entries, int rows_per_cb)
+{
+    __shared__ __align__(16) uint4_t table[256];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int row0 = blockIdx.x * kGemvTile + wave * kGemvRows;
+    constexpr int J = RUNS * kRunCodes;  // codes per row
+
+    // codes first (the longest latency), then x, then the table
+    uint32_t cw[kGemvRows][RUNS];
+#pragma unroll
+    for (int r = 0; r < kGemvRows; r++)
+#pragma unroll
+        for (int q = 0; q < RUNS; q++)
+            cw[r][q] = *reinterpret_cast<const uint32_t *>(codes + (int64_t)(row0 + r) * J + q * kRunCodes + 4 * lane);
+    uint4_t xr[RUNS][4];
+#pragma unroll
+    for (int q = 0; q < RUNS; q++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            xr[q][c] = *reinterpret_cast<const uint4_t *>(x + (q * kRunCodes + 4 * lane + c) * 8);
+    const int book = (blockIdx.x * kGemvTile) / rows_per_cb;
+    if ((int)threadIdx.x < entries)
+        table[threadIdx.x] = reinterpret_cast<const uint4_t *>(cb)[(int64_t)book * entries + threadIdx.x];
+    __syncthreads();
+
+    float acc[kGemvRows];
+#pragma unroll
+    for (int r = 0; r < kGemvRows; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int q = 0; q < RUNS; q++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < kGemvRows; r++) {
+                const uint32_t code = (cw[r][q] >> (8 * c)) & 0xffu;
+                const uint4_t w = table[code];
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    // (through scalars: a bit cast applied to a vector element reads element 0)
+                    const uint32_t wd = w[d], xd = xr[q][c][d];
+                    acc[r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[r], false);
+                }
+            }
+    half4_t out;
+#pragma unroll
+    for (int r = 0; r < kGemvRows; r++) {
+        float s = wave_sum(acc[r]);
+        if (bias) s += (float)bias[row0 + r];
+        out[r] = (half_t)s;
+    }
+    if (lane == 0) *reinterpret_cast<half4_t *>(y + row0) = out;
+    (void)N;
+}
+
+}  // namespace
+
+bool decode_gemv_supports(const ProblemB &p)
+{
+    return p.M == 1 && !p.packed && p.vec == 8 && p.code_bits == 8 && p.entries <= 256 && p.K >= kRunK &&
+           p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns && p.N % kGemvTile == 0 && p.rows_per_cb % kGemvTile == 0;
+}
+
+hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
+{
+    if (!decode_gemv_supports(p)) return hipErrorInvalidValue;
+    const dim3 grid(p.N / kGemvTile), block(kGemvWaves * 64);
+    const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
+    switch (p.K / kRunK) {
+    case 1: hipLaunchKernelGGL(decode_gemv_kernel<1>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
+    case 2: hipLaunchKernelGGL(decode_gemv_kernel<2>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
+    case 3: hipLaunchKernelGGL(decode_gemv_kernel<3>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
+    default: hipLaunchKernelGGL(decode_gemv_kernel<4>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace vq

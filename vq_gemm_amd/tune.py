@@ -52,7 +52,7 @@ def tune(M: int, K: int, N: int, vec: int = 8, entries: int = 256, n_codebooks: 
     # a first untimed pass of the heaviest variant brings the device out of its idle clocks
     cabi.e2e_gemm_b(x, codes, cb, out=y, variant=cabi.VARIANT_TWOPASS, workspace=workspace)
     torch.cuda.synchronize()
-    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_PREFILL_SMALL,
+    for variant in (cabi.VARIANT_DECODE, cabi.VARIANT_DECODE_GEMV, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW, cabi.VARIANT_PREFILL_SMALL,
                     cabi.VARIANT_TWOPASS, cabi.VARIANT_AUTO):
         try:
             times[variant] = time_graph(lambda: cabi.e2e_gemm_b(x, codes, cb, out=y, variant=variant, workspace=workspace))
