@@ -225,25 +225,32 @@ def test_packed_codes_small_shapes_bias_and_rejections():
     # the automatic choice never takes the packed variant
     assert cabi.select_variant_b(1, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(16, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(2, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
+    assert cabi.select_variant_b(3, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.pack_codes_b(torch.zeros(0, 64, dtype=torch.uint8, device=DEV), 8).shape == (0, 64)
 
 
 GEMV_B = [
-    # name, K, N, E, G
-    ("one_run", 2048, 64, 256, 1),
-    ("c2", 4096, 4096, 256, 1),
-    ("few_entries_4_books", 4096, 4096, 100, 4),
-    ("three_runs_2_books", 6144, 1024, 256, 2),
-    ("four_runs", 8192, 2048, 256, 1),
-    ("16_row_books", 2048, 256, 256, 16),
-    ("many_tiles", 4096, 32768, 256, 1),
+    # name, K, N, E, G, M
+    ("one_run", 2048, 64, 256, 1, 1),
+    ("c2", 4096, 4096, 256, 1, 1),
+    ("few_entries_4_books", 4096, 4096, 100, 4, 1),
+    ("three_runs_2_books", 6144, 1024, 256, 2, 1),
+    ("four_runs", 8192, 2048, 256, 1, 1),
+    ("16_row_books", 2048, 256, 256, 16, 1),
+    ("many_tiles", 4096, 32768, 256, 1, 1),
+    ("two_rows_of_x", 4096, 4096, 256, 1, 2),
+    ("two_rows_four_runs", 8192, 512, 256, 2, 2),
+    ("three_rows", 2048, 1024, 256, 1, 3),
+    ("four_rows_two_runs", 4096, 1024, 200, 4, 4),
 ]
 
 
 @pytest.mark.parametrize("row", GEMV_B, ids=[r[0] for r in GEMV_B])
-def test_gemv_kernel_one_row_of_x(row):
-    name, K, N, E, G = row
-    spec = ProblemSpec(name, GEOM_B, 1, K, N, 8, E, G, 8, codebook_3d=(G > 1))
+def test_gemv_kernel_few_rows_of_x(row):
+    name, K, N, E, G, M = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, 8, E, G, 8, codebook_3d=(G > 1))
     x, codes, cb = make_problem(spec, seed=31, device=DEV)
     _say("gemv", spec)
     y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
@@ -252,10 +259,12 @@ def test_gemv_kernel_one_row_of_x(row):
     # one-hot x reads a column of W out bit for bit (fp16 subnormals included: nothing is flushed)
     w = vo.dequant_b(_np(codes), _np(cb))
     for col in (0, 7, K // 2 + 3, K - 1):
-        eye = torch.zeros(1, K, dtype=torch.float16, device=DEV)
-        eye[0, col] = 1.0
+        eye = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+        cols = [(col + 41 * m) % K for m in range(M)]
+        for m, c in enumerate(cols):
+            eye[m, c] = 1.0
         yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
-        assert np.array_equal(_np(yw).view(np.uint16)[0], w[:, col].copy().view(np.uint16))
+        assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
     bias = torch.randn(N, device=DEV).half()
     yb = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV, bias=bias)
     ref = _np(x).astype(np.float64) @ w.astype(np.float64).T + _np(bias).astype(np.float64)
@@ -270,7 +279,7 @@ def test_gemv_kernel_one_row_of_x(row):
 
 def test_gemv_kernel_refuses_other_shapes():
     cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
-    for (M, K, N, v, bits) in [(2, 2048, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 10240, 64, 8, 8), (1, 2048, 24, 8, 8),
+    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 10240, 64, 8, 8), (1, 2048, 24, 8, 8),
                                (1, 2048, 64, 4, 8), (1, 2048, 64, 8, 16)]:
         x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
         codes = torch.zeros(N, K // v, dtype=torch.uint8 if bits == 8 else torch.uint16, device=DEV)

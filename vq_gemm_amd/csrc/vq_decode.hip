@@ -828,7 +828,8 @@ bool decode_preferred(const ProblemB &p)
 // kernel streams long runs of tiles better.  Measured on a 256-CU MI355X at K = 4096 (us, batched ->
 // GEMV, cold HBM): 1 tile of 16 rows per compute unit 4.96 -> 3.85, 2 tiles 6.0 -> 4.8, 4 tiles
 // 7.5 -> 6.6, 8 tiles 11.1 -> 11.1; K = 8192 (x takes 64 registers, two waves per SIMD) is a tie
-// already at 2 tiles.
+// already at 2 tiles.  Two rows of X (every gathered codeword meets both): one tile per unit 5.0 -> 4.8,
+// two tiles a tie; three and four rows lose everywhere (5.1 -> 5.6 and 6.6 on one tile).
 #ifndef VQ_GEMV_MAX_TILES_PER_CU
 #define VQ_GEMV_MAX_TILES_PER_CU 4
 #endif
@@ -836,7 +837,8 @@ constexpr int kGemvAutoMaxK = 6144;
 
 bool decode_gemv_preferred(const ProblemB &p)
 {
-    return decode_gemv_supports(p) && p.K <= kGemvAutoMaxK && p.N / kTileN <= VQ_GEMV_MAX_TILES_PER_CU * device_cu_count();
+    const int max_tiles_per_cu = p.M == 1 ? VQ_GEMV_MAX_TILES_PER_CU : (p.M == 2 ? 1 : 0);
+    return decode_gemv_supports(p) && p.K <= kGemvAutoMaxK && p.N / kTileN <= max_tiles_per_cu * device_cu_count();
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)

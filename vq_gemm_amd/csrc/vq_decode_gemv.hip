@@ -1,4 +1,4 @@
-// Decode GEMV proper (one row of X): y[n] = sum_k x[k] W[n,k], W given as 8-bit codes of 8-vectors
+// Decode GEMV proper (one to four rows of X): y[m,n] = sum_k x[m,k] W[n,k], W given as 8-bit codes of 8-vectors
 // and a codebook of at most 256 entries.  A short launch of this path is a chain of latencies, not
 // a stream, so the kernel is built to keep the chain short rather than to share work:
 //
@@ -28,7 +28,8 @@ constexpr int kGemvRows = 4;                                // rows of W per wav
 constexpr int kGemvTile = kGemvWaves * kGemvRows;           // rows of W per workgroup
 constexpr int kRunCodes = 256;                              // codes of a row one wave load covers
 constexpr int kRunK = kRunCodes * 8;                        // 2048 k
-constexpr int kGemvMaxRuns = 4;                             // x stays in registers: 16 per run
+constexpr int kGemvMaxRuns = 4;                             // x stays in registers: 16 per run and row of X,
+constexpr int kGemvMaxXRegs = 128;                          // at most this many in all
 
 __device__ __forceinline__ float dpp_add_quad_perm_1032(float v)
 {
@@ -62,13 +63,14 @@ __device__ __forceinline__ float wave_sum(float v)
     return (r0 + r1) + (r2 + r3);
 }
 
-template <int RUNS>
+// RUNS: runs of 2048 k in a row of W; MX: rows of X (each gathered codeword meets MX shares of x).
+template <int RUNS, int MX>
 __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half_t *__restrict__ x,
                                                                        const uint8_t *__restrict__ codes,
                                                                        const half_t *__restrict__ cb,
                                                                        half_t *__restrict__ y,
-                                                                       const half_t *__restrict__ bias, int N,
-                                                                       int entries, int rows_per_cb)
+                                                                       const half_t *__restrict__ bias, int K,
+                                                                       int N, int entries, int rows_per_cb)
 {
     __shared__ __align__(16) uint4_t table[256];
     const int lane = threadIdx.x & 63;
@@ -83,20 +85,24 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
 #pragma unroll
         for (int q = 0; q < RUNS; q++)
             cw[r][q] = *reinterpret_cast<const uint32_t *>(codes + (int64_t)(row0 + r) * J + q * kRunCodes + 4 * lane);
-    uint4_t xr[RUNS][4];
+    uint4_t xr[MX][RUNS][4];
 #pragma unroll
-    for (int q = 0; q < RUNS; q++)
+    for (int m = 0; m < MX; m++)
 #pragma unroll
-        for (int c = 0; c < 4; c++)
-            xr[q][c] = *reinterpret_cast<const uint4_t *>(x + (q * kRunCodes + 4 * lane + c) * 8);
+        for (int q = 0; q < RUNS; q++)
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                xr[m][q][c] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * K + (q * kRunCodes + 4 * lane + c) * 8);
     const int book = (blockIdx.x * kGemvTile) / rows_per_cb;
     if ((int)threadIdx.x < entries)
         table[threadIdx.x] = reinterpret_cast<const uint4_t *>(cb)[(int64_t)book * entries + threadIdx.x];
     __syncthreads();
 
-    float acc[kGemvRows];
+    float acc[MX][kGemvRows];
 #pragma unroll
-    for (int r = 0; r < kGemvRows; r++) acc[r] = 0.f;
+    for (int m = 0; m < MX; m++)
+#pragma unroll
+        for (int r = 0; r < kGemvRows; r++) acc[m][r] = 0.f;
 #pragma unroll
     for (int q = 0; q < RUNS; q++)
 #pragma unroll
@@ -106,28 +112,33 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
                 const uint32_t code = (cw[r][q] >> (8 * c)) & 0xffu;
                 const uint4_t w = table[code];
 #pragma unroll
-                for (int d = 0; d < 4; d++) {
-                    // (through scalars: a bit cast applied to a vector element reads element 0)
-                    const uint32_t wd = w[d], xd = xr[q][c][d];
-                    acc[r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[r], false);
-                }
-            }
-    half4_t out;
+                for (int m = 0; m < MX; m++)
 #pragma unroll
-    for (int r = 0; r < kGemvRows; r++) {
-        float s = wave_sum(acc[r]);
-        if (bias) s += (float)bias[row0 + r];
-        out[r] = (half_t)s;
+                    for (int d = 0; d < 4; d++) {
+                        // (through scalars: a bit cast applied to a vector element reads element 0)
+                        const uint32_t wd = w[d], xd = xr[m][q][c][d];
+                        acc[m][r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd),
+                                                           acc[m][r], false);
+                    }
+            }
+#pragma unroll
+    for (int m = 0; m < MX; m++) {
+        half4_t out;
+#pragma unroll
+        for (int r = 0; r < kGemvRows; r++) {
+            float s = wave_sum(acc[m][r]);
+            if (bias) s += (float)bias[row0 + r];
+            out[r] = (half_t)s;
+        }
+        if (lane == 0) *reinterpret_cast<half4_t *>(y + (int64_t)m * N + row0) = out;
     }
-    if (lane == 0) *reinterpret_cast<half4_t *>(y + row0) = out;
-    (void)N;
 }
 
 }  // namespace
 
 bool decode_gemv_supports(const ProblemB &p)
 {
-    return p.M == 1 && !p.packed && p.vec == 8 && p.code_bits == 8 && p.entries <= 256 && p.K >= kRunK &&
+    return p.M >= 1 && p.M <= 4 && (int)(p.K / kRunK) * p.M * 16 <= kGemvMaxXRegs && !p.packed && p.vec == 8 && p.code_bits == 8 && p.entries <= 256 && p.K >= kRunK &&
            p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns && p.N % kGemvTile == 0 && p.rows_per_cb % kGemvTile == 0;
 }
 
@@ -136,11 +147,23 @@ hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
     if (!decode_gemv_supports(p)) return hipErrorInvalidValue;
     const dim3 grid(p.N / kGemvTile), block(kGemvWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
-    switch (p.K / kRunK) {
-    case 1: hipLaunchKernelGGL(decode_gemv_kernel<1>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
-    case 2: hipLaunchKernelGGL(decode_gemv_kernel<2>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
-    case 3: hipLaunchKernelGGL(decode_gemv_kernel<3>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
-    default: hipLaunchKernelGGL(decode_gemv_kernel<4>, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.N, p.entries, p.rows_per_cb); break;
+    auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.K, p.N, p.entries, p.rows_per_cb);
+    };
+    switch ((p.K / kRunK) * 10 + p.M) {
+    case 11: launch(decode_gemv_kernel<1, 1>); break;
+    case 12: launch(decode_gemv_kernel<1, 2>); break;
+    case 13: launch(decode_gemv_kernel<1, 3>); break;
+    case 14: launch(decode_gemv_kernel<1, 4>); break;
+    case 21: launch(decode_gemv_kernel<2, 1>); break;
+    case 22: launch(decode_gemv_kernel<2, 2>); break;
+    case 23: launch(decode_gemv_kernel<2, 3>); break;
+    case 24: launch(decode_gemv_kernel<2, 4>); break;
+    case 31: launch(decode_gemv_kernel<3, 1>); break;
+    case 32: launch(decode_gemv_kernel<3, 2>); break;
+    case 41: launch(decode_gemv_kernel<4, 1>); break;
+    case 42: launch(decode_gemv_kernel<4, 2>); break;
+    default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
