@@ -162,8 +162,9 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
     spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
     x, codes, cb = make_problem(spec, seed=21, device=DEV)
     _say("batched decode", spec)
-    assert cabi.select_variant_b(M, K, N, v, E, G, bits) == cabi.VARIANT_DECODE
-    y = cabi.e2e_gemm_b(x, codes, cb)
+    # (the automatic choice: this kernel, or the GEMV kernel for a short run with one row of X)
+    assert cabi.select_variant_b(M, K, N, v, E, G, bits) in (cabi.VARIANT_DECODE, cabi.VARIANT_DECODE_GEMV)
+    y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
     torch.cuda.synchronize()
     w = vo.dequant_b(_np(codes), _np(cb))
     xf = _np(x).astype(np.float64)
@@ -176,9 +177,9 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
     cols = [(37 * m + 11) % K for m in range(M)]
     for m, c in enumerate(cols):
         eye[m, c] = 1.0
-    yw = cabi.e2e_gemm_b(eye, codes, cb)
+    yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_DECODE)
     assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
-    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE), y)
     # The same through the packed code matrix: the re-layout against the oracle's, the GEMM bit for
     # bit the plain layout's (same arithmetic in the same order), W read back through a one-hot X.
     assert cabi.decode_packed_supports(M, K, N, v, E, G, bits)
@@ -227,7 +228,9 @@ def test_packed_codes_small_shapes_bias_and_rejections():
     assert cabi.select_variant_b(16, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.select_variant_b(2, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(3, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
-    assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
+    assert cabi.select_variant_b(1, 4096, 131072, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 2, 8) == cabi.VARIANT_DECODE
     assert cabi.pack_codes_b(torch.zeros(0, 64, dtype=torch.uint8, device=DEV), 8).shape == (0, 64)
 
 
@@ -240,6 +243,9 @@ GEMV_B = [
     ("four_runs", 8192, 2048, 256, 1, 1),
     ("16_row_books", 2048, 256, 256, 16, 1),
     ("many_tiles", 4096, 32768, 256, 1, 1),
+    ("many_tiles_two_books", 4096, 32768, 256, 2, 1),   # not the streaming form: one codebook only
+    ("many_tiles_three_runs_ragged_walk", 6144, 16 * 1500, 256, 1, 1),
+    ("many_tiles_one_run", 2048, 65536, 77, 1, 1),
     ("two_rows_of_x", 4096, 4096, 256, 1, 2),
     ("two_rows_four_runs", 8192, 512, 256, 2, 2),
     ("three_rows", 2048, 1024, 256, 1, 3),
@@ -272,9 +278,9 @@ def test_gemv_kernel_few_rows_of_x(row):
     assert e1 <= TOL
     for _ in range(4):
         assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), y)
-    # the decode variant takes this kernel for short launches and the batched kernel for long ones:
-    # same product within the bar either way
+    # the K-sliced MFMA kernel and the automatic choice on the same inputs: same product within the bar
     _check_gemm(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE), x, codes, cb, what=name + " (decode)")
+    _check_gemm(cabi.e2e_gemm_b(x, codes, cb), x, codes, cb, what=name + " (auto)")
 
 
 def test_gemv_kernel_refuses_other_shapes():

@@ -76,10 +76,12 @@ hipError_t launch_pack_codes(const void *src, void *dst, int64_t N, int64_t K, i
 // whether launch_decode_b takes the shape with p.packed set (the batched kernel only)
 bool decode_packed_supports(const ProblemB &p);
 // the GEMV kernel behind launch_decode_b (vq_decode_gemv.hip): one row of X, 8-vectors, 8-bit codes,
-// whole rows of W per wave; launch_decode_b takes it while a compute unit has few rows to do
+// whole rows of W per wave; the automatic choice takes it while a compute unit has few rows to do
 bool decode_gemv_supports(const ProblemB &p);
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s);
-// whether launch_decode_b takes the GEMV kernel for the shape
+// the persistent form of the GEMV kernel that launch_decode_gemv takes for long runs of rows (one row of X, one codebook)
+bool decode_gemv_stream_supports(const ProblemB &p);
+// whether the automatic choice takes the GEMV kernel rather than launch_decode_b for a shape both serve
 bool decode_gemv_preferred(const ProblemB &p);
 // the general kernel behind launch_decode_b: one slab of at most 16 rows of X
 bool decode_general_supports(const ProblemB &p);

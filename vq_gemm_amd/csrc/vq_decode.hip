@@ -837,14 +837,16 @@ constexpr int kGemvAutoMaxK = 6144;
 
 bool decode_gemv_preferred(const ProblemB &p)
 {
-    const int max_tiles_per_cu = p.M == 1 ? VQ_GEMV_MAX_TILES_PER_CU : (p.M == 2 ? 1 : 0);
+    // (one row of X and one codebook: the GEMV path walks longer runs with its streaming kernel, which
+    // beats the batched kernel on the plain code matrix up to about 16 tiles per unit - 8 tiles 11.1 ->
+    // 9.6 us cold, 16 tiles 14.8 -> 13.4 warm - and falls behind at 32)
+    const int max_tiles_per_cu = p.M == 1 ? (decode_gemv_stream_supports(p) ? 16 : VQ_GEMV_MAX_TILES_PER_CU) : (p.M == 2 ? 1 : 0);
     return decode_gemv_supports(p) && p.K <= kGemvAutoMaxK && p.N / kTileN <= max_tiles_per_cu * device_cu_count();
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
-    if (decode_gemv_preferred(p)) return launch_decode_gemv(p, s);
     const bool u8 = p.code_bits == 8;
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension

@@ -23,8 +23,15 @@ namespace vq {
 
 namespace {
 
-constexpr int kGemvWaves = 4;
-constexpr int kGemvRows = 4;                                // rows of W per wave
+#ifndef VQ_GEMV_WAVES
+#define VQ_GEMV_WAVES 4
+#endif
+#ifndef VQ_GEMV_ROWS
+#define VQ_GEMV_ROWS 4
+#endif
+constexpr int kGemvWaves = VQ_GEMV_WAVES;
+constexpr int kGemvRows = VQ_GEMV_ROWS;                     // rows of W per wave
+typedef _Float16 gemv_out_t __attribute__((ext_vector_type(kGemvRows)));
 constexpr int kGemvTile = kGemvWaves * kGemvRows;           // rows of W per workgroup
 constexpr int kRunCodes = 256;                              // codes of a row one wave load covers
 constexpr int kRunK = kRunCodes * 8;                        // 2048 k
@@ -94,7 +101,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
             for (int c = 0; c < 4; c++)
                 xr[m][q][c] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * K + (q * kRunCodes + 4 * lane + c) * 8);
     const int book = (blockIdx.x * kGemvTile) / rows_per_cb;
-    if ((int)threadIdx.x < entries)
+    if ((int)threadIdx.x < entries)  // (entries <= 256 <= threads)
         table[threadIdx.x] = reinterpret_cast<const uint4_t *>(cb)[(int64_t)book * entries + threadIdx.x];
     __syncthreads();
 
@@ -123,18 +130,126 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
             }
 #pragma unroll
     for (int m = 0; m < MX; m++) {
-        half4_t out;
+        gemv_out_t out;
 #pragma unroll
         for (int r = 0; r < kGemvRows; r++) {
             float s = wave_sum(acc[m][r]);
             if (bias) s += (float)bias[row0 + r];
             out[r] = (half_t)s;
         }
-        if (lane == 0) *reinterpret_cast<half4_t *>(y + (int64_t)m * N + row0) = out;
+        if (lane == 0) *reinterpret_cast<gemv_out_t *>(y + (int64_t)m * N + row0) = out;
+    }
+}
+
+// The same for long runs of rows: two workgroups per compute unit (four waves alone do not cover the
+// latency of their own gathers; 64 KB of table each), each walking 16-row blocks of W with x and the
+// table kept.  What a block no longer pays (x, the table, the launch of its
+// waves) buys a bank-replicated table - one 256-byte bank row per entry holding 16 copies, lane l
+// reading copy l % 16, so that the gathers are free of bank conflicts - and the codes of the next
+// block are requested before the current one is multiplied.  One row of X, one codebook.
+template <int RUNS>
+__global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_stream_kernel(const half_t *__restrict__ x,
+                                                                              const uint8_t *__restrict__ codes,
+                                                                              const half_t *__restrict__ cb,
+                                                                              half_t *__restrict__ y,
+                                                                              const half_t *__restrict__ bias,
+                                                                              int n_blocks, int entries)
+{
+#ifndef VQ_GEMV_STREAM_COPIES
+#define VQ_GEMV_STREAM_COPIES 16
+#endif
+#ifndef VQ_GEMV_STREAM_WGS_PER_CU
+#define VQ_GEMV_STREAM_WGS_PER_CU 2
+#endif
+    constexpr int kCopies = VQ_GEMV_STREAM_COPIES;
+    __shared__ __align__(16) uint4_t table[256 * kCopies];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int J = RUNS * kRunCodes;  // codes per row
+    const uint8_t *lane_codes = codes + (int64_t)(wave * kGemvRows) * J + 4 * lane;
+    auto load_block = [&](int b, uint32_t (&cw)[kGemvRows][RUNS]) {
+#pragma unroll
+        for (int r = 0; r < kGemvRows; r++)
+#pragma unroll
+            for (int q = 0; q < RUNS; q++)
+                cw[r][q] = *reinterpret_cast<const uint32_t *>(lane_codes + ((int64_t)b * kGemvTile + r) * J + q * kRunCodes);
+    };
+    int b = blockIdx.x;
+    uint32_t cur[kGemvRows][RUNS], nxt[kGemvRows][RUNS];
+    load_block(b, cur);
+    uint4_t xr[RUNS][4];
+#pragma unroll
+    for (int q = 0; q < RUNS; q++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) xr[q][c] = *reinterpret_cast<const uint4_t *>(x + (q * kRunCodes + 4 * lane + c) * 8);
+    if ((int)threadIdx.x < entries) {
+        const uint4_t e = reinterpret_cast<const uint4_t *>(cb)[threadIdx.x];
+        // (copy (l + i) % 16 in turn i: the sixteen lanes of a group write sixteen different bank groups)
+#pragma unroll
+        for (int i = 0; i < kCopies; i++) table[threadIdx.x * kCopies + ((lane + i) & (kCopies - 1))] = e;
+    }
+    __syncthreads();
+    const uint32_t copy = lane & (kCopies - 1);
+    for (; b < n_blocks; b += gridDim.x) {
+        const int bn = b + gridDim.x;
+        if (bn < n_blocks) load_block(bn, nxt);
+        float acc[kGemvRows];
+#pragma unroll
+        for (int r = 0; r < kGemvRows; r++) acc[r] = 0.f;
+#pragma unroll
+        for (int q = 0; q < RUNS; q++)
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int r = 0; r < kGemvRows; r++) {
+                    const uint32_t code = (cur[r][q] >> (8 * c)) & 0xffu;
+                    const uint4_t w = table[code * kCopies + copy];
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        const uint32_t wd = w[d], xd = xr[q][c][d];
+                        acc[r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[r], false);
+                    }
+                }
+        const int row0 = b * kGemvTile + wave * kGemvRows;
+        gemv_out_t out;
+#pragma unroll
+        for (int r = 0; r < kGemvRows; r++) {
+            float s = wave_sum(acc[r]);
+            if (bias) s += (float)bias[row0 + r];
+            out[r] = (half_t)s;
+        }
+        if (lane == 0) *reinterpret_cast<gemv_out_t *>(y + row0) = out;
+#pragma unroll
+        for (int r = 0; r < kGemvRows; r++)
+#pragma unroll
+            for (int q = 0; q < RUNS; q++) cur[r][q] = nxt[r][q];
     }
 }
 
 }  // namespace
+
+bool decode_gemv_stream_supports(const ProblemB &p)
+{
+    return decode_gemv_supports(p) && p.M == 1 && p.n_codebooks == 1;
+}
+
+hipError_t launch_decode_gemv_stream(const ProblemB &p, hipStream_t s)
+{
+    if (!decode_gemv_stream_supports(p)) return hipErrorInvalidValue;
+    const int n_blocks = p.N / kGemvTile;
+    const int cus = device_cu_count();
+    const int wgs = cus * VQ_GEMV_STREAM_WGS_PER_CU;
+    const dim3 grid(n_blocks < wgs ? n_blocks : wgs), block(kGemvWaves * 64);
+    const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
+    auto launch = [&](auto kern) { hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, n_blocks, p.entries); };
+    switch (p.K / kRunK) {
+    case 1: launch(decode_gemv_stream_kernel<1>); break;
+    case 2: launch(decode_gemv_stream_kernel<2>); break;
+    case 3: launch(decode_gemv_stream_kernel<3>); break;
+    default: launch(decode_gemv_stream_kernel<4>); break;
+    }
+    return hipGetLastError();
+}
 
 bool decode_gemv_supports(const ProblemB &p)
 {
@@ -142,9 +257,16 @@ bool decode_gemv_supports(const ProblemB &p)
            p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns && p.N % kGemvTile == 0 && p.rows_per_cb % kGemvTile == 0;
 }
 
+// From this many 16-row blocks per compute unit on, one row of X goes to the streaming kernel.
+#ifndef VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU
+#define VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU 4
+#endif
+
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
 {
     if (!decode_gemv_supports(p)) return hipErrorInvalidValue;
+    if (decode_gemv_stream_supports(p) && p.N / kGemvTile >= VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU * device_cu_count())
+        return launch_decode_gemv_stream(p, s);
     const dim3 grid(p.N / kGemvTile), block(kGemvWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
     auto launch = [&](auto kern) {
