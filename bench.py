@@ -252,6 +252,10 @@ def main():
         others["decode_m1_k8192_n28672"], _ = bench_config(
             ProblemSpec("decode_m1_k8192_n28672", GEOM_B, 1, 8192, 28672, 8, 256, 1, 8),
             max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        # a medium run of rows with one row of X: the streaming form of the GEMV kernel
+        others["decode_m1_k4096_n28672"], _ = bench_config(
+            ProblemSpec("decode_m1_k4096_n28672", GEOM_B, 1, 4096, 28672, 8, 256, 1, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         others["C1"], _ = bench_config("C1", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=False)
         others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
         others["C5"], _ = bench_config("C5", 10, 3, cold_pool=False)
