@@ -49,9 +49,11 @@ extern "C" {
                                             in the order the kernel's lanes load it (never chosen by AUTO: the
                                             layout is a property of the caller's data); the K-sliced MFMA kernel
                                             whatever the shape, same results as on the plain matrix bit for bit */
-#define VQGEMM_VARIANT_DECODE_GEMV 8     /* the GEMV kernel: M <= 4, 8-vectors, 8-bit codes, at most 256 entries, K a
-                                            multiple of 2048 with (K / 2048) * M <= 8, N and N / n_codebooks multiples
-                                            of 16; whole rows of W per wave, no matrix core.  AUTO takes it for short
+#define VQGEMM_VARIANT_DECODE_GEMV 8     /* the GEMV kernel: M <= 4 for 8-vectors with 8-bit codes, M <= 2 for 4-vectors,
+                                            8-vectors with 16-bit codes and 2-vectors with 8-bit codes; at most 256
+                                            resp. 4096 entries, entries * vec a multiple of 8; K a multiple of 2048
+                                            with (K / 2048) * M <= 8, N and N / n_codebooks multiples of 16; whole
+                                            rows of W per wave, no matrix core.  AUTO takes it for short
                                             launches (K <= 6144; M == 1 and at most 4 tiles of 16 rows per compute
                                             unit - 16 with a single codebook - or M == 2 and at most one) and
                                             VQGEMM_VARIANT_DECODE, the K-sliced MFMA kernels, otherwise */

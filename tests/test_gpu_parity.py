@@ -283,10 +283,44 @@ def test_gemv_kernel_few_rows_of_x(row):
     _check_gemm(cabi.e2e_gemm_b(x, codes, cb), x, codes, cb, what=name + " (auto)")
 
 
+GEMV_FORMATS = [
+    # name, M, K, N, vec, E, bits, G
+    ("v4_u16_e4096_c3_weights", 1, 4096, 11008, 4, 4096, 16, 1),
+    ("v4_u16_two_rows_two_books", 2, 2048, 256, 4, 1000, 16, 2),
+    ("v4_u8", 1, 4096, 1024, 4, 256, 8, 1),
+    ("v4_u8_three_runs_two_rows", 2, 6144, 512, 4, 100, 8, 4),
+    ("v8_u16_e4096", 1, 4096, 512, 8, 4096, 16, 1),
+    ("v8_u16_four_runs", 1, 8192, 256, 8, 333, 16, 1),
+    ("v2_u8", 1, 2048, 1024, 2, 256, 8, 1),
+    ("v2_u8_two_rows", 2, 4096, 256, 2, 200, 8, 2),
+]
+
+
+@pytest.mark.parametrize("row", GEMV_FORMATS, ids=[r[0] for r in GEMV_FORMATS])
+def test_gemv_kernel_code_formats(row):
+    name, M, K, N, v, E, bits, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+    x, codes, cb = make_problem(spec, seed=37, device=DEV)
+    _say("gemv format", spec)
+    y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+    torch.cuda.synchronize()
+    _check_gemm(y, x, codes, cb, what=name)
+    w = vo.dequant_b(_np(codes), _np(cb))
+    for col in (0, 3, K // 2 + 5, K - 1):
+        eye = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+        cols = [(col + 29 * m) % K for m in range(M)]
+        for m, c in enumerate(cols):
+            eye[m, c] = 1.0
+        yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+        assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), y)
+    _check_gemm(cabi.e2e_gemm_b(x, codes, cb), x, codes, cb, what=name + " (auto)")
+
+
 def test_gemv_kernel_refuses_other_shapes():
     cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
     for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 10240, 64, 8, 8), (1, 2048, 24, 8, 8),
-                               (1, 2048, 64, 4, 8), (1, 2048, 64, 8, 16)]:
+                               (1, 2048, 64, 2, 16), (3, 2048, 64, 4, 8)]:
         x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
         codes = torch.zeros(N, K // v, dtype=torch.uint8 if bits == 8 else torch.uint16, device=DEV)
         c = cb if v == 8 else torch.zeros(256, v, dtype=torch.float16, device=DEV)

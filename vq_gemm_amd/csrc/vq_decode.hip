@@ -840,6 +840,12 @@ bool decode_gemv_preferred(const ProblemB &p)
     // (one row of X and one codebook: the GEMV path walks longer runs with its streaming kernel, which
     // beats the batched kernel on the plain code matrix up to about 16 tiles per unit - 8 tiles 11.1 ->
     // 9.6 us cold, 16 tiles 14.8 -> 13.4 warm - and falls behind at 32)
+    // Other code formats (same kernel, other gather width): one row of X only, and not with a table
+    // of more than 32 KB, which every workgroup has to fill (us cold at K = 4096, batched -> GEMV:
+    // 4-vectors / 8-bit codes N = 4096 5.0 -> 4.2, N = 16384 9.2 -> 7.3; 2-vectors 6.0 -> 5.6; 4-vectors /
+    // 16-bit codes / 4096 entries N = 11008 9.9 -> 9.5; 8-vectors / 16-bit codes / 4096 entries 5.6 -> 5.9).
+    const bool first_format = p.vec == 8 && p.code_bits == 8;
+    if (!first_format && (p.M != 1 || (int64_t)p.entries * p.vec * 2 > 32 * 1024)) return false;
     const int max_tiles_per_cu = p.M == 1 ? (decode_gemv_stream_supports(p) ? 16 : VQ_GEMV_MAX_TILES_PER_CU) : (p.M == 2 ? 1 : 0);
     return decode_gemv_supports(p) && p.K <= kGemvAutoMaxK && p.N / kTileN <= max_tiles_per_cu * device_cu_count();
 }

@@ -1,5 +1,5 @@
-// Decode GEMV proper (one to four rows of X): y[m,n] = sum_k x[m,k] W[n,k], W given as 8-bit codes of 8-vectors
-// and a codebook of at most 256 entries.  A short launch of this path is a chain of latencies, not
+// Decode GEMV proper (one to four rows of X): y[m,n] = sum_k x[m,k] W[n,k], W given as codes and a codebook
+// (described below for 8-bit codes of 8-vectors; GemvCfg holds what changes with the format).  A short launch of this path is a chain of latencies, not
 // a stream, so the kernel is built to keep the chain short rather than to share work:
 //
 //   * A wave owns whole rows of W (four of them), so nothing is summed across waves: no partial
@@ -70,39 +70,63 @@ __device__ __forceinline__ float wave_sum(float v)
     return (r0 + r1) + (r2 + r3);
 }
 
+// Format of the codes: a lane takes the 32 / VEC codes that meet 32 consecutive halves of x in every
+// run of 2048 k, as one load of 4, 8 or 16 bytes.
+template <int VEC, typename CodeT>
+struct GemvCfg {
+    static constexpr int CPR = 32 / VEC;                      // codes per lane and run
+    static constexpr int CW = CPR * (int)sizeof(CodeT) / 4;   // dwords per lane and run
+    static constexpr int kMaxEntries = sizeof(CodeT) == 1 ? 256 : 4096;
+    static constexpr int kTableBytes = kMaxEntries * VEC * 2;
+    static_assert(CW == 1 || CW == 2 || CW == 4, "one load of 4, 8 or 16 bytes");
+    static_assert(kTableBytes <= 64 * 1024, "the table is a static LDS array");
+};
+
 // RUNS: runs of 2048 k in a row of W; MX: rows of X (each gathered codeword meets MX shares of x).
-template <int RUNS, int MX>
+template <int VEC, typename CodeT, int RUNS, int MX>
 __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half_t *__restrict__ x,
-                                                                       const uint8_t *__restrict__ codes,
+                                                                       const CodeT *__restrict__ codes,
                                                                        const half_t *__restrict__ cb,
                                                                        half_t *__restrict__ y,
                                                                        const half_t *__restrict__ bias, int K,
                                                                        int N, int entries, int rows_per_cb)
 {
-    __shared__ __align__(16) uint4_t table[256];
+    typedef GemvCfg<VEC, CodeT> C;
+    typedef uint32_t words_t __attribute__((ext_vector_type(C::CW)));
+    __shared__ __align__(16) uint4_t table[C::kTableBytes / 16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int row0 = blockIdx.x * kGemvTile + wave * kGemvRows;
-    constexpr int J = RUNS * kRunCodes;  // codes per row
+    constexpr int J = RUNS * 64 * C::CPR;  // codes per row
 
     // codes first (the longest latency), then x, then the table
-    uint32_t cw[kGemvRows][RUNS];
+    uint32_t cw[kGemvRows][RUNS][C::CW];
 #pragma unroll
     for (int r = 0; r < kGemvRows; r++)
 #pragma unroll
-        for (int q = 0; q < RUNS; q++)
-            cw[r][q] = *reinterpret_cast<const uint32_t *>(codes + (int64_t)(row0 + r) * J + q * kRunCodes + 4 * lane);
-    uint4_t xr[MX][RUNS][4];
+        for (int q = 0; q < RUNS; q++) {
+            const words_t v = *reinterpret_cast<const words_t *>(codes + (int64_t)(row0 + r) * J + (q * 64 + lane) * C::CPR);
+#pragma unroll
+            for (int i = 0; i < C::CW; i++) cw[r][q][i] = v[i];
+        }
+    uint32_t xr[MX][RUNS][16];  // the lane's 32 halves of x per run and row of X
 #pragma unroll
     for (int m = 0; m < MX; m++)
 #pragma unroll
         for (int q = 0; q < RUNS; q++)
 #pragma unroll
-            for (int c = 0; c < 4; c++)
-                xr[m][q][c] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * K + (q * kRunCodes + 4 * lane + c) * 8);
+            for (int c = 0; c < 4; c++) {
+                const uint4_t v = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * K + ((q * 64 + lane) * 4 + c) * 8);
+#pragma unroll
+                for (int d = 0; d < 4; d++) xr[m][q][4 * c + d] = v[d];
+            }
     const int book = (blockIdx.x * kGemvTile) / rows_per_cb;
-    if ((int)threadIdx.x < entries)  // (entries <= 256 <= threads)
-        table[threadIdx.x] = reinterpret_cast<const uint4_t *>(cb)[(int64_t)book * entries + threadIdx.x];
+    {
+        // (entries * VEC * 2 is a multiple of 16, so every codebook starts on a 16-byte boundary)
+        const int chunks = entries * VEC * 2 / 16;
+        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)book * entries * VEC);
+        for (int i = threadIdx.x; i < chunks; i += kGemvWaves * 64) table[i] = src[i];
+    }
     __syncthreads();
 
     float acc[MX][kGemvRows];
@@ -110,20 +134,35 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     for (int m = 0; m < MX; m++)
 #pragma unroll
         for (int r = 0; r < kGemvRows; r++) acc[m][r] = 0.f;
+    const uint8_t *tbl = reinterpret_cast<const uint8_t *>(table);
 #pragma unroll
     for (int q = 0; q < RUNS; q++)
 #pragma unroll
-        for (int c = 0; c < 4; c++)
+        for (int c = 0; c < C::CPR; c++)
 #pragma unroll
             for (int r = 0; r < kGemvRows; r++) {
-                const uint32_t code = (cw[r][q] >> (8 * c)) & 0xffu;
-                const uint4_t w = table[code];
+                uint32_t code;
+                if constexpr (sizeof(CodeT) == 1) code = (cw[r][q][c >> 2] >> (8 * (c & 3))) & 0xffu;
+                else code = (cw[r][q][c >> 1] >> (16 * (c & 1))) & 0xffffu;
+                // the codeword: VEC halves = VEC / 2 words
+                uint32_t w[VEC / 2];
+                if constexpr (VEC == 8) {
+                    const uint4_t v = *reinterpret_cast<const uint4_t *>(tbl + code * 16);
+#pragma unroll
+                    for (int d = 0; d < 4; d++) w[d] = v[d];
+                } else if constexpr (VEC == 4) {
+                    const uint2_t v = *reinterpret_cast<const uint2_t *>(tbl + code * 8);
+                    w[0] = v[0];
+                    w[1] = v[1];
+                } else {
+                    w[0] = *reinterpret_cast<const uint32_t *>(tbl + code * 4);
+                }
 #pragma unroll
                 for (int m = 0; m < MX; m++)
 #pragma unroll
-                    for (int d = 0; d < 4; d++) {
+                    for (int d = 0; d < VEC / 2; d++) {
                         // (through scalars: a bit cast applied to a vector element reads element 0)
-                        const uint32_t wd = w[d], xd = xr[m][q][c][d];
+                        const uint32_t wd = w[d], xd = xr[m][q][c * (VEC / 2) + d];
                         acc[m][r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd),
                                                            acc[m][r], false);
                     }
@@ -230,7 +269,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_stream_kernel(con
 
 bool decode_gemv_stream_supports(const ProblemB &p)
 {
-    return decode_gemv_supports(p) && p.M == 1 && p.n_codebooks == 1;
+    return decode_gemv_supports(p) && p.vec == 8 && p.code_bits == 8 && p.M == 1 && p.n_codebooks == 1;
 }
 
 hipError_t launch_decode_gemv_stream(const ProblemB &p, hipStream_t s)
@@ -253,7 +292,13 @@ hipError_t launch_decode_gemv_stream(const ProblemB &p, hipStream_t s)
 
 bool decode_gemv_supports(const ProblemB &p)
 {
-    return p.M >= 1 && p.M <= 4 && (int)(p.K / kRunK) * p.M * 16 <= kGemvMaxXRegs && !p.packed && p.vec == 8 && p.code_bits == 8 && p.entries <= 256 && p.K >= kRunK &&
+    const bool u8 = p.code_bits == 8;
+    // 8- and 4-vectors with either code width, 2-vectors with 8-bit codes (one load of at most 16 bytes per run)
+    if (!(p.vec == 8 || p.vec == 4 || (p.vec == 2 && u8))) return false;
+    if (p.entries > (u8 ? 256 : 4096) || (p.entries * p.vec * 2) % 16 != 0) return false;
+    // two rows of X at most outside the first format (three and four never pay)
+    const int max_m = (p.vec == 8 && u8) ? 4 : 2;
+    return p.M >= 1 && p.M <= max_m && (int)(p.K / kRunK) * p.M * 16 <= kGemvMaxXRegs && !p.packed && p.K >= kRunK &&
            p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns && p.N % kGemvTile == 0 && p.rows_per_cb % kGemvTile == 0;
 }
 
@@ -262,32 +307,54 @@ bool decode_gemv_supports(const ProblemB &p)
 #define VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU 4
 #endif
 
+namespace {
+
+template <int VEC, typename CodeT>
+hipError_t launch_gemv_format(const ProblemB &p, hipStream_t s)
+{
+    const dim3 grid(p.N / kGemvTile), block(kGemvWaves * 64);
+    const CodeT *codes = static_cast<const CodeT *>(p.codes);
+    auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.K, p.N, p.entries, p.rows_per_cb);
+    };
+    switch ((p.K / kRunK) * 10 + p.M) {
+    case 11: launch(decode_gemv_kernel<VEC, CodeT, 1, 1>); break;
+    case 12: launch(decode_gemv_kernel<VEC, CodeT, 1, 2>); break;
+    case 21: launch(decode_gemv_kernel<VEC, CodeT, 2, 1>); break;
+    case 22: launch(decode_gemv_kernel<VEC, CodeT, 2, 2>); break;
+    case 31: launch(decode_gemv_kernel<VEC, CodeT, 3, 1>); break;
+    case 32: launch(decode_gemv_kernel<VEC, CodeT, 3, 2>); break;
+    case 41: launch(decode_gemv_kernel<VEC, CodeT, 4, 1>); break;
+    case 42: launch(decode_gemv_kernel<VEC, CodeT, 4, 2>); break;
+    default:
+        if constexpr (VEC == 8 && sizeof(CodeT) == 1) {
+            switch ((p.K / kRunK) * 10 + p.M) {
+            case 13: launch(decode_gemv_kernel<8, uint8_t, 1, 3>); break;
+            case 14: launch(decode_gemv_kernel<8, uint8_t, 1, 4>); break;
+            case 23: launch(decode_gemv_kernel<8, uint8_t, 2, 3>); break;
+            case 24: launch(decode_gemv_kernel<8, uint8_t, 2, 4>); break;
+            default: return hipErrorInvalidValue;
+            }
+            break;
+        }
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
 {
     if (!decode_gemv_supports(p)) return hipErrorInvalidValue;
     if (decode_gemv_stream_supports(p) && p.N / kGemvTile >= VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU * device_cu_count())
         return launch_decode_gemv_stream(p, s);
-    const dim3 grid(p.N / kGemvTile), block(kGemvWaves * 64);
-    const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
-    auto launch = [&](auto kern) {
-        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.K, p.N, p.entries, p.rows_per_cb);
-    };
-    switch ((p.K / kRunK) * 10 + p.M) {
-    case 11: launch(decode_gemv_kernel<1, 1>); break;
-    case 12: launch(decode_gemv_kernel<1, 2>); break;
-    case 13: launch(decode_gemv_kernel<1, 3>); break;
-    case 14: launch(decode_gemv_kernel<1, 4>); break;
-    case 21: launch(decode_gemv_kernel<2, 1>); break;
-    case 22: launch(decode_gemv_kernel<2, 2>); break;
-    case 23: launch(decode_gemv_kernel<2, 3>); break;
-    case 24: launch(decode_gemv_kernel<2, 4>); break;
-    case 31: launch(decode_gemv_kernel<3, 1>); break;
-    case 32: launch(decode_gemv_kernel<3, 2>); break;
-    case 41: launch(decode_gemv_kernel<4, 1>); break;
-    case 42: launch(decode_gemv_kernel<4, 2>); break;
-    default: return hipErrorInvalidValue;
+    const bool u8 = p.code_bits == 8;
+    switch (p.vec) {
+    case 8: return u8 ? launch_gemv_format<8, uint8_t>(p, s) : launch_gemv_format<8, uint16_t>(p, s);
+    case 4: return u8 ? launch_gemv_format<4, uint8_t>(p, s) : launch_gemv_format<4, uint16_t>(p, s);
+    default: return launch_gemv_format<2, uint8_t>(p, s);
     }
-    return hipGetLastError();
 }
 
 }  // namespace vq
