@@ -53,10 +53,11 @@ extern "C" {
                                             8-vectors with 16-bit codes and 2-vectors with 8-bit codes; at most 256
                                             resp. 4096 entries, entries * vec a multiple of 8; K a multiple of 2048
                                             with (K / 2048) * M <= 8, N and N / n_codebooks multiples of 16; whole
-                                            rows of W per wave, no matrix core.  AUTO takes it for short
-                                            launches (K <= 6144; M == 1 and at most 4 tiles of 16 rows per compute
-                                            unit - 16 with a single codebook - or M == 2 and at most one) and
-                                            VQGEMM_VARIANT_DECODE, the K-sliced MFMA kernels, otherwise */
+                                            rows of W per wave, no matrix core.  AUTO takes it where it was measured
+                                            faster (M == 1: at most 4 tiles of 16 rows per compute unit, 16 with a
+                                            single codebook of 8-vectors; M == 2: at most one; K <= 6144, K = 8192
+                                            between 4 and 8 tiles per unit) and VQGEMM_VARIANT_DECODE, the K-sliced
+                                            MFMA kernels, otherwise */
 
 /*
  * Fused VQ GEMM, geometry B.

@@ -847,7 +847,11 @@ bool decode_gemv_preferred(const ProblemB &p)
     const bool first_format = p.vec == 8 && p.code_bits == 8;
     if (!first_format && (p.M != 1 || (int64_t)p.entries * p.vec * 2 > 32 * 1024)) return false;
     const int max_tiles_per_cu = p.M == 1 ? (decode_gemv_stream_supports(p) ? 16 : VQ_GEMV_MAX_TILES_PER_CU) : (p.M == 2 ? 1 : 0);
-    return decode_gemv_supports(p) && p.K <= kGemvAutoMaxK && p.N / kTileN <= max_tiles_per_cu * device_cu_count();
+    if (!decode_gemv_supports(p) || p.N / kTileN > max_tiles_per_cu * device_cu_count()) return false;
+    // K = 8192: only where the streaming form runs and up to 8 blocks per unit (us cold, batched -> GEMV:
+    // N = 16384 12.6 -> 11.3, N = 28672 18.3 -> 17.0, N = 57344 27.0 -> 29.9)
+    const int tiles = p.N / kTileN, cus = device_cu_count();
+    return p.K <= kGemvAutoMaxK || (decode_gemv_stream_supports(p) && tiles >= 4 * cus && tiles <= 8 * cus);
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)

@@ -277,7 +277,8 @@ hipError_t launch_decode_gemv_stream(const ProblemB &p, hipStream_t s)
     if (!decode_gemv_stream_supports(p)) return hipErrorInvalidValue;
     const int n_blocks = p.N / kGemvTile;
     const int cus = device_cu_count();
-    const int wgs = cus * VQ_GEMV_STREAM_WGS_PER_CU;
+    // (four runs: x alone takes 64 registers, a unit holds one workgroup's waves, and a second one would only queue)
+    const int wgs = cus * (p.K / kRunK <= 3 ? VQ_GEMV_STREAM_WGS_PER_CU : 1);
     const dim3 grid(n_blocks < wgs ? n_blocks : wgs), block(kGemvWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
     auto launch = [&](auto kern) { hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, n_blocks, p.entries); };
