@@ -99,7 +99,15 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     const int row0 = blockIdx.x * kGemvTile + wave * kGemvRows;
     constexpr int J = RUNS * 64 * C::CPR;  // codes per row
 
-    // codes first (the longest latency), then x, then the table
+    // The table's load goes out first and is the first to be back (it comes out of the L2): its copy
+    // into the LDS and the barrier then pass while the codes (HBM) and x are still on their way.
+    // (no division in front of the first load when there is one codebook)
+    const int book = rows_per_cb >= N ? 0 : (blockIdx.x * kGemvTile) / rows_per_cb;
+    // (entries * VEC * 2 is a multiple of 16, so every codebook starts on a 16-byte boundary)
+    const int chunks = entries * VEC * 2 / 16;
+    const uint4_t *tsrc = reinterpret_cast<const uint4_t *>(cb + (int64_t)book * entries * VEC);
+    uint4_t t0 = {0u, 0u, 0u, 0u};
+    if ((int)threadIdx.x < chunks) t0 = tsrc[threadIdx.x];
     uint32_t cw[kGemvRows][RUNS][C::CW];
 #pragma unroll
     for (int r = 0; r < kGemvRows; r++)
@@ -120,13 +128,8 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
 #pragma unroll
                 for (int d = 0; d < 4; d++) xr[m][q][4 * c + d] = v[d];
             }
-    const int book = (blockIdx.x * kGemvTile) / rows_per_cb;
-    {
-        // (entries * VEC * 2 is a multiple of 16, so every codebook starts on a 16-byte boundary)
-        const int chunks = entries * VEC * 2 / 16;
-        const uint4_t *src = reinterpret_cast<const uint4_t *>(cb + (int64_t)book * entries * VEC);
-        for (int i = threadIdx.x; i < chunks; i += kGemvWaves * 64) table[i] = src[i];
-    }
+    if ((int)threadIdx.x < chunks) table[threadIdx.x] = t0;
+    for (int i = threadIdx.x + kGemvWaves * 64; i < chunks; i += kGemvWaves * 64) table[i] = tsrc[i];
     __syncthreads();
 
     float acc[MX][kGemvRows];
@@ -215,6 +218,9 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_stream_kernel(con
     };
     int b = blockIdx.x;
     uint32_t cur[kGemvRows][RUNS], nxt[kGemvRows][RUNS];
+    // (the table entry's load goes out first: it is back, copied and published while the codes are on their way)
+    uint4_t entry = {0u, 0u, 0u, 0u};
+    if ((int)threadIdx.x < entries) entry = reinterpret_cast<const uint4_t *>(cb)[threadIdx.x];
     load_block(b, cur);
     uint4_t xr[RUNS][4];
 #pragma unroll
@@ -222,7 +228,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_stream_kernel(con
 #pragma unroll
         for (int c = 0; c < 4; c++) xr[q][c] = *reinterpret_cast<const uint4_t *>(x + (q * kRunCodes + 4 * lane + c) * 8);
     if ((int)threadIdx.x < entries) {
-        const uint4_t e = reinterpret_cast<const uint4_t *>(cb)[threadIdx.x];
+        const uint4_t e = entry;
         // (copy (l + i) % 16 in turn i: the sixteen lanes of a group write sixteen different bank groups)
 #pragma unroll
         for (int i = 0; i < kCopies; i++) table[threadIdx.x * kCopies + ((lane + i) & (kCopies - 1))] = e;
