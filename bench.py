@@ -35,8 +35,8 @@ HBM_PEAK_GBPS = 8000.0
 FP16_MFMA_PEAK_TFLOPS = 2500.0
 POOL_BYTES = 640 << 20  # distinct code matrices rotated through by the bandwidth-bound configs
 # HBM bytes one cold decode launch moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 256 MiB copy (summary under profiles/): 1098.5 KiB x 2.0 read + 8 KiB written.
-MEASURED_C2_HBM_BYTES_PER_LAUNCH = 2_257_920
+# 256 MiB copy (summary under profiles/): 1099.5 KiB x 2.0 read + 8 KiB written.
+MEASURED_C2_HBM_BYTES_PER_LAUNCH = 2_259_968
 
 
 def parse_args():
