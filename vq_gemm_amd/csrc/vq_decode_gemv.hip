@@ -1,6 +1,7 @@
-// Decode GEMV proper (one to four rows of X): y[m,n] = sum_k x[m,k] W[n,k], W given as codes and a codebook
-// (described below for 8-bit codes of 8-vectors; GemvCfg holds what changes with the format).  A short launch of this path is a chain of latencies, not
-// a stream, so the kernel is built to keep the chain short rather than to share work:
+// Decode GEMV proper (one to four rows of X): y[m,n] = sum_k x[m,k] W[n,k], W given as codes and a
+// codebook (described below for 8-bit codes of 8-vectors; GemvCfg holds what changes with the
+// format).  A short launch of this path is a chain of latencies, not a stream, so the kernel is
+// built to keep the chain short rather than to share work:
 //
 //   * A wave owns whole rows of W (four of them), so nothing is summed across waves: no partial
 //     sums in the LDS, no barrier behind the multiply.  A row's sum is folded inside the wave with
@@ -12,11 +13,13 @@
 //   * Lane l takes the codes 4l..4l+3 of every run of 256 codes: one dword load per row and run
 //     (a wave reads 256 contiguous bytes), x in 64-byte pieces per lane.
 //   * The only barrier publishes the codebook (4 KB, one 16-byte entry per thread) in the LDS; the
-//     gathers are 16-byte reads at code*16.
+//     gathers are 16-byte reads at code*16.  The codebook's load is the first one issued, so that
+//     its copy and the barrier pass while the codes are still on their way from HBM.
 //
 // Four waves per workgroup, 16 rows of W: as many workgroups as the batched kernel has tiles.  It
-// wins while a compute unit has a tile or two; for long runs of tiles the batched kernel, whose
-// waves share X and the table over many tiles, is the better stream.
+// wins while a compute unit has a few tiles; longer runs of rows go to the persistent form below
+// (decode_gemv_stream_kernel) and, beyond that, to the batched kernel, whose waves share X and the
+// table over many tiles.
 #include "vq_common.h"
 
 namespace vq {
