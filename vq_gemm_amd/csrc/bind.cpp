@@ -1,6 +1,7 @@
 // Torch extension boundary: the two functions the reference exports from bind.cpp:3-8,
 //   e2e_gemm(input, w, codebook) -> Tensor      gemm(input, w) -> Tensor
-// with the same positional signatures, plus dequant(w, codebook) -> Tensor.
+// with the same positional signatures (e2e_gemm also takes an optional `out=`), plus
+// dequant(w, codebook) -> Tensor.
 // This file is host-only C++: it validates tensors, allocates the result with torch's
 // allocator and forwards raw pointers and the current HIP stream to the C ABI of
 // libvqgemm.so (and libvqgemm_ref.so for the hipBLASLt baseline module).
@@ -11,6 +12,8 @@
 #include <torch/extension.h>
 #include <c10/hip/HIPStream.h>
 #include <c10/core/DeviceGuard.h>
+
+#include <cstdlib>
 
 #include "../../include/vq_gemm.h"
 #include "../../include/vq_gemm_ref.h"
@@ -99,7 +102,27 @@ Geometry classify(const torch::Tensor &input, const torch::Tensor &w, const torc
 
 #ifndef VQ_REF_MODULE
 
-torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codebook)
+// VQGEMM_CHECK_CODES=1 in the environment: every e2e_gemm / dequant call first verifies that all
+// codes are below the number of codebook entries (one extra pass over the codes and a
+// synchronisation), and raises instead of returning a result that depends on the kernel.
+bool check_codes_enabled()
+{
+    const char *e = std::getenv("VQGEMM_CHECK_CODES");
+    return e && e[0] != '\0' && e[0] != '0';
+}
+
+void check_code_range(const torch::Tensor &codes, int code_bits, int64_t entries, void *stream)
+{
+    if (!check_codes_enabled() || codes.numel() == 0 || entries >= (int64_t(1) << code_bits)) return;
+    torch::Tensor mx = torch::empty({1}, codes.options().dtype(torch::kInt32));
+    check_rc(vqgemm_max_code(codes.data_ptr(), codes.numel(), code_bits, mx.data_ptr(), stream), "code-range check");
+    const int64_t m = mx.item<int32_t>();
+    TORCH_CHECK(m < entries, "w holds the code ", m, " but the codebook has only ", entries, " entries");
+}
+
+// e2e_gemm(input, w, codebook[, out]): `out`, when given, receives the result (fp16 [M,N], contiguous,
+// on input's device) and is returned; the reference's three-argument call allocates as before.
+torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codebook, c10::optional<torch::Tensor> out_opt)
 {
     check_dev_tensor(input, "input");
     check_dev_tensor(w, "w");
@@ -109,38 +132,40 @@ torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codeb
     const Geometry g = classify(input, w, codebook);
     c10::DeviceGuard guard(input.device());
     torch::Tensor x = canon(input), c = canon(w), cb = canon(codebook);
-    torch::Tensor out = torch::empty({g.M, g.N}, input.options());
+    torch::Tensor out;
+    if (out_opt.has_value() && out_opt->defined()) {
+        out = *out_opt;
+        check_dev_tensor(out, "out");
+        TORCH_CHECK(out.device() == input.device(), "out must be on input's device");
+        TORCH_CHECK(out.scalar_type() == torch::kFloat16 && out.dim() == 2 && out.size(0) == g.M && out.size(1) == g.N,
+                    "out must be float16 [", g.M, ", ", g.N, "], got ", out.sizes());
+        TORCH_CHECK(out.is_contiguous() && (reinterpret_cast<uintptr_t>(out.data_ptr()) & 15) == 0,
+                    "out must be contiguous and 16-byte aligned");
+    } else {
+        out = torch::empty({g.M, g.N}, input.options());
+    }
+    check_code_range(c, g.code_bits, g.entries, cur_stream(input));
     torch::Tensor ws;
     void *ws_ptr = nullptr;
-    if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS && !g.is_a) {
-        ws = torch::empty({g.N, g.K}, input.options());
-        ws_ptr = ws.data_ptr();
-    }
     int rc;
     if (g.is_a) {
-        // Reference-native tensors.  The fused tiled kernel where it is expected to win (the reference's
-        // own scheme: codebooks in shared memory, W dequantised into a tile there).  Otherwise, and in
-        // the s1 module, the reference's two-pass strategy (strategy_1/src.cu:323-399): the bit-exact
-        // dequant kernel writes W_dec[K, 2*Nc], then a plain GEMM multiplies - this library's own in
-        // s1, as the reference's s1 keeps its own, a library GEMM (hipBLASLt) in the other modules.
-        const bool fused = VQ_VARIANT != VQGEMM_VARIANT_TWOPASS &&
-                           vqgemm_select_variant_a(g.M, g.K, g.Nc, 1) == VQGEMM_VARIANT_PREFILL;
-        if (fused) {
-            rc = vqgemm_e2e_gemm_a(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.Nc,
-                                   VQGEMM_VARIANT_PREFILL, nullptr, cur_stream(input));
-        } else {
-            torch::Tensor dec = torch::empty({g.K, g.N}, input.options());
-            rc = vqgemm_dequant_a(c.data_ptr(), cb.data_ptr(), dec.data_ptr(), g.K, g.Nc, cur_stream(input));
-            check_rc(rc, "e2e_gemm (dequant pass)");
-            if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS) {
-                rc = vqgemm_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, cur_stream(input));
-            } else {
-                const int rrc = vqref_gemm_f16(x.data_ptr(), dec.data_ptr(), out.data_ptr(), g.M, g.K, g.N, 0, cur_stream(input));
-                TORCH_CHECK(rrc == 0, "e2e_gemm (GEMM pass) failed: ", vqref_error_string(rrc), " (code ", rrc, ")");
-                rc = 0;
-            }
+        // Reference-native tensors.  The library chooses: its fused tiled kernel where that is expected
+        // to win (the reference's own scheme: codebooks in shared memory, W dequantised into a tile
+        // there), otherwise the reference's two-pass strategy (strategy_1/src.cu:323-399): the bit-exact
+        // dequant kernel writes W_dec[K, 2*Nc] into the scratch allocated here, then the library's own
+        // tiled MFMA GEMM multiplies.  The s1 module always takes the two-pass route.
+        const int variant = VQ_VARIANT == VQGEMM_VARIANT_TWOPASS ? VQGEMM_VARIANT_TWOPASS : VQGEMM_VARIANT_AUTO;
+        if (variant == VQGEMM_VARIANT_TWOPASS || vqgemm_select_variant_a(g.M, g.K, g.Nc, 1) == VQGEMM_VARIANT_TWOPASS) {
+            ws = torch::empty({g.K, g.N}, input.options());
+            ws_ptr = ws.data_ptr();
         }
+        rc = vqgemm_e2e_gemm_a(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.Nc, variant, ws_ptr,
+                               cur_stream(input));
     } else {
+        if (VQ_VARIANT == VQGEMM_VARIANT_TWOPASS) {
+            ws = torch::empty({g.N, g.K}, input.options());
+            ws_ptr = ws.data_ptr();
+        }
         rc = vqgemm_e2e_gemm_b(x.data_ptr(), c.data_ptr(), cb.data_ptr(), out.data_ptr(), g.M, g.K, g.N, g.vec,
                                g.entries, g.n_codebooks, g.code_bits, VQ_VARIANT, ws_ptr, cur_stream(input));
     }
@@ -180,6 +205,7 @@ torch::Tensor dequant(torch::Tensor w, torch::Tensor codebook)
     const bool is_a = w.scalar_type() == torch::kUInt8 && codebook.dim() == 3 && v == 2 && E == 256 && G * 4 == w.size(1);
     c10::DeviceGuard guard(w.device());
     torch::Tensor c = canon(w), cb = canon(codebook);
+    if (!is_a) check_code_range(c, w.scalar_type() == torch::kUInt8 ? 8 : 16, E, cur_stream(w));
     auto opts = codebook.options();
     if (is_a) {
         torch::Tensor out = torch::empty({w.size(0), 2 * w.size(1)}, opts);
@@ -216,9 +242,10 @@ torch::Tensor gemm(torch::Tensor input, torch::Tensor w)
 
 // The reference's baseline module also exports e2e_gemm, as a stub that returns zeros
 // (ref_gemm/cublas_gemm_fp16.cu:51-62, "Should not be called").  Same here.
-torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codebook)
+torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codebook, c10::optional<torch::Tensor> out_opt)
 {
     (void)codebook;
+    (void)out_opt;
     return torch::zeros({input.size(0), w.size(1)}, input.options());
 }
 
@@ -226,7 +253,8 @@ torch::Tensor e2e_gemm(torch::Tensor input, torch::Tensor w, torch::Tensor codeb
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
-    m.def("e2e_gemm", &e2e_gemm, "VQ GEMM");
+    m.def("e2e_gemm", &e2e_gemm, "VQ GEMM", pybind11::arg("input"), pybind11::arg("w"), pybind11::arg("codebook"),
+          pybind11::arg("out") = pybind11::none());
     m.def("gemm", &gemm, "Normal GEMM");
 #ifndef VQ_REF_MODULE
     m.def("dequant", &dequant, "Codes + codebook -> fp16 weights");

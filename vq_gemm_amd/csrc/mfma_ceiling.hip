@@ -5,7 +5,8 @@
 // operands the device runs into its power limit and lowers the clock, and how far depends on the
 // MFMA shape; this is the ceiling the prefill kernel is measured against.
 //
-// Stand-alone program (no library, no torch): prints one line per case with the time per launch,
+// Stand-alone measurement tool (no library, no torch), run by `bench.py --mfma-ceiling` and by the
+// bench's reporting leg; not part of libvqgemm.so.  Prints one line per case with the time per launch,
 // the rate, and the time, cycle count and clock seen from inside the kernel.
 #include <hip/hip_runtime.h>
 

@@ -318,6 +318,16 @@ int vqgemm_silu_mul(const void *gate_up, void *out, int64_t M, int64_t N, void *
                                             static_cast<hipStream_t>(stream)));
 }
 
+int vqgemm_max_code(const void *codes, int64_t count, int32_t code_bits, void *max_out, void *stream)
+{
+    if (count < 0) return VQGEMM_E_SHAPE;
+    if (code_bits != 8 && code_bits != 16) return VQGEMM_E_CODEBITS;
+    if (!max_out || (count > 0 && !codes)) return VQGEMM_E_NULL;
+    if (!aligned(max_out, 4) || !aligned(codes, code_bits / 8)) return VQGEMM_E_ALIGN;
+    return static_cast<int>(launch_max_code(codes, count, code_bits, static_cast<uint32_t *>(max_out),
+                                            static_cast<hipStream_t>(stream)));
+}
+
 int vqgemm_dequant_a(const void *w, const void *codebook, void *w_out, int64_t K, int64_t Nc, void *stream)
 {
     if (K < 0 || Nc < 0 || K > INT_MAX / 2 || Nc > INT_MAX / 4 || Nc % 4 != 0) return VQGEMM_E_SHAPE;

@@ -53,6 +53,18 @@ __device__ __forceinline__ half8_t as_half8(T v)
     return u.h;
 }
 
+// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
+// compiler knows nothing about this transfer (completion is only visible through vmcnt), so
+// every consumer sits behind an explicit vmcnt wait + barrier.  `lds_base` must be wave-uniform.
+// The statement writes m0 and says so, so that compiler-generated uses of m0 stay correct.
+__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+}
+
 // ---- launchers (defined one per .hip file) -------------------------------------------
 hipError_t launch_dequant_b(const ProblemB &p, half_t *w_out, hipStream_t s);
 hipError_t launch_dequant_a(const ProblemA &p, half_t *w_out, hipStream_t s);
@@ -117,6 +129,9 @@ hipError_t launch_fused_a(const ProblemA &p, hipStream_t s);
 
 // out[M,N] = silu(a[:, :N]) * a[:, N:] for a [M, 2N]
 hipError_t launch_silu_mul(const half_t *a, half_t *out, int64_t M, int64_t N, hipStream_t s);
+
+// out[0] = the largest code of codes[0 .. count) (0 when count == 0); out is device memory
+hipError_t launch_max_code(const void *codes, int64_t count, int code_bits, uint32_t *out, hipStream_t s);
 
 int device_cu_count();
 

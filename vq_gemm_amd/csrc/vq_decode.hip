@@ -211,16 +211,6 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");  // keep the compiler from moving LDS reads above the wait
 }
 
-// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].
-// `lds_base` must be wave-uniform; completion is only visible through vmcnt.
-__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base), "v"(voff), "s"(sbase)
-                 : "memory");
-}
-
 // ---- batched kernel -----------------------------------------------------------------------
 // The common case (one codebook, K a multiple of 256 and at most 4096, N a multiple of 16) gets
 // a loop that is lean in instructions: a CU issues one vector and one scalar instruction per

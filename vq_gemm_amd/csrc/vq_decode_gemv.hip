@@ -131,7 +131,12 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
 #pragma unroll
                 for (int d = 0; d < 4; d++) xr[m][q][4 * c + d] = v[d];
             }
-    if ((int)threadIdx.x < chunks) table[threadIdx.x] = t0;
+    // 8-bit codes: the whole table is written, zeros past a short codebook, so that a code at or past
+    // `entries` gathers a defined value (16-bit codes can point past any table: the LDS returns zero
+    // for reads outside the allocation, and short tables of that format are left as they are).
+    constexpr int kSlots = C::kTableBytes / 16;
+    static_assert(sizeof(CodeT) != 1 || kSlots <= kGemvWaves * 64, "one slot per thread covers a table of 8-bit codes");
+    if ((int)threadIdx.x < (sizeof(CodeT) == 1 ? kSlots : chunks)) table[threadIdx.x] = t0;
     for (int i = threadIdx.x + kGemvWaves * 64; i < chunks; i += kGemvWaves * 64) table[i] = tsrc[i];
     __syncthreads();
 
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_stream_kernel(con
     for (int q = 0; q < RUNS; q++)
 #pragma unroll
         for (int c = 0; c < 4; c++) xr[q][c] = *reinterpret_cast<const uint4_t *>(x + (q * kRunCodes + 4 * lane + c) * 8);
-    if ((int)threadIdx.x < entries) {
+    {   // (every thread writes: entries past a short codebook are zeros, so any 8-bit code gathers a defined value)
         const uint4_t e = entry;
         // (copy (l + i) % 16 in turn i: the sixteen lanes of a group write sixteen different bank groups)
 #pragma unroll

@@ -89,16 +89,6 @@ __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");  // keep the compiler from moving LDS reads above the wait
 }
 
-// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].
-// `lds_base` must be wave-uniform; completion is only visible through vmcnt.
-__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base), "v"(voff), "s"(sbase)
-                 : "memory");
-}
-
 // stage_off >= 0: the X slices are staged through the LDS at that offset (n_chunks == 1 only);
 // `aliased` says that the staging area overlaps the codebook, which is then loaded afterwards.
 //
@@ -399,8 +389,14 @@ hipError_t launch_decode_steps(const ProblemB &p, hipStream_t s)
 template <int VEC, typename CodeT>
 hipError_t launch_decode_typed(const ProblemB &p, hipStream_t s)
 {
-    // 512-wide K slices up to K = 4096 (eight waves cover it), 1024-wide beyond.
-    return p.K <= 8 * 512 ? launch_decode_steps<VEC, CodeT, 16>(p, s) : launch_decode_steps<VEC, CodeT, 32>(p, s);
+    // 512-wide K slices up to K = 4096 (eight waves cover it), 1024-wide beyond - for the code
+    // formats whose 1024-wide slice fits the registers (at most four lane loads per slice: 8-vectors,
+    // 4-vectors with 8-bit codes).  The others would spill; they keep 512-wide slices and walk a
+    // longer K in chunks.
+    if constexpr (DecodeCfg<VEC, CodeT, 32>::LPT <= 4) {
+        if (p.K > 8 * 512) return launch_decode_steps<VEC, CodeT, 32>(p, s);
+    }
+    return launch_decode_steps<VEC, CodeT, 16>(p, s);
 }
 
 template <int VEC, typename CodeT>

@@ -15,17 +15,6 @@ __device__ __forceinline__ void wait_vmcnt()
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-// 16-byte global load straight into the LDS: lane l writes smem[lds_base + 16*l ..].  The
-// compiler knows nothing about this transfer, so every consumer sits behind an explicit
-// wait_vmcnt + barrier.  `lds_base` must be wave-uniform.
-__device__ __forceinline__ void load_to_lds_16(uint32_t lds_base, uint32_t voff, const void *sbase)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(lds_base), "v"(voff), "s"(sbase)
-                 : "memory");
-}
-
 // acc += a . b with the accumulator pinned to one AGPR tuple.  Left to itself the register
 // allocator renames the 64 four-register accumulators from MFMA to MFMA and pays for it with
 // copies at the loop edge and with spills.  The compiler cannot see into the statement, so the

@@ -41,6 +41,7 @@ class VQLinear(torch.nn.Module):
         if self.bias is not None and self.bias.shape != (self.out_features,):
             raise ValueError("bias must have one entry per output feature")
         self.register_buffer("codes_packed", None, persistent=False)  # derived from `codes`: not part of the state
+        self._packed_from = None  # (version counter, address) of `codes` when `codes_packed` was made
 
     def prepack_for_decode(self) -> "VQLinear":
         """Keep a second copy of the codes in the decode kernel's packed layout (`cabi.pack_codes_b`;
@@ -52,7 +53,19 @@ class VQLinear(torch.nn.Module):
             self.codes_packed = cabi.pack_codes_b(self.codes, self.codebook.shape[-1])
         except cabi.VqGemmError as e:
             raise ValueError("the packed layout needs K % 256 == 0, out_features % 16 == 0 and vec in (2, 4, 8)") from e
+        self._packed_from = self._codes_key()
         return self
+
+    def _codes_key(self):
+        return (self.codes._version, self.codes.data_ptr())
+
+    def _fresh_packed_codes(self):
+        """The packed copy, re-made first if `codes` changed since it was packed (`load_state_dict`,
+        an in-place update, a move to another device): short and tall inputs must multiply by the
+        same weights."""
+        if self._packed_from != self._codes_key() or self.codes_packed.device != self.codes.device:
+            self.prepack_for_decode()
+        return self.codes_packed
 
     @classmethod
     def from_float(cls, weight: torch.Tensor, vec: int = 8, entries: int = 256, n_codebooks: int = 1,
@@ -83,7 +96,7 @@ class VQLinear(torch.nn.Module):
             g, e, v = cabi._cb_dims(self.codebook)
             dims = (x.numel() // x.shape[-1], x.shape[-1], self.out_features, v, e, g, 8 * self.codes.element_size())
             if cabi.select_variant_b(*dims) == cabi.VARIANT_DECODE and cabi.decode_packed_supports(*dims):
-                return vq_linear_packed(x, self.codes_packed, self.codebook, self.bias)
+                return vq_linear_packed(x, self._fresh_packed_codes(), self.codebook, self.bias)
         return vq_linear(x, self.codes, self.codebook, self.bias)
 
     def extra_repr(self) -> str:

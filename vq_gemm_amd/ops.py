@@ -36,9 +36,10 @@ def load_module(key: str = DEFAULT_VARIANT):
     return _modules[key]
 
 
-def e2e_gemm(input, w, codebook, variant: str = DEFAULT_VARIANT):
-    """Fused VQ GEMM; same positional arguments as the reference's e2e_gemm."""
-    return load_module(variant).e2e_gemm(input, w, codebook)
+def e2e_gemm(input, w, codebook, variant: str = DEFAULT_VARIANT, out=None):
+    """Fused VQ GEMM; same positional arguments as the reference's e2e_gemm.  `out` (fp16 [M,N],
+    contiguous, on input's device) receives the result instead of a new tensor."""
+    return load_module(variant).e2e_gemm(input, w, codebook, out=out)
 
 
 def gemm(input, w, variant: str = DEFAULT_VARIANT):

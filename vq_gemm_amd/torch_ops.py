@@ -20,6 +20,8 @@ from . import cabi
 def _out_shape(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor):
     if codes.dim() != 2 or codebook.dim() not in (2, 3) or x.dim() < 1:
         raise ValueError("vq_linear: x [..., K], codes [N, K/vec], codebook [E, vec] or [G, E, vec]")
+    if codes.dtype not in (torch.uint8, torch.uint16):
+        raise ValueError(f"vq_linear: codes must be uint8 or uint16, got {codes.dtype}")
     if x.shape[-1] != codes.shape[1] * codebook.shape[-1]:
         raise ValueError(f"vq_linear: x has {x.shape[-1]} features, codes x vec give {codes.shape[1] * codebook.shape[-1]}")
     return (*x.shape[:-1], codes.shape[0])
