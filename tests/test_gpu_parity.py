@@ -622,7 +622,8 @@ def test_random_shapes_agree_across_kernels():
         y_scalar = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_GENERIC, bias=bias)
         ref = y_scalar.float()
         # the oracle on the same inputs (fp64 sums, the bias added before the one rounding)
-        want = vo.vq_gemm_b(_np(x), _np(codes), _np(cb), acc=np.float64)
+        # (the unrounded product in float64: the oracle's own GEMM returns it rounded to fp16)
+        want = _np(x).astype(np.float64) @ vo.dequant_b(_np(codes), _np(cb)).astype(np.float64).T
         if bias is not None:
             want = want + _np(bias).astype(np.float64)[None, :]
         e1, _ = vo.rel_err(_np(y_scalar), want)
@@ -1138,11 +1139,11 @@ def test_code_range_check_and_defined_results_for_codes_past_a_short_table(monke
 
 def test_vqlinear_repacks_after_its_codes_change():
     from vq_gemm_amd.nn import VQLinear
-    spec = ProblemSpec("lin", GEOM_B, 1, 4096, 8192, 8, 256, 1, 8)   # a shape the K-sliced decode kernel takes
+    spec = ProblemSpec("lin", GEOM_B, 16, 4096, 8192, 8, 256, 1, 8)   # a shape the K-sliced decode kernel takes
     x, codes, cb = make_problem(spec, seed=1, device=DEV)
     _, codes2, _ = make_problem(spec, seed=2, device=DEV)
     layer = VQLinear(codes.clone(), cb).prepack_for_decode()
-    dims = (1, spec.K, spec.N, 8, 256, 1, 8)
+    dims = (16, spec.K, spec.N, 8, 256, 1, 8)
     assert cabi.select_variant_b(*dims) == cabi.VARIANT_DECODE and cabi.decode_packed_supports(*dims)
     assert torch.equal(layer(x), cabi.e2e_gemm_b(x, codes, cb))
     state = {k: v.clone() for k, v in layer.state_dict().items()}
