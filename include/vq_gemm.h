@@ -32,6 +32,7 @@ extern "C" {
 #define VQGEMM_E_CODEBITS (-3)  /* code_bits not 8/16, or entries > 2^code_bits */
 #define VQGEMM_E_VARIANT (-4)   /* unknown variant, or the variant cannot serve this shape */
 #define VQGEMM_E_ALIGN (-5)     /* a pointer is not aligned to its element size */
+#define VQGEMM_E_SCRATCH (-6)   /* the problem needs more scratch than the library's fixed device array holds */
 
 /* kernel selection for the fused GEMM */
 #define VQGEMM_VARIANT_AUTO 0     /* pick by shape */
@@ -97,6 +98,25 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
 int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *out,
                       int64_t M, int64_t K, int64_t Nc, int32_t variant,
                       void *workspace, void *stream);
+
+/*
+ * vqgemm_e2e_gemm_a without a workspace argument and without any allocation: the scratch of the
+ * two-pass route (W_dec[K, 2*Nc] fp16) is a fixed device array inside the library,
+ * VQGEMM_NOALLOC_SCRATCH_BYTES large, which every GPU the library runs on holds from load to the
+ * end of the process.  No counterpart in the reference (its s1 wrapper allocates the intermediate
+ * tensor per call, strategy_1/src.cu:351); it is for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call makes no hipMalloc,
+ * hipFree or other allocating call.  Same arguments, same kernels, same results as
+ * vqgemm_e2e_gemm_a with a workspace; shapes with K * 2*Nc * 2 bytes beyond the array are refused
+ * with VQGEMM_E_SCRATCH, whichever route they would take.  All calls on one GPU share that GPU's
+ * array: calls that overlap in time on one GPU (different streams) race on it.  Nothing in it has to
+ * be cleared between calls - the dequant pass overwrites every element the GEMM pass reads.  The
+ * first call on a device looks the array's address up (which makes the runtime load the code object
+ * that holds it); make that call outside stream capture.
+ */
+#define VQGEMM_NOALLOC_SCRATCH_BYTES (16 << 20)
+int vqgemm_e2e_gemm_a_noalloc(const void *x, const void *w, const void *codebook, void *out,
+                              int64_t M, int64_t K, int64_t Nc, int32_t variant, void *stream);
 
 /*
  * Which kernel VQGEMM_VARIANT_AUTO resolves to for a geometry-A shape with 16-byte aligned operands

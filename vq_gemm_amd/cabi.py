@@ -24,6 +24,7 @@ _SIGNATURES = {
     "vqgemm_e2e_gemm_b": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_b_bias": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_a": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _P]),
+    "vqgemm_e2e_gemm_a_noalloc": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P]),
     "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
     "vqgemm_dequant_a": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "vqgemm_encode_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
@@ -212,6 +213,21 @@ def e2e_gemm_a(x, w, codebook, variant=VARIANT_AUTO, out=None, workspace=None):
                                  _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_e2e_gemm_a")
+    return out
+
+
+def e2e_gemm_a_noalloc(x, w, codebook, out, variant=VARIANT_AUTO):
+    """vqgemm_e2e_gemm_a_noalloc: geometry A with the library's own fixed scratch array.  `out` is required
+    (the call itself allocates nothing); raises VqGemmError(-6) when W_dec would not fit the array."""
+    _require(x.dim() == 2, "x must be [M, K]")
+    M, K = x.shape
+    _check_f16(x, (M, K), "x")
+    _, Nc = _check_geometry_a(w, codebook, K)
+    _same_device(x, w, codebook, out)
+    _check_f16(out, (M, 2 * Nc), "out")
+    rc = lib().vqgemm_e2e_gemm_a_noalloc(_ptr(x), _ptr(w), _ptr(codebook), _ptr(out), M, K, Nc, variant, _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_e2e_gemm_a_noalloc")
     return out
 
 

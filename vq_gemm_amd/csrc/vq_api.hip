@@ -113,6 +113,7 @@ const char *vqgemm_error_string(int code)
     case VQGEMM_E_CODEBITS: return "code_bits must be 8 or 16 and entries <= 2^code_bits";
     case VQGEMM_E_VARIANT: return "unknown kernel variant, or the variant cannot serve this shape";
     case VQGEMM_E_ALIGN: return "pointer not aligned as the selected kernel requires";
+    case VQGEMM_E_SCRATCH: return "the problem needs more scratch than the library's fixed device array holds";
     default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
