@@ -229,8 +229,10 @@ def test_packed_codes_small_shapes_bias_and_rejections():
     assert cabi.select_variant_b(2, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(3, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
-    assert cabi.select_variant_b(1, 4096, 131072, 8, 256, 1, 8) == cabi.VARIANT_DECODE
-    assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 2, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(1, 4096, 131072, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
+    assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 2, 8) == cabi.VARIANT_DECODE_GEMV
+    assert cabi.select_variant_b(1, 4096, 64 * 16 * 256 + 16, 8, 256, 1, 8) == cabi.VARIANT_DECODE   # more than 64 rows per wave
+    assert cabi.select_variant_b(1, 4096, 32768, 4, 256, 1, 8) == cabi.VARIANT_DECODE               # other code formats
     assert cabi.pack_codes_b(torch.zeros(0, 64, dtype=torch.uint8, device=DEV), 8).shape == (0, 64)
 
 
@@ -243,7 +245,14 @@ GEMV_B = [
     ("four_runs", 8192, 2048, 256, 1, 1),
     ("16_row_books", 2048, 256, 256, 16, 1),
     ("many_tiles", 4096, 32768, 256, 1, 1),
-    ("many_tiles_two_books", 4096, 32768, 256, 2, 1),   # not the streaming form: one codebook only
+    ("many_tiles_two_books", 4096, 32768, 256, 2, 1),
+    # the wide form (one row of X from one row per wave on): rows that do not divide by anything, workgroups whose
+    # rows reach into a second codebook (two tables), small codebooks, short codebooks
+    ("wide_ragged_n", 4096, 5003, 256, 1, 1),
+    ("wide_three_books_straddled", 2048, 12288, 256, 3, 1),
+    ("wide_128_row_books_straddled", 4096, 6144, 256, 48, 1),
+    ("wide_128_row_books_aligned", 2048, 8192, 200, 64, 1),
+    ("wide_four_runs_two_books", 8192, 4096 + 32, 256, 2, 1),
     ("many_tiles_three_runs_ragged_walk", 6144, 16 * 1500, 256, 1, 1),
     ("many_tiles_one_run", 2048, 65536, 77, 1, 1),
     ("two_rows_of_x", 4096, 4096, 256, 1, 2),
@@ -281,6 +290,33 @@ def test_gemv_kernel_few_rows_of_x(row):
     # the K-sliced MFMA kernel and the automatic choice on the same inputs: same product within the bar
     _check_gemm(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE), x, codes, cb, what=name + " (decode)")
     _check_gemm(cabi.e2e_gemm_b(x, codes, cb), x, codes, cb, what=name + " (auto)")
+
+
+def test_gemv_wide_form_at_its_longest_64_rows_per_wave():
+    """As many rows as the wide form takes: one result per lane, 63 or 64 rows per wave on a 256-CU device.  The oracle
+    multiplies a sample of the rows (rows are independent): the first and last rows and a few thousand others."""
+    K, N = 2048, 64 * 16 * 256 - 777
+    spec = ProblemSpec("wide_longest", GEOM_B, 1, K, N, 8, 256, 1, 8)
+    x, codes, cb = make_problem(spec, seed=33, device=DEV)
+    _say("gemv wide, long", spec)
+    y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(5)
+    rows = np.unique(np.concatenate([np.arange(0, 400), np.arange(N - 400, N), rng.integers(0, N, 4000)]))
+    ref = vo.vq_gemm_b(_np(x), _np(codes)[rows], _np(cb), acc=np.float64)
+    e1, e2 = vo.rel_err(_np(y)[:, rows], ref)
+    _say(f"  sampled rows: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+    assert e1 <= TOL
+    # every row against the K-sliced MFMA kernel (pinned against the oracle elsewhere)
+    yd = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
+    scale = yd.float().abs().max().item()
+    assert ((y.float() - yd.float()).abs().max() / scale).item() <= TOL
+    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb), y)   # the automatic choice is this kernel, and it is deterministic
+    # one row more per wave than it takes, in a shape the four-wave kernel refuses as well (N not a multiple of 16)
+    n_big = 64 * 16 * 256 + 8
+    with pytest.raises(cabi.VqGemmError) as ei:
+        cabi.e2e_gemm_b(x, torch.zeros(n_big, K // 8, dtype=torch.uint8, device=DEV), cb, variant=cabi.VARIANT_DECODE_GEMV)
+    assert ei.value.code == -4
 
 
 GEMV_FORMATS = [

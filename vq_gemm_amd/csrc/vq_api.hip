@@ -88,6 +88,7 @@ ProblemB make_b(const void *x, const void *codes, const void *codebook, void *y,
 int select_b(const ProblemB &p, bool all_aligned16)
 {
     if (p.K == 0 || !all_aligned16) return VQGEMM_VARIANT_GENERIC;
+    if (decode_gemv_wide_preferred(p)) return VQGEMM_VARIANT_DECODE_GEMV;  // (also shapes the K-sliced kernels refuse)
     const bool prefill_ok = prefill_supports(p);
     if (decode_supports(p) && (!prefill_ok || decode_preferred(p)))
         return decode_gemv_preferred(p) ? VQGEMM_VARIANT_DECODE_GEMV : VQGEMM_VARIANT_DECODE;

@@ -91,8 +91,10 @@ bool decode_packed_supports(const ProblemB &p);
 // whole rows of W per wave; the automatic choice takes it while a compute unit has few rows to do
 bool decode_gemv_supports(const ProblemB &p);
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s);
-// the persistent form of the GEMV kernel that launch_decode_gemv takes for long runs of rows (one row of X, one codebook)
-bool decode_gemv_stream_supports(const ProblemB &p);
+// the wide form of the GEMV kernel (one 16-wave workgroup per compute unit, one row of X, 8-vectors, 8-bit
+// codes) and whether launch_decode_gemv takes it for the shape (from one row per wave on)
+bool decode_gemv_wide_supports(const ProblemB &p);
+bool decode_gemv_wide_preferred(const ProblemB &p);
 // whether the automatic choice takes the GEMV kernel rather than launch_decode_b for a shape both serve
 bool decode_gemv_preferred(const ProblemB &p);
 // the general kernel behind launch_decode_b: one slab of at most 16 rows of X

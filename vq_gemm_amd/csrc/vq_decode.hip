@@ -814,12 +814,16 @@ bool decode_preferred(const ProblemB &p)
     return t_decode <= t_prefill;
 }
 
-// The GEMV kernel has no work shared between its waves and a short chain of latencies; the batched
-// kernel streams long runs of tiles better.  Measured on a 256-CU MI355X at K = 4096 (us, batched ->
-// GEMV, cold HBM): 1 tile of 16 rows per compute unit 4.96 -> 3.85, 2 tiles 6.0 -> 4.8, 4 tiles
-// 7.5 -> 6.6, 8 tiles 11.1 -> 11.1; K = 8192 (x takes 64 registers, two waves per SIMD) is a tie
-// already at 2 tiles.  Two rows of X (every gathered codeword meets both): one tile per unit 5.0 -> 4.8,
-// two tiles a tie; three and four rows lose everywhere (5.1 -> 5.6 and 6.6 on one tile).
+// The GEMV kernels have no work shared between their waves.  One row of X in the first format
+// (8-vectors, 8-bit codes, at most two codebooks per workgroup's share of the rows) goes to the wide
+// form from one row per wave on (4096 rows on a 256-CU device): measured against the batched kernel
+// on a 256-CU MI355X, cold HBM, K = 4096: N = 4096 4.96 -> 3.4 us, N = 16384 7.5 -> 5.1, N = 28672
+// 9.9 -> 7.1, N = 65536 15.6 -> 12.4; K = 8192: N = 8192 8.3 -> 5.6, N = 28672 18.3 -> 10.8.
+// The four-wave kernel takes what is left where it was measured faster than the batched kernel
+// (us, batched -> GEMV, cold HBM, K = 4096): 1 tile of 16 rows per compute unit 4.96 -> 3.85, 2 tiles
+// 6.0 -> 4.8, 4 tiles 7.5 -> 6.6, 8 tiles 11.1 -> 11.1; K = 8192 (x takes 64 registers, two waves per
+// SIMD) is a tie already at 2 tiles.  Two rows of X (every gathered codeword meets both): one tile per
+// unit 5.0 -> 4.8, two tiles a tie; three and four rows lose everywhere (5.1 -> 5.6 and 6.6 on one tile).
 #ifndef VQ_GEMV_MAX_TILES_PER_CU
 #define VQ_GEMV_MAX_TILES_PER_CU 4
 #endif
@@ -827,21 +831,16 @@ constexpr int kGemvAutoMaxK = 6144;
 
 bool decode_gemv_preferred(const ProblemB &p)
 {
-    // (one row of X and one codebook: the GEMV path walks longer runs with its streaming kernel, which
-    // beats the batched kernel on the plain code matrix up to about 16 tiles per unit - 8 tiles 11.1 ->
-    // 9.6 us cold, 16 tiles 14.8 -> 13.4 warm - and falls behind at 32)
+    if (decode_gemv_wide_preferred(p)) return true;
     // Other code formats (same kernel, other gather width): one row of X only, and not with a table
     // of more than 32 KB, which every workgroup has to fill (us cold at K = 4096, batched -> GEMV:
     // 4-vectors / 8-bit codes N = 4096 5.0 -> 4.2, N = 16384 9.2 -> 7.3; 2-vectors 6.0 -> 5.6; 4-vectors /
     // 16-bit codes / 4096 entries N = 11008 9.9 -> 9.5; 8-vectors / 16-bit codes / 4096 entries 5.6 -> 5.9).
     const bool first_format = p.vec == 8 && p.code_bits == 8;
     if (!first_format && (p.M != 1 || (int64_t)p.entries * p.vec * 2 > 32 * 1024)) return false;
-    const int max_tiles_per_cu = p.M == 1 ? (decode_gemv_stream_supports(p) ? 16 : VQ_GEMV_MAX_TILES_PER_CU) : (p.M == 2 ? 1 : 0);
+    const int max_tiles_per_cu = p.M == 1 ? VQ_GEMV_MAX_TILES_PER_CU : (p.M == 2 ? 1 : 0);
     if (!decode_gemv_supports(p) || p.N / kTileN > max_tiles_per_cu * device_cu_count()) return false;
-    // K = 8192: only where the streaming form runs and up to 8 blocks per unit (us cold, batched -> GEMV:
-    // N = 16384 12.6 -> 11.3, N = 28672 18.3 -> 17.0, N = 57344 27.0 -> 29.9)
-    const int tiles = p.N / kTileN, cus = device_cu_count();
-    return p.K <= kGemvAutoMaxK || (decode_gemv_stream_supports(p) && tiles >= 4 * cus && tiles <= 8 * cus);
+    return p.K <= kGemvAutoMaxK;
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)

@@ -17,10 +17,13 @@
 //     its copy and the barrier pass while the codes are still on their way from HBM.
 //
 // Four waves per workgroup, 16 rows of W: as many workgroups as the batched kernel has tiles.  It
-// wins while a compute unit has a few tiles; longer runs of rows go to the persistent form below
-// (decode_gemv_stream_kernel) and, beyond that, to the batched kernel, whose waves share X and the
-// table over many tiles.
+// serves two to four rows of X, the other code formats and launches with fewer rows than the device
+// has waves; one row of X in the first format goes to the wide form below (decode_gemv_wide_kernel)
+// from one row per wave on.
 #include "vq_common.h"
+
+#include <limits.h>
+#include <type_traits>
 
 namespace vq {
 
@@ -191,121 +194,310 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     }
 }
 
-// The same for long runs of rows: two workgroups per compute unit (four waves alone do not cover the
-// latency of their own gathers; 64 KB of table each), each walking 16-row blocks of W with x and the
-// table kept.  What a block no longer pays (x, the table, the launch of its
-// waves) buys a bank-replicated table - one 256-byte bank row per entry holding 16 copies, lane l
-// reading copy l % 16, so that the gathers are free of bank conflicts - and the codes of the next
-// block are requested before the current one is multiplied.  One row of X, one codebook.
-template <int RUNS>
-__global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_stream_kernel(const half_t *__restrict__ x,
-                                                                              const uint8_t *__restrict__ codes,
-                                                                              const half_t *__restrict__ cb,
-                                                                              half_t *__restrict__ y,
-                                                                              const half_t *__restrict__ bias,
-                                                                              int n_blocks, int entries)
+// ---- the wide form: long runs of rows, and every single-row launch of at least one row per wave -------
+// One workgroup of sixteen waves per compute unit over a bank-replicated table (64 KB: 16 copies of
+// each entry in one 256-byte bank row, lane l reading copy l % 16, so the gathers never collide):
+// four waves per SIMD cover the latency of each other's gathers.  One row of X, 8-vectors, 8-bit codes.
+//   * The rows of W are dealt out to the waves of the whole grid in contiguous runs of equal length
+//     (one more for the first N % waves), so no unit idles while another finishes a longer share.
+//     A workgroup's rows may reach into a second codebook: it then holds two tables (128 KB) and a
+//     row picks its table through the third byte of the gather address.
+//   * x goes through the LDS once per workgroup (4 to 16 KB, laid out so that a wave reads its 16-byte
+//     pieces side by side): sixteen waves each pulling all of x through the L1 would cost more than
+//     the table.
+//   * A wave works through its rows in groups of G, the codes of the next NBUF - 1 groups already
+//     requested.  The loop holds no store: a wave keeps the result of its i-th row in lane i (at most
+//     64 rows per wave) and writes them all at the end, so the only outstanding vector-memory operations inside the loop
+//     are the code loads, they complete in order, and the compiler's own wait counts stay exact (a
+//     pending store would make it drain every load).  The loads are unconditional (past the end the
+//     last group is requested again) and only the multiply is skipped, for the same reason: a load
+//     inside a branch would make the counts at the join imprecise.
+//   * A row's sum is folded with six DPP additions (the last two broadcast row totals onward, so that
+//     lane 63 holds the sum in a fixed order) and one lane read.
+constexpr int kWideWaves = 16;
+constexpr int kWideCopies = 16;
+constexpr int kWideTableBytes = 256 * kWideCopies * 16;  // 64 KB
+
+// (One instruction each: the rows the mask leaves out keep their value, which the compiler does not
+// express through the builtin.  The s_nop covers the two wait states a DPP read needs behind a VALU write.)
+__device__ __forceinline__ float dpp_add_row_bcast15(float v)
 {
-#ifndef VQ_GEMV_STREAM_COPIES
-#define VQ_GEMV_STREAM_COPIES 16
-#endif
-#ifndef VQ_GEMV_STREAM_WGS_PER_CU
-#define VQ_GEMV_STREAM_WGS_PER_CU 2
-#endif
-    constexpr int kCopies = VQ_GEMV_STREAM_COPIES;
-    __shared__ __align__(16) uint4_t table[256 * kCopies];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    constexpr int J = RUNS * kRunCodes;  // codes per row
-    const uint8_t *lane_codes = codes + (int64_t)(wave * kGemvRows) * J + 4 * lane;
-    auto load_block = [&](int b, uint32_t (&cw)[kGemvRows][RUNS]) {
+    // lane 15 of rows 0 and 2 is added to every lane of rows 1 and 3
+    asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ float dpp_add_row_bcast31(float v)
+{
+    // lane 31 is added to every lane of rows 2 and 3
+    asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf" : "+v"(v));
+    return v;
+}
+
+// Sum of v over the 64 lanes, valid in lane 63 (returned from there as a wave-uniform value).
+__device__ __forceinline__ float wave_sum_to_uniform(float v)
+{
+    v = dpp_add_quad_perm_1032(v);
+    v = dpp_add_quad_perm_2301(v);
+    v = dpp_add_row_half_mirror(v);
+    v = dpp_add_row_mirror(v);
+    v = dpp_add_row_bcast15(v);
+    v = dpp_add_row_bcast31(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// floor(x / d) for 0 <= x < 2^23 or so through a float reciprocal and one correction step; rcp = 1.0f / d.
+__device__ __forceinline__ int small_quotient(int x, int d, float rcp)
+{
+    int q = (int)((float)x * rcp);
+    const int rem = x - q * d;
+    q += rem >= d ? 1 : 0;
+    q -= rem < 0 ? 1 : 0;
+    return q;
+}
+
+// BOOKS: 0 = one codebook; 1 = several, no workgroup's rows reach into a second one; 2 = some workgroup's rows
+// do, and every workgroup then fills two tables.  (A compile-time flag, like the unconditional loads below: a
+// load inside a branch makes the compiler's wait counts at the join imprecise, and the table would then
+// wait for the codes.)
+//
+// The order of the prologue matters more than its length suggests.  Loads complete in the order they were
+// issued, so what is issued behind the code loads (which come from HBM) is only usable once they have
+// landed: the table entry and the piece of x (both out of the L2) go out first, the code loads right
+// behind them.  And a launch starts with a cold instruction cache, so every instruction ahead of these
+// loads delays the one wait that cannot be shortened: nothing is computed ahead of them that they do not need.
+template <int RUNS, int G, int NBUF, int BOOKS>
+__global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const half_t *__restrict__ x,
+                                                                           const uint8_t *__restrict__ codes,
+                                                                           const half_t *__restrict__ cb,
+                                                                           half_t *__restrict__ y,
+                                                                           const half_t *__restrict__ bias, int entries,
+                                                                           int rows_q, int rows_r, int rows_per_cb,
+                                                                           float rcp_rows_per_cb, int n_books, int n_total)
+{
+    constexpr bool TWO = BOOKS == 2;
+    constexpr int kXChunks = RUNS * kRunCodes;  // 16-byte pieces of x
+    // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
+    // permute) | table of the second one (TWO) | x
+    constexpr int kTableSlots = (TWO ? 2 : 1) * 256 * kWideCopies;
+    __shared__ __align__(16) uint4_t lds[kTableSlots + kXChunks];
+    uint4_t *table = lds, *xs = lds + kTableSlots;
+    // All kernel arguments are fetched at once: left to first use, each pointer costs the prologue a
+    // scalar-load round trip of its own.
+    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(bias), "s"(entries), "s"(rows_q), "s"(rows_r), "s"(rows_per_cb),
+                 "s"(rcp_rows_per_cb), "s"(n_books), "s"(n_total));
+    const int tid = threadIdx.x;
+    constexpr int J = RUNS * kRunCodes;  // codes (bytes) per row
+
+    // The prologue's duties are split between the waves so that each has little queued ahead of its code loads:
+    // waves 0-7 fetch the table (two threads per entry), waves 8-15 fetch x (one or two pieces per thread).
+    // These loads sit in wave-uniform branches; the code loads behind them are unconditional, so the wait
+    // counts stay exact (the conditional loads are older than the code loads on every path).
+    int book0 = 0, second_book_row = INT_MAX;  // the workgroup's first codebook; rows from second_book_row on read the second table
+    if constexpr (BOOKS > 0) {
+        const int wg_row0 = min((int)blockIdx.x * kWideWaves * rows_q + min((int)blockIdx.x * kWideWaves, rows_r), n_total - 1);
+        book0 = small_quotient(wg_row0, rows_per_cb, rcp_rows_per_cb);
+        if (TWO) second_book_row = (book0 + 1) * rows_per_cb;
+    }
+    // (only the workgroups whose rows cross into the next codebook fetch and fill the second table)
+    const int wg_row1 = ((int)blockIdx.x + 1) * kWideWaves * rows_q + min(((int)blockIdx.x + 1) * kWideWaves, rows_r);
+    const bool second_table = TWO && second_book_row < wg_row1;
+    constexpr int kDutyThreads = kWideWaves * 64 / 2;
+    constexpr int kXPerThread = (kXChunks + kDutyThreads - 1) / kDutyThreads;
+    const bool table_duty = tid < kDutyThreads;
+    const int e = tid >> 1, half_of_copies = tid & 1;   // table duty: entry and which eight of its sixteen copies
+    const int xt = tid - kDutyThreads;                  // x duty: pieces xt, xt + 512
+    uint4_t entry0 = {0u, 0u, 0u, 0u}, entry1 = {0u, 0u, 0u, 0u};
+    uint4_t xpiece[kXPerThread];
+    if (table_duty) {
+        // (entries past a short codebook are loaded clamped and zeroed afterwards)
+        const int ec = min(e, entries - 1);
+        entry0 = reinterpret_cast<const uint4_t *>(cb + (int64_t)book0 * entries * 8)[ec];
+        if (second_table) entry1 = reinterpret_cast<const uint4_t *>(cb + (int64_t)min(book0 + 1, n_books - 1) * entries * 8)[ec];
+    } else {
 #pragma unroll
-        for (int r = 0; r < kGemvRows; r++)
+        for (int i = 0; i < kXPerThread; i++) xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, kXChunks - 1)];
+    }
+
+    // the wave's rows [row0, row0 + n_rows): at most 64, one result per lane
+    const uint32_t lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int gw = blockIdx.x * kWideWaves + wave;
+    const int row0 = gw * rows_q + min(gw, rows_r);
+    const int n_rows = rows_q + (gw < rows_r ? 1 : 0);
+    const int n_groups = (n_rows + G - 1) / G;
+    const int last_row = min(row0 + max(n_rows, 1), n_total) - 1;  // (a wave without rows reads the last row)
+
+    uint32_t cw[NBUF][G][RUNS];
+    auto load_group = [&](int g, uint32_t (&dst)[G][RUNS]) {
+#pragma unroll
+        for (int r = 0; r < G; r++) {
+            // (a wave-uniform row pointer and the lane as a 32-bit index: one scalar base per row, no vector address arithmetic)
+            const uint32_t *row = reinterpret_cast<const uint32_t *>(codes + (int64_t)min(row0 + g * G + r, last_row) * J);
 #pragma unroll
             for (int q = 0; q < RUNS; q++)
-                cw[r][q] = *reinterpret_cast<const uint32_t *>(lane_codes + ((int64_t)b * kGemvTile + r) * J + q * kRunCodes);
+                // (a relaxed atomic load of wavefront scope is an ordinary load instruction that the compiler
+                // leaves where it is written: ahead of the table's stores and the barrier)
+                dst[r][q] = __hip_atomic_load(row + q * (kRunCodes / 4) + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
     };
-    int b = blockIdx.x;
-    uint32_t cur[kGemvRows][RUNS], nxt[kGemvRows][RUNS];
-    // (the table entry's load goes out first: it is back, copied and published while the codes are on their way)
-    uint4_t entry = {0u, 0u, 0u, 0u};
-    if ((int)threadIdx.x < entries) entry = reinterpret_cast<const uint4_t *>(cb)[threadIdx.x];
-    load_block(b, cur);
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; u++) load_group(min(u, max(n_groups, 1) - 1), cw[u]);
+
+    if (table_duty) {
+        // Table: thread (e, h) writes copies 8h .. 8h+7 of entry e, in an order that sends the sixteen lanes
+        // served together to sixteen different copies (bank groups).  Entries past a short codebook are zeros,
+        // so any 8-bit code gathers a defined value.
+        if (e >= entries) entry0 = entry1 = uint4_t{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 8; i++) table[e * kWideCopies + half_of_copies * 8 + ((e + i) & 7)] = entry0;
+        if (second_table) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) table[256 * kWideCopies + e * kWideCopies + half_of_copies * 8 + ((e + i) & 7)] = entry1;
+        }
+    } else {
+        // x: piece i = q*256 + 4*l + c (the 8 halves that code c of lane l's dword in run q meets) is kept at
+        // q*256 + c*64 + l, so that the lanes of a wave read 64 neighbouring pieces.
+#pragma unroll
+        for (int i = 0; i < kXPerThread; i++) {
+            const int xi = xt + i * kDutyThreads;
+            if (xi < kXChunks) xs[(xi & ~255) + (xi & 3) * 64 + ((xi >> 2) & 63)] = xpiece[i];
+        }
+    }
+    __syncthreads();
+    if (n_rows <= 0) return;
     uint4_t xr[RUNS][4];
 #pragma unroll
     for (int q = 0; q < RUNS; q++)
 #pragma unroll
-        for (int c = 0; c < 4; c++) xr[q][c] = *reinterpret_cast<const uint4_t *>(x + (q * kRunCodes + 4 * lane + c) * 8);
-    {   // (every thread writes: entries past a short codebook are zeros, so any 8-bit code gathers a defined value)
-        const uint4_t e = entry;
-        // (copy (l + i) % 16 in turn i: the sixteen lanes of a group write sixteen different bank groups)
+        for (int c = 0; c < 4; c++) xr[q][c] = xs[q * kRunCodes + c * 64 + lane];
+
+    // Gather address = table * 65536 + code * 256 + copy * 16, put together by one byte permute out of the
+    // lane's dword of codes (byte 1) and a per-row base (bytes 0 and 2).
+    const uint32_t copy_base = (lane & (kWideCopies - 1)) * 16u;
+    const uint8_t *tbl = reinterpret_cast<const uint8_t *>(table);
+    float res = 0.f;  // lane i: the sum of the wave's row i
+    // rows [g*G, g*G + R) of the wave, R <= G (a compile-time count: the last group may be short)
+    auto multiply_rows = [&](int g, const uint32_t (&cur)[G][RUNS], auto r_const) {
+        constexpr int R = decltype(r_const)::value;
+        float acc[R];
+        uint32_t base[R];
 #pragma unroll
-        for (int i = 0; i < kCopies; i++) table[threadIdx.x * kCopies + ((lane + i) & (kCopies - 1))] = e;
-    }
-    __syncthreads();
-    const uint32_t copy = lane & (kCopies - 1);
-    for (; b < n_blocks; b += gridDim.x) {
-        const int bn = b + gridDim.x;
-        if (bn < n_blocks) load_block(bn, nxt);
-        float acc[kGemvRows];
+        for (int r = 0; r < R; r++) {
+            acc[r] = 0.f;
+            base[r] = TWO ? copy_base | (row0 + g * G + r >= second_book_row ? 0x10000u : 0u) : copy_base;
+        }
 #pragma unroll
-        for (int r = 0; r < kGemvRows; r++) acc[r] = 0.f;
+        for (int q = 0; q < RUNS; q++) {
+            // the four gathers of every row's dword go out together, the sixteen products follow
+            uint4_t w[R][4];
 #pragma unroll
-        for (int q = 0; q < RUNS; q++)
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    // result bytes: 0 = byte 0 of the base, 1 = byte c of the codes, 2 = byte 2 of the base, 3 = zero
+                    const uint32_t addr = __builtin_amdgcn_perm(cur[r][q], base[r], 0x0c020000u | ((4u + c) << 8));
+                    w[r][c] = *reinterpret_cast<const uint4_t *>(tbl + addr);
+                }
 #pragma unroll
             for (int c = 0; c < 4; c++)
 #pragma unroll
-                for (int r = 0; r < kGemvRows; r++) {
-                    const uint32_t code = (cur[r][q] >> (8 * c)) & 0xffu;
-                    const uint4_t w = table[code * kCopies + copy];
+                for (int r = 0; r < R; r++)
 #pragma unroll
                     for (int d = 0; d < 4; d++) {
-                        const uint32_t wd = w[d], xd = xr[q][c][d];
+                        const uint32_t wd = w[r][c][d], xd = xr[q][c][d];
                         acc[r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[r], false);
                     }
-                }
-        const int row0 = b * kGemvTile + wave * kGemvRows;
-        gemv_out_t out;
-#pragma unroll
-        for (int r = 0; r < kGemvRows; r++) {
-            float s = wave_sum(acc[r]);
-            if (bias) s += (float)bias[row0 + r];
-            out[r] = (half_t)s;
         }
-        if (lane == 0) *reinterpret_cast<gemv_out_t *>(y + row0) = out;
 #pragma unroll
-        for (int r = 0; r < kGemvRows; r++)
+        for (int r = 0; r < R; r++) {
+            const float s = wave_sum_to_uniform(acc[r]);
+            res = (int)lane == g * G + r ? s : res;
+        }
+    };
+    auto multiply_group = [&](int g, const uint32_t (&cur)[G][RUNS]) {
+        const int left = n_rows - g * G;  // wave-uniform
+        if (left >= G) multiply_rows(g, cur, std::integral_constant<int, G>{});
+        else if (G > 1 && left == 1) multiply_rows(g, cur, std::integral_constant<int, 1>{});
+        else if (G > 2 && left == 2) multiply_rows(g, cur, std::integral_constant<int, (G > 2 ? 2 : 1)>{});
+        else if (G > 3) multiply_rows(g, cur, std::integral_constant<int, (G > 3 ? 3 : 1)>{});
+    };
+    for (int g = 0; g < n_groups; g += NBUF) {
 #pragma unroll
-            for (int q = 0; q < RUNS; q++) cur[r][q] = nxt[r][q];
+        for (int u = 0; u < NBUF; u++) {
+            // (unconditional: see the header; the group requested past the end is the last one again)
+            load_group(min(g + u + NBUF - 1, n_groups - 1), cw[(u + NBUF - 1) % NBUF]);
+            if (g + u < n_groups) multiply_group(g + u, cw[u]);
+        }
+    }
+    if ((int)lane < n_rows) {
+        float s = res;
+        if (bias) s += (float)bias[row0 + lane];
+        y[row0 + lane] = (half_t)s;
     }
 }
 
 }  // namespace
 
-bool decode_gemv_stream_supports(const ProblemB &p)
+#ifndef VQ_GEMV_WIDE_G
+#define VQ_GEMV_WIDE_G 2
+#endif
+#ifndef VQ_GEMV_WIDE_NBUF
+#define VQ_GEMV_WIDE_NBUF 2
+#endif
+#ifndef VQ_GEMV_WIDE_G4
+#define VQ_GEMV_WIDE_G4 1
+#endif
+#ifndef VQ_GEMV_WIDE_NBUF4
+#define VQ_GEMV_WIDE_NBUF4 2
+#endif
+
+// One row of X, 8-vectors, 8-bit codes, K a multiple of 2048 up to 8192, and no workgroup's share of
+// the rows reaching into more than two codebooks.
+bool decode_gemv_wide_supports(const ProblemB &p)
 {
-    return decode_gemv_supports(p) && p.vec == 8 && p.code_bits == 8 && p.M == 1 && p.n_codebooks == 1;
+    if (p.M != 1 || p.vec != 8 || p.code_bits != 8 || p.entries > 256 || p.packed) return false;
+    if (p.K < kRunK || p.K % kRunK != 0 || p.K / kRunK > kGemvMaxRuns || p.N < 1) return false;
+    const int waves = device_cu_count() * kWideWaves;
+    const int rows_per_wave = (p.N + waves - 1) / waves;
+    if (rows_per_wave > 64) return false;  // one result per lane
+    return p.n_codebooks == 1 || (int64_t)kWideWaves * rows_per_wave <= p.rows_per_cb;
 }
 
-hipError_t launch_decode_gemv_stream(const ProblemB &p, hipStream_t s)
+hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
 {
-    if (!decode_gemv_stream_supports(p)) return hipErrorInvalidValue;
-    const int n_blocks = p.N / kGemvTile;
+    if (!decode_gemv_wide_supports(p)) return hipErrorInvalidValue;
     const int cus = device_cu_count();
-    // (four runs: x alone takes 64 registers, a unit holds one workgroup's waves, and a second one would only queue)
-    const int wgs = cus * (p.K / kRunK <= 3 ? VQ_GEMV_STREAM_WGS_PER_CU : 1);
-    const dim3 grid(n_blocks < wgs ? n_blocks : wgs), block(kGemvWaves * 64);
+    const int waves = cus * kWideWaves;
+    const dim3 grid(cus), block(kWideWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
-    auto launch = [&](auto kern) { hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, n_blocks, p.entries); };
+    // a second table only when some workgroup's rows cross a codebook boundary: then every workgroup fills two
+    const bool straddle = p.n_codebooks > 1 && !(p.N % waves == 0 && p.rows_per_cb % (kWideWaves * (p.N / waves)) == 0);
+    const int books = p.n_codebooks == 1 ? 0 : (straddle ? 2 : 1);
+    auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.entries, p.N / waves, p.N % waves,
+                           p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, p.N);
+        return hipGetLastError();
+    };
+    auto pick = [&](auto runs_c, auto g_c, auto nbuf_c) {
+        constexpr int R = decltype(runs_c)::value, GG = decltype(g_c)::value, NB = decltype(nbuf_c)::value;
+        return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, NB, 0>)
+             : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1>) : launch(decode_gemv_wide_kernel<R, GG, NB, 2>);
+    };
+    using std::integral_constant;
     switch (p.K / kRunK) {
-    case 1: launch(decode_gemv_stream_kernel<1>); break;
-    case 2: launch(decode_gemv_stream_kernel<2>); break;
-    case 3: launch(decode_gemv_stream_kernel<3>); break;
-    default: launch(decode_gemv_stream_kernel<4>); break;
+    case 1: return pick(integral_constant<int, 1>{}, integral_constant<int, VQ_GEMV_WIDE_G>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF>{});
+    case 2: return pick(integral_constant<int, 2>{}, integral_constant<int, VQ_GEMV_WIDE_G>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF>{});
+    case 3: return pick(integral_constant<int, 3>{}, integral_constant<int, VQ_GEMV_WIDE_G4>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF4>{});
+    default: return pick(integral_constant<int, 4>{}, integral_constant<int, VQ_GEMV_WIDE_G4>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF4>{});
     }
-    return hipGetLastError();
 }
 
-bool decode_gemv_supports(const ProblemB &p)
+bool decode_gemv_wide_preferred(const ProblemB &p);
+
+namespace {
+
+// the four-wave kernel (decode_gemv_kernel)
+bool decode_gemv_plain_supports(const ProblemB &p)
 {
     const bool u8 = p.code_bits == 8;
     // 8- and 4-vectors with either code width, 2-vectors with 8-bit codes (one load of at most 16 bytes per run)
@@ -317,10 +509,19 @@ bool decode_gemv_supports(const ProblemB &p)
            p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns && p.N % kGemvTile == 0 && p.rows_per_cb % kGemvTile == 0;
 }
 
-// From this many 16-row blocks per compute unit on, one row of X goes to the streaming kernel.
-#ifndef VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU
-#define VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU 4
+}  // namespace
+
+bool decode_gemv_supports(const ProblemB &p) { return decode_gemv_wide_preferred(p) || decode_gemv_plain_supports(p); }
+
+// From this many rows per wave of the wide form on (sixteen waves per compute unit), one row of X goes to it.
+#ifndef VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE
+#define VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE 1
 #endif
+
+bool decode_gemv_wide_preferred(const ProblemB &p)
+{
+    return decode_gemv_wide_supports(p) && p.N >= VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE * kWideWaves * device_cu_count();
+}
 
 namespace {
 
@@ -361,9 +562,8 @@ hipError_t launch_gemv_format(const ProblemB &p, hipStream_t s)
 
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
 {
-    if (!decode_gemv_supports(p)) return hipErrorInvalidValue;
-    if (decode_gemv_stream_supports(p) && p.N / kGemvTile >= VQ_GEMV_STREAM_MIN_BLOCKS_PER_CU * device_cu_count())
-        return launch_decode_gemv_stream(p, s);
+    if (decode_gemv_wide_preferred(p)) return launch_decode_gemv_wide(p, s);
+    if (!decode_gemv_plain_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
     case 8: return u8 ? launch_gemv_format<8, uint8_t>(p, s) : launch_gemv_format<8, uint16_t>(p, s);
