@@ -334,8 +334,12 @@ struct FusedACfg {
     static constexpr int kCodeRead1 = MPA == 8 ? 2 : 1;          // second code read (the first is at 0)
     static constexpr int kGather0 = MPA == 8 ? 9 : 3;            // eight gathers from here on
     static constexpr int kWrite0 = MPA == 8 ? 24 : 12;           // two writes
-    static constexpr int kXIssue0 = MPA == 8 ? 1 : 13, kXIssueGap = MPA == 8 ? 5 : 2;   // global loads of X
-    static constexpr int kCodeIssue = MPA == 8 ? 21 : 14;        // the code tile load of even steps
+    static constexpr int kXIssue0 = MPA == 8 ? 1 : 13, kXIssueGap = MPA == 8 ? 5 : 1;   // global loads of X
+    // the code tile load of even steps: behind the step's last X load, as the counted waits of the main loop assume
+    // (with the code tile between two X loads, the wait of an odd step let the last X load of the next stage
+    // still be in flight)
+    static constexpr int kCodeIssue = MPA == 8 ? 21 : 15;
+    static_assert(kCodeIssue > kXIssue0 + (kXLoads - 1) * kXIssueGap && kCodeIssue < 4 * MPA, "code tile behind the X loads, inside the step");
     static_assert(kLdsBytes <= 160 * 1024, "the fused geometry-A kernel fits the LDS");
 };
 
