@@ -85,6 +85,25 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
                            void *workspace, void *stream);
 
 /*
+ * The fused VQ GEMM with a gated epilogue, for a gate/up projection pair (the MLP shapes among the measured
+ * configurations): the rows of W (as codes) are the gate rows and the up rows of the pair interleaved in groups of
+ * 16 - rows 32g .. 32g+15 are gate rows 16g .. 16g+15, rows 32g+16 .. 32g+31 the up rows of the same columns -
+ * and
+ *     y[m, 16g + r] = silu(P[m, 32g + r]) * P[m, 32g + 16 + r],   P = X . W^T (+ bias[n], indexed like the rows of W),
+ * silu(t) = t / (1 + exp(-t)), everything in fp32 with one rounding to fp16: y is [M, N/2] and the [M, N] product
+ * never exists in memory.  N % 32 == 0.  No counterpart in the reference (its storeC has no epilogue,
+ * strategy_2/bsz128/src.cu:163-177).  The prefill kernels (variants 3, 5, 6), the wide GEMV kernel (variant 8: one
+ * row of X) and the scalar kernel (variant 1) carry the epilogue; the K-sliced decode kernels do not:
+ * VQGEMM_VARIANT_TWOPASS here means the plain product into `workspace` ([M, N] fp16) followed by the element-wise
+ * pass, and VQGEMM_VARIANT_AUTO takes that route where the plain product would run a decode kernel and a
+ * workspace is given (NULL: the prefill kernels or the scalar kernel take the shape after all).
+ */
+int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebook, const void *bias, void *y,
+                            int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                            int32_t n_codebooks, int32_t code_bits, int32_t variant,
+                            void *workspace, void *stream);
+
+/*
  * Fused VQ GEMM, geometry A (reference-native tensors, same entry point of the reference:
  * bind.cpp:3,7; kernels strategy_2/bsz128/src.cu:213-253 and siblings, indexing per
  * strategy_2/bsz512/src.cu:163-176 and bench.py:46-56).  out is [M, 2*Nc].

@@ -170,6 +170,37 @@ def silu_mul(gate_up: np.ndarray) -> np.ndarray:
         return (g / (1.0 + np.exp(-g)) * u).astype(np.float16)
 
 
+def interleave_gate_up(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """The row order of a gate/up pair under the gated epilogue: rows 32g .. 32g+15 of the result are gate rows
+    16g .. 16g+15, rows 32g+16 .. 32g+31 the up rows of the same numbers (first axis; a multiple of 16 rows each).
+    Works on codes, weights or biases alike.  No counterpart in the reference."""
+    gate, up = np.asarray(gate), np.asarray(up)
+    if gate.shape != up.shape or gate.shape[0] % 16 != 0:
+        raise ValueError("gate and up must have the same shape and a multiple of 16 rows")
+    h = gate.shape[0]
+    rest = gate.shape[1:]
+    return np.stack([gate.reshape(h // 16, 16, *rest), up.reshape(h // 16, 16, *rest)], axis=1).reshape(2 * h, *rest)
+
+
+def gated_gemm_b(x, codes, codebook, bias=None) -> np.ndarray:
+    """y[m, 16g + r] = silu(P[m, 32g + r]) * P[m, 32g + 16 + r] with P = X . W^T (+ bias) in float64, W dequantised
+    from interleaved gate/up rows (see interleave_gate_up); one rounding to fp16.  The math behind
+    vqgemm_e2e_gemm_b_gated; no counterpart in the reference (its kernels store the plain product,
+    strategy_2/bsz128/src.cu:163-177).  Pinned in tests/test_oracle.py by a loop over the definition and by the
+    element-wise silu_mul on the de-interleaved product."""
+    w = dequant_b(codes, codebook).astype(np.float64)
+    if w.shape[0] % 32 != 0:
+        raise ValueError("the interleaved W needs a multiple of 32 rows")
+    p = np.asarray(x).astype(np.float64) @ w.T
+    if bias is not None:
+        p = p + np.asarray(bias).astype(np.float64)[None, :]
+    m, n = p.shape
+    pg = p.reshape(m, n // 32, 2, 16)
+    g, u = pg[:, :, 0, :].reshape(m, n // 2), pg[:, :, 1, :].reshape(m, n // 2)
+    with np.errstate(over="ignore"):
+        return (g / (1.0 + np.exp(-g)) * u).astype(np.float16)
+
+
 def pack_lane_bytes(vec: int, code_bytes: int) -> int:
     """Bytes of codes one lane of the decode kernel loads at a time: 16, or 8 where four lanes'
     16 bytes would cover more than the 256 k a wave owns (8-vectors with 8-bit codes)."""

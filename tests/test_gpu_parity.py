@@ -1217,3 +1217,106 @@ def test_ctypes_wrappers_check_dtypes_and_shapes_before_the_gpu_sees_them():
         cabi.e2e_gemm_a(xa, wa, cba[:3].contiguous())
     with pytest.raises(ValueError):
         cabi.e2e_gemm_a(xa, wa[:32].contiguous(), cba)
+
+
+# ------------------------------------------------------------------ the gated epilogue (gate/up pairs)
+GATED_B = [
+    # name, M, K, N (rows of the interleaved W), vec, E, bits, G
+    ("wide_tile", 300, 512, 1024, 8, 256, 8, 1),              # 256x256 tiles, ragged M
+    ("wide_tile_books_and_tail", 512, 1056, 768, 4, 4096, 16, 3),
+    ("narrow_tile", 1024, 256, 1152, 8, 256, 8, 9),
+    ("small_tile", 200, 256, 416, 8, 256, 8, 13),              # 128x128 tiles, 32-row codebooks, ragged N in tiles
+    ("small_tile_v2", 129, 256, 160, 2, 256, 8, 1),
+    ("gemv_wide", 1, 4096, 8192, 8, 256, 8, 1),                  # one row of X: one output per group of two code rows
+    ("gemv_wide_ragged_two_books", 1, 2048, 8192 + 64, 8, 200, 8, 2),
+    ("gemv_wide_many_books", 1, 4096, 16384, 8, 256, 8, 16),
+    ("decode_shape", 16, 1024, 2048, 4, 4096, 16, 1),           # the K-sliced kernels have no gated epilogue
+    ("decode_shape_m2", 2, 4096, 4096, 8, 256, 8, 1),
+    ("odd_k_scalar_only", 5, 72, 64, 8, 256, 8, 1),
+]
+
+
+@pytest.mark.parametrize("row", GATED_B, ids=[r[0] for r in GATED_B])
+def test_gated_epilogue_against_the_oracle(row):
+    name, M, K, N, v, E, bits, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1), codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=51, device=DEV)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(52)) * 0.5).half().to(DEV)
+    ws = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    want = vo.gated_gemm_b(_np(x), _np(codes), _np(cb)).astype(np.float64)
+    want_b = vo.gated_gemm_b(_np(x), _np(codes), _np(cb), _np(bias)).astype(np.float64)
+    ran = []
+    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
+                    cabi.VARIANT_PREFILL_SMALL, cabi.VARIANT_DECODE_GEMV, cabi.VARIANT_TWOPASS, cabi.VARIANT_DECODE):
+        for b, ref in ((None, want), (bias, want_b)):
+            _say("gated", name, cabi.VARIANT_NAMES[variant], "bias" if b is not None else "")
+            try:
+                y = cabi.e2e_gemm_b_gated(x, codes, cb, variant=variant, bias=b, workspace=ws)
+            except cabi.VqGemmError as e:
+                assert e.code == -4 and variant not in (cabi.VARIANT_AUTO, cabi.VARIANT_GENERIC, cabi.VARIANT_TWOPASS), e
+                continue
+            torch.cuda.synchronize()
+            assert y.shape == (M, N // 2)
+            # Bar: the error over the largest output within 2e-3 as for the GEMM itself; element by element (with the
+            # floor) twice that: an output is a product of two fp32 sums, each with the GEMM's own error, and where the
+            # gate is near zero its slope turns the sum's absolute error into a relative one of the (small) product.
+            # The two-pass route also rounds the product to fp16 before the gate.
+            e1, e2 = vo.rel_err(_np(y), ref)
+            _say(f"    rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+            assert e2 <= TOL and e1 <= 2 * TOL, (name, variant, e1, e2)
+            ran.append(variant)
+    assert cabi.VARIANT_DECODE not in ran and cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran
+    if name.startswith("gemv_wide"):
+        assert cabi.VARIANT_DECODE_GEMV in ran
+    if name.endswith("_tile") or "tile_" in name:
+        assert cabi.VARIANT_PREFILL in ran
+    # without a workspace the automatic choice still answers (prefill or scalar kernel), and answers the same twice
+    y0 = cabi.e2e_gemm_b_gated(x, codes, cb)
+    e1, e2 = vo.rel_err(_np(y0), want)
+    assert e2 <= TOL and e1 <= 2 * TOL and torch.equal(cabi.e2e_gemm_b_gated(x, codes, cb), y0)
+
+
+def test_gated_epilogue_equals_the_plain_product_followed_by_the_gate():
+    """The fused epilogue against this library's own plain product: gate and up sums are the same fp32 numbers, so
+    silu(gate) * up computed from the unfused product (rounded to fp16 in between) sits within an fp16 step."""
+    spec = ProblemSpec("pair", GEOM_B, 384, 1024, 2048, 8, 256, 4, 8, codebook_3d=True, codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=53, device=DEV)
+    fused = cabi.e2e_gemm_b_gated(x, codes, cb)
+    p = cabi.e2e_gemm_b(x, codes, cb).float().view(384, 2048 // 32, 2, 16)
+    g, u = p[:, :, 0, :].reshape(384, 1024), p[:, :, 1, :].reshape(384, 1024)
+    unfused = torch.nn.functional.silu(g) * u
+    scale = unfused.abs().max().item()
+    assert ((fused.float() - unfused).abs().max() / scale).item() <= TOL
+    # rejections: rows of W that are no whole pairs; a null output
+    with pytest.raises(ValueError):
+        cabi.e2e_gemm_b_gated(x, codes[:2048 - 16].contiguous(), cb[:1].contiguous())
+
+
+def test_gated_mlp_module_with_interleaved_rows():
+    from vq_gemm_amd.nn import VQGatedMLP, VQLinear
+    from vq_gemm_amd.quantize import interleave_gate_up
+    K, H = 512, 768
+    s_g = ProblemSpec("g", GEOM_B, 1, K, H, 8, 256, 1, 8, codebook_std=0.05)
+    s_d = ProblemSpec("d", GEOM_B, 1, H, K, 8, 256, 1, 8, codebook_std=0.05)
+    _, c_g, cb_gu = make_problem(s_g, seed=31, device=DEV)
+    _, c_u, _ = make_problem(s_g, seed=33, device=DEV)
+    _, c_d, cb_d = make_problem(s_d, seed=32, device=DEV)
+    codes = interleave_gate_up(c_g, c_u)
+    assert np.array_equal(_np(codes), vo.interleave_gate_up(_np(c_g), _np(c_u)))
+    mlp = VQGatedMLP(VQLinear(codes, cb_gu), VQLinear(c_d, cb_d), interleaved=True)
+    stacked = VQGatedMLP(VQLinear(torch.cat([c_g, c_u]), cb_gu), VQLinear(c_d, cb_d))
+    w_d = vo.dequant_b(_np(c_d), _np(cb_d)).astype(np.float64)
+    for M in (1, 3, 200):
+        x = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).half().to(DEV)
+        _say("gated mlp, interleaved", M)
+        y = mlp(x)
+        torch.cuda.synchronize()
+        h = vo.gated_gemm_b(_np(x), _np(codes), _np(cb_gu))
+        ref = h.astype(np.float64) @ w_d.T
+        e1, e2 = vo.rel_err(_np(y), ref)
+        _say(f"  M={M}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+        # (a chain with an fp16 tensor in the middle: held to the bound on the largest output, as the stacked module's test)
+        assert e2 <= TOL and e1 <= 0.25, (e1, e2)
+        # the stacked layout with the element-wise kernel computes the same layer
+        ys = stacked(x)
+        assert ((y.float() - ys.float()).abs().max() / ys.float().abs().max()).item() <= 2 * TOL

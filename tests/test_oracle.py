@@ -418,3 +418,37 @@ def test_pack_codes_rejects_shapes_the_kernel_does_not_take():
         vo.pack_codes_b(np.zeros((16, 31), np.uint8), 8)
     with pytest.raises(ValueError):
         vo.pack_codes_b(np.zeros((8, 32), np.uint8), 8)
+
+
+def test_gated_gemm_is_the_definition_and_agrees_with_the_element_wise_function():
+    import math
+    rng = np.random.default_rng(11)
+    M, K, H, v, E = 3, 16, 32, 4, 16
+    cg = rng.integers(0, E, (H, K // v)).astype(np.uint8)
+    cu = rng.integers(0, E, (H, K // v)).astype(np.uint8)
+    cb = (rng.standard_normal((E, v)) * 0.5).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    bg = rng.standard_normal(H).astype(np.float16)
+    bu = rng.standard_normal(H).astype(np.float16)
+    codes = vo.interleave_gate_up(cg, cu)
+    # the interleave, entry by entry
+    assert codes.shape == (2 * H, K // v)
+    for o in range(H):
+        assert np.array_equal(codes[32 * (o // 16) + o % 16], cg[o]) and np.array_equal(codes[32 * (o // 16) + 16 + o % 16], cu[o])
+    bias = vo.interleave_gate_up(bg, bu)
+    got = vo.gated_gemm_b(x, codes, cb, bias)
+    # the definition as loops over separate gate and up matrices
+    wg = vo.dequant_b(cg, cb).astype(np.float64)
+    wu = vo.dequant_b(cu, cb).astype(np.float64)
+    for m in range(M):
+        for o in range(H):
+            g = sum(float(x[m, k]) * wg[o, k] for k in range(K)) + float(bg[o])
+            u = sum(float(x[m, k]) * wu[o, k] for k in range(K)) + float(bu[o])
+            want = np.float16(g / (1.0 + math.exp(-g)) * u)
+            assert got[m, o] == want, (m, o, got[m, o], want)
+    # with factors that are exact in fp16, the element-wise function on the stacked product gives the same
+    xi = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    cbi = rng.integers(-2, 3, (E, v)).astype(np.float16)
+    pg = (xi.astype(np.float64) @ vo.dequant_b(cg, cbi).astype(np.float64).T).astype(np.float16)
+    pu = (xi.astype(np.float64) @ vo.dequant_b(cu, cbi).astype(np.float64).T).astype(np.float16)
+    assert np.array_equal(vo.gated_gemm_b(xi, codes, cbi), vo.silu_mul(np.concatenate([pg, pu], axis=1)))

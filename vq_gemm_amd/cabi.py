@@ -23,6 +23,7 @@ _I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
 _SIGNATURES = {
     "vqgemm_e2e_gemm_b": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_b_bias": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
+    "vqgemm_e2e_gemm_b_gated": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_a": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _P]),
     "vqgemm_e2e_gemm_a_noalloc": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P]),
     "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
@@ -182,6 +183,37 @@ def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=Non
                                           bits, variant, _ptr(workspace), _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_e2e_gemm_b")
+    return out
+
+
+def e2e_gemm_b_gated(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=None, bias=None):
+    """The fused GEMM with the gated epilogue: `codes` [N, K/vec] hold gate and up rows interleaved in groups of 16
+    (N % 32 == 0), the result is [M, N/2] = silu(gate product) * up product.  `workspace` ([M, N] fp16) lets the
+    shapes of the K-sliced decode kernels run as the plain product plus the element-wise pass."""
+    import torch
+    _require(x.dim() == 2 and codes.dim() == 2, "x must be [M, K] and codes [N, K/vec]")
+    G, E, v = _check_codebook(codebook)
+    bits = _code_bits(codes)
+    M, K = x.shape
+    N = codes.shape[0]
+    _check_f16(x, (M, K), "x")
+    _require(codes.shape[1] * v == K, f"codes have {codes.shape[1]} columns of {v}-vectors but x has K = {K}")
+    _require(N % 32 == 0, "the interleaved gate/up rows come in whole groups of 32")
+    _require(N % G == 0, "rows of codes must be a multiple of the number of codebooks")
+    _same_device(x, codes, codebook, out, workspace, bias)
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.float16, device=x.device)
+    else:
+        _check_f16(out, (M, N // 2), "out")
+    if variant == VARIANT_TWOPASS and workspace is None:
+        workspace = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    _check_workspace(workspace, M * N)
+    if bias is not None:
+        _check_f16(bias, (N,), "bias")
+    rc = lib().vqgemm_e2e_gemm_b_gated(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(bias), _ptr(out), M, K, N, v, E, G, bits,
+                                       variant, _ptr(workspace), _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_e2e_gemm_b_gated")
     return out
 
 

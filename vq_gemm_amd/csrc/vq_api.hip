@@ -82,6 +82,7 @@ ProblemB make_b(const void *x, const void *codes, const void *codebook, void *y,
     p.rows_per_cb = N > 0 ? (int)(N / n_codebooks) : 1;
     if (p.rows_per_cb < 1) p.rows_per_cb = 1;
     p.packed = false;
+    p.gated = false;
     return p;
 }
 
@@ -194,6 +195,83 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
         break;
     default:
         return VQGEMM_E_VARIANT;
+    }
+    return static_cast<int>(e);
+}
+
+int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebook, const void *bias, void *y, int64_t M,
+                            int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits,
+                            int32_t variant, void *workspace, void *stream)
+{
+    int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (N % 32 != 0) return VQGEMM_E_SHAPE;  // whole pairs of 16 gate rows and 16 up rows
+    if (M == 0 || N == 0) return VQGEMM_OK;
+    if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
+    const uintptr_t code_align = code_bits / 8;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(codebook, 2) || !aligned(codes, code_align) || !aligned(bias, 2) ||
+        !aligned(workspace, 2))
+        return VQGEMM_E_ALIGN;
+    const bool a16 = aligned(x, 16) && aligned(y, 16) && aligned(codebook, 16) && aligned(codes, 16) && aligned(bias, 8) &&
+                     aligned(workspace, 16);
+    ProblemB p = make_b(x, codes, codebook, y, M, K, N, vec, entries, n_codebooks, code_bits);
+    p.bias = static_cast<const half_t *>(bias);
+    p.gated = true;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // the plain product of the same shape, for the kernels without a gated epilogue (into the workspace)
+    ProblemB plain = p;
+    plain.gated = false;
+    plain.y = static_cast<half_t *>(workspace);
+    if (variant == VQGEMM_VARIANT_AUTO) {
+        if (K == 0 || !a16) variant = VQGEMM_VARIANT_GENERIC;
+        else if (decode_gemv_wide_preferred(p)) variant = VQGEMM_VARIANT_DECODE_GEMV;
+        else {
+            // What the plain product would run on decides: the prefill kernels carry the gated epilogue themselves;
+            // where a decode kernel would be chosen, the product goes to the workspace and the element-wise pass
+            // follows (two launches), or - without a workspace - the prefill kernels take it after all.
+            const int plain_variant = select_b(plain, true);
+            const bool decode_like = plain_variant == VQGEMM_VARIANT_DECODE || plain_variant == VQGEMM_VARIANT_DECODE_GEMV;
+            if (decode_like && workspace) variant = VQGEMM_VARIANT_TWOPASS;
+            else if (prefill_supports(plain)) variant = VQGEMM_VARIANT_PREFILL;
+            else variant = VQGEMM_VARIANT_GENERIC;
+        }
+    }
+    hipError_t e = hipSuccess;
+    switch (variant) {
+    case VQGEMM_VARIANT_GENERIC:
+        e = launch_generic_b(p, s);
+        break;
+    case VQGEMM_VARIANT_DECODE_GEMV:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !decode_gemv_wide_preferred(p)) return VQGEMM_E_VARIANT;
+        e = launch_decode_gemv(p, s);
+        break;
+    case VQGEMM_VARIANT_PREFILL:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !prefill_supports(plain)) return VQGEMM_E_VARIANT;
+        e = launch_prefill_b(p, s);
+        break;
+    case VQGEMM_VARIANT_PREFILL_NARROW:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !prefill_narrow_supports(plain)) return VQGEMM_E_VARIANT;
+        e = launch_prefill_b(p, s, 2);
+        break;
+    case VQGEMM_VARIANT_PREFILL_SMALL:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !prefill_small_supports(plain)) return VQGEMM_E_VARIANT;
+        e = launch_prefill_small_b(p, s);
+        break;
+    case VQGEMM_VARIANT_TWOPASS: {
+        // (here: the fused product as the automatic choice runs it, then the element-wise pass)
+        if (!workspace) return VQGEMM_E_NULL;
+        rc = vqgemm_e2e_gemm_b_bias(x, codes, codebook, bias, workspace, M, K, N, vec, entries, n_codebooks, code_bits,
+                                    VQGEMM_VARIANT_AUTO, nullptr, stream);
+        if (rc != VQGEMM_OK) return rc;
+        e = launch_silu_mul(static_cast<const half_t *>(workspace), p.y, M, N / 2, s, /*interleaved=*/true);
+        break;
+    }
+    default:
+        return VQGEMM_E_VARIANT;  // the K-sliced decode kernels have no gated epilogue
     }
     return static_cast<int>(e);
 }

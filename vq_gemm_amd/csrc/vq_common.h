@@ -28,7 +28,13 @@ struct ProblemB {
     int vec, entries, n_codebooks, code_bits;
     int rows_per_cb;      // N / G
     bool packed;          // codes are in the packed layout of the batched decode kernel (launch_pack_codes)
+    bool gated;           // gated epilogue: the rows of W are gate and up rows interleaved in groups of 16 (rows
+                          // 32g .. 32g+15 gate, 32g+16 .. 32g+31 up) and y is [M, N/2]:
+                          // y[m, 16g + r] = silu(P[m, 32g + r]) * P[m, 32g + 16 + r], P = X . W^T (+ bias) in fp32
 };
+
+// silu(g) = g / (1 + exp(-g)) in fp32, as every kernel with the gated epilogue and the element-wise kernel compute it
+__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
 
 struct ProblemA {
     const half_t *x;      // [M,K]
@@ -101,6 +107,9 @@ bool decode_gemv_preferred(const ProblemB &p);
 bool decode_general_supports(const ProblemB &p);
 hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);
 
+// whether some fused kernel takes the shape with p.gated set (the prefill kernels, the wide GEMV kernel, the scalar kernel)
+bool gated_supports(const ProblemB &p);
+
 bool prefill_supports(const ProblemB &p);
 // whether the 256x128 tile of the prefill kernel can serve the shape (a subset of prefill_supports)
 bool prefill_narrow_supports(const ProblemB &p);
@@ -130,7 +139,8 @@ bool fused_a_supports(const ProblemA &p);
 hipError_t launch_fused_a(const ProblemA &p, hipStream_t s);
 
 // out[M,N] = silu(a[:, :N]) * a[:, N:] for a [M, 2N]
-hipError_t launch_silu_mul(const half_t *a, half_t *out, int64_t M, int64_t N, hipStream_t s);
+// (interleaved: gate and up columns alternate in groups of 16 instead of lying in the two halves of a row)
+hipError_t launch_silu_mul(const half_t *a, half_t *out, int64_t M, int64_t N, hipStream_t s, bool interleaved = false);
 
 // out[0] = the largest code of codes[0 .. count) (0 when count == 0); out is device memory
 hipError_t launch_max_code(const void *codes, int64_t count, int code_bits, uint32_t *out, hipStream_t s);

@@ -845,7 +845,7 @@ bool decode_gemv_preferred(const ProblemB &p)
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
-    if (!decode_supports(p)) return hipErrorInvalidValue;
+    if (p.gated || !decode_supports(p)) return hipErrorInvalidValue;  // (the K-sliced kernels have no gated epilogue)
     const bool u8 = p.code_bits == 8;
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension

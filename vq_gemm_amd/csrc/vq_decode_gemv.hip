@@ -272,8 +272,12 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
                                                                            half_t *__restrict__ y,
                                                                            const half_t *__restrict__ bias, int entries,
                                                                            int rows_q, int rows_r, int rows_per_cb,
-                                                                           float rcp_rows_per_cb, int n_books, int n_total)
+                                                                           float rcp_rows_per_cb, int n_books, int n_total,
+                                                                           int gated)
 {
+    // gated: the epilogue of a gate/up pair.  The rows of W are gate and up rows interleaved in groups of 16; what
+    // is dealt out to the waves (rows_q, rows_r, n_total) are then the N/2 outputs, a wave's code rows are the gate
+    // and the up row of each of its outputs in turn, and a group of two rows is one output (G = 2).
     constexpr bool TWO = BOOKS == 2;
     constexpr int kXChunks = RUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
@@ -284,7 +288,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     // All kernel arguments are fetched at once: left to first use, each pointer costs the prologue a
     // scalar-load round trip of its own.
     asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(bias), "s"(entries), "s"(rows_q), "s"(rows_r), "s"(rows_per_cb),
-                 "s"(rcp_rows_per_cb), "s"(n_books), "s"(n_total));
+                 "s"(rcp_rows_per_cb), "s"(n_books), "s"(n_total), "s"(gated));
     const int tid = threadIdx.x;
     constexpr int J = RUNS * kRunCodes;  // codes (bytes) per row
 
@@ -293,14 +297,20 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     // These loads sit in wave-uniform branches; the code loads behind them are unconditional, so the wait
     // counts stay exact (the conditional loads are older than the code loads on every path).
     int book0 = 0, second_book_row = INT_MAX;  // the workgroup's first codebook; rows from second_book_row on read the second table
+    // row of W behind a gated output: its gate row (the up row lies 16 further on)
+    auto gate_row = [](int o) { return 32 * (o >> 4) + (o & 15); };
+    bool second_table = false;
     if constexpr (BOOKS > 0) {
-        const int wg_row0 = min((int)blockIdx.x * kWideWaves * rows_q + min((int)blockIdx.x * kWideWaves, rows_r), n_total - 1);
+        // the workgroup's first and last share (rows, or outputs when gated) and the rows of W they reach
+        const int wg_first = min((int)blockIdx.x * kWideWaves * rows_q + min((int)blockIdx.x * kWideWaves, rows_r), n_total - 1);
+        const int wg_last = min(((int)blockIdx.x + 1) * kWideWaves * rows_q + min(((int)blockIdx.x + 1) * kWideWaves, rows_r), n_total) - 1;
+        const int wg_row0 = gated ? gate_row(wg_first) : wg_first;
+        const int wg_row_last = gated ? gate_row(max(wg_last, wg_first)) + 16 : wg_last;
         book0 = small_quotient(wg_row0, rows_per_cb, rcp_rows_per_cb);
         if (TWO) second_book_row = (book0 + 1) * rows_per_cb;
+        // (only the workgroups whose rows cross into the next codebook fetch and fill the second table)
+        second_table = TWO && second_book_row <= wg_row_last;
     }
-    // (only the workgroups whose rows cross into the next codebook fetch and fill the second table)
-    const int wg_row1 = ((int)blockIdx.x + 1) * kWideWaves * rows_q + min(((int)blockIdx.x + 1) * kWideWaves, rows_r);
-    const bool second_table = TWO && second_book_row < wg_row1;
     constexpr int kDutyThreads = kWideWaves * 64 / 2;
     constexpr int kXPerThread = (kXChunks + kDutyThreads - 1) / kDutyThreads;
     const bool table_duty = tid < kDutyThreads;
@@ -318,21 +328,35 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         for (int i = 0; i < kXPerThread; i++) xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, kXChunks - 1)];
     }
 
-    // the wave's rows [row0, row0 + n_rows): at most 64, one result per lane
+    // the wave's share [row0, row0 + n_share) of the rows (gated: of the outputs) and its code rows: at most 64, one
+    // result per lane
     const uint32_t lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int gw = blockIdx.x * kWideWaves + wave;
-    const int row0 = gw * rows_q + min(gw, rows_r);
-    const int n_rows = rows_q + (gw < rows_r ? 1 : 0);
+    const int row0 = min(gw * rows_q + min(gw, rows_r), n_total - 1);  // (a wave without a share reads the last row)
+    const int n_share = rows_q + (gw < rows_r ? 1 : 0);
+    const int n_rows = gated ? 2 * n_share : n_share;
     const int n_groups = (n_rows + G - 1) / G;
-    const int last_row = min(row0 + max(n_rows, 1), n_total) - 1;  // (a wave without rows reads the last row)
+    // code row t of the wave (clamped: loads past the end read the last row again)
+    auto code_row = [&](int t) {
+        t = min(t, max(n_rows, 1) - 1);
+        return gated ? gate_row(row0 + (t >> 1)) + 16 * (t & 1) : row0 + t;
+    };
+    // gated with a bias: lane i keeps the bias of its i-th output's gate and up row (loaded ahead of the codes, so
+    // that the loop stays free of loads other than the codes)
+    float bias_gate = 0.f, bias_up = 0.f;
+    if (gated && bias) {
+        const int o = row0 + min((int)lane, max(n_share, 1) - 1);
+        bias_gate = (float)bias[gate_row(o)];
+        bias_up = (float)bias[gate_row(o) + 16];
+    }
 
     uint32_t cw[NBUF][G][RUNS];
     auto load_group = [&](int g, uint32_t (&dst)[G][RUNS]) {
 #pragma unroll
         for (int r = 0; r < G; r++) {
             // (a wave-uniform row pointer and the lane as a 32-bit index: one scalar base per row, no vector address arithmetic)
-            const uint32_t *row = reinterpret_cast<const uint32_t *>(codes + (int64_t)min(row0 + g * G + r, last_row) * J);
+            const uint32_t *row = reinterpret_cast<const uint32_t *>(codes + (int64_t)code_row(g * G + r) * J);
 #pragma unroll
             for (int q = 0; q < RUNS; q++)
                 // (a relaxed atomic load of wavefront scope is an ordinary load instruction that the compiler
@@ -384,7 +408,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
         for (int r = 0; r < R; r++) {
             acc[r] = 0.f;
-            base[r] = TWO ? copy_base | (row0 + g * G + r >= second_book_row ? 0x10000u : 0u) : copy_base;
+            base[r] = TWO ? copy_base | (code_row(g * G + r) >= second_book_row ? 0x10000u : 0u) : copy_base;
         }
 #pragma unroll
         for (int q = 0; q < RUNS; q++) {
@@ -408,6 +432,13 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
                         acc[r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[r], false);
                     }
         }
+        if (G == 2 && R == 2 && gated) {
+            // one output: gate and up sums, the bias of the output's lane, silu(gate) * up
+            const float sg = wave_sum_to_uniform(acc[0]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), g));
+            const float su = wave_sum_to_uniform(acc[R - 1]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), g));
+            res = (int)lane == g ? silu_f32(sg) * su : res;
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const float s = wave_sum_to_uniform(acc[r]);
@@ -429,9 +460,9 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
             if (g + u < n_groups) multiply_group(g + u, cw[u]);
         }
     }
-    if ((int)lane < n_rows) {
+    if ((int)lane < n_share) {
         float s = res;
-        if (bias) s += (float)bias[row0 + lane];
+        if (bias && !gated) s += (float)bias[row0 + lane];
         y[row0 + lane] = (half_t)s;
     }
 }
@@ -458,6 +489,14 @@ bool decode_gemv_wide_supports(const ProblemB &p)
     if (p.M != 1 || p.vec != 8 || p.code_bits != 8 || p.entries > 256 || p.packed) return false;
     if (p.K < kRunK || p.K % kRunK != 0 || p.K / kRunK > kGemvMaxRuns || p.N < 1) return false;
     const int waves = device_cu_count() * kWideWaves;
+    if (p.gated) {
+        // two code rows per output, one output per group of two rows: K up to 4096 (the instantiations with G = 2)
+        if (p.N % 32 != 0 || p.K / kRunK > 2 || VQ_GEMV_WIDE_G != 2) return false;
+        const int outs_per_wave = (p.N / 2 + waves - 1) / waves;
+        if (outs_per_wave > 32) return false;
+        // a workgroup's rows of W: its outputs' gate and up rows, in whole groups of 32
+        return p.n_codebooks == 1 || (int64_t)2 * kWideWaves * outs_per_wave + 32 <= p.rows_per_cb;
+    }
     const int rows_per_wave = (p.N + waves - 1) / waves;
     if (rows_per_wave > 64) return false;  // one result per lane
     return p.n_codebooks == 1 || (int64_t)kWideWaves * rows_per_wave <= p.rows_per_cb;
@@ -470,12 +509,13 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
     const int waves = cus * kWideWaves;
     const dim3 grid(cus), block(kWideWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
-    // a second table only when some workgroup's rows cross a codebook boundary: then every workgroup fills two
-    const bool straddle = p.n_codebooks > 1 && !(p.N % waves == 0 && p.rows_per_cb % (kWideWaves * (p.N / waves)) == 0);
+    // a second table only when some workgroup's rows cross a codebook boundary: then every workgroup has room for two
+    const bool straddle = p.n_codebooks > 1 && (p.gated || !(p.N % waves == 0 && p.rows_per_cb % (kWideWaves * (p.N / waves)) == 0));
     const int books = p.n_codebooks == 1 ? 0 : (straddle ? 2 : 1);
+    const int n_dealt = p.gated ? p.N / 2 : p.N;  // what is dealt out to the waves: rows of W, or outputs
     auto launch = [&](auto kern) {
-        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.entries, p.N / waves, p.N % waves,
-                           p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, p.N);
+        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.entries, n_dealt / waves, n_dealt % waves,
+                           p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, n_dealt, p.gated ? 1 : 0);
         return hipGetLastError();
     };
     auto pick = [&](auto runs_c, auto g_c, auto nbuf_c) {
@@ -520,7 +560,7 @@ bool decode_gemv_supports(const ProblemB &p) { return decode_gemv_wide_preferred
 
 bool decode_gemv_wide_preferred(const ProblemB &p)
 {
-    return decode_gemv_wide_supports(p) && p.N >= VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE * kWideWaves * device_cu_count();
+    return decode_gemv_wide_supports(p) && (p.gated ? p.N / 2 : p.N) >= VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE * kWideWaves * device_cu_count();
 }
 
 namespace {
@@ -563,7 +603,7 @@ hipError_t launch_gemv_format(const ProblemB &p, hipStream_t s)
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
 {
     if (decode_gemv_wide_preferred(p)) return launch_decode_gemv_wide(p, s);
-    if (!decode_gemv_plain_supports(p)) return hipErrorInvalidValue;
+    if (p.gated || !decode_gemv_plain_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
     case 8: return u8 ? launch_gemv_format<8, uint8_t>(p, s) : launch_gemv_format<8, uint16_t>(p, s);

@@ -34,9 +34,56 @@ __global__ __launch_bounds__(256) void generic_b_kernel(const half_t *__restrict
     }
 }
 
+// Gated epilogue: one thread per output column computes the gate and the up product (rows 32g + r and
+// 32g + 16 + r of the interleaved W for output column 16g + r).
+template <typename CodeT>
+__global__ __launch_bounds__(256) void generic_b_gated_kernel(const half_t *__restrict__ x,
+                                                              const CodeT *__restrict__ codes,
+                                                              const half_t *__restrict__ cb,
+                                                              half_t *__restrict__ y,
+                                                              const half_t *__restrict__ bias, int M, int K, int N,
+                                                              int vec, int entries, int rows_per_cb)
+{
+    const int o = blockIdx.x * blockDim.x + threadIdx.x;
+    if (o >= N / 2) return;
+    const int J = K / vec;
+    const int ng = 32 * (o >> 4) + (o & 15), nu = ng + 16;
+    const half_t *book_g = cb + (int64_t)(ng / rows_per_cb) * entries * vec;
+    const half_t *book_u = cb + (int64_t)(nu / rows_per_cb) * entries * vec;
+    const CodeT *crow_g = codes + (int64_t)ng * J, *crow_u = codes + (int64_t)nu * J;
+    const float bg = bias ? (float)bias[ng] : 0.0f, bu = bias ? (float)bias[nu] : 0.0f;
+    for (int m = blockIdx.y * blockDim.y + threadIdx.y; m < M; m += gridDim.y * blockDim.y) {
+        const half_t *xrow = x + (int64_t)m * K;
+        float ag = 0.0f, au = 0.0f;
+        for (int j = 0; j < J; j++) {
+            uint32_t cg = crow_g[j], cu = crow_u[j];
+            cg = cg < (uint32_t)entries ? cg : (uint32_t)entries - 1;  // memory safety only
+            cu = cu < (uint32_t)entries ? cu : (uint32_t)entries - 1;
+            const half_t *wg = book_g + (int64_t)cg * vec, *wu = book_u + (int64_t)cu * vec;
+            for (int t = 0; t < vec; t++) {
+                const float xv = (float)xrow[j * vec + t];
+                ag += xv * (float)wg[t];
+                au += xv * (float)wu[t];
+            }
+        }
+        y[(int64_t)m * (N / 2) + o] = (half_t)(silu_f32(ag + bg) * (au + bu));
+    }
+}
+
 hipError_t launch_generic_b(const ProblemB &p, hipStream_t s)
 {
     if (p.M == 0 || p.N == 0) return hipSuccess;
+    if (p.gated) {
+        dim3 block(64, 4);
+        dim3 grid((p.N / 2 + 63) / 64, (unsigned)(((p.M + 3) / 4) < 32768 ? (p.M + 3) / 4 : 32768));
+        if (p.code_bits == 8)
+            hipLaunchKernelGGL((generic_b_gated_kernel<uint8_t>), grid, block, 0, s, p.x, static_cast<const uint8_t *>(p.codes),
+                               p.cb, p.y, p.bias, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
+        else
+            hipLaunchKernelGGL((generic_b_gated_kernel<uint16_t>), grid, block, 0, s, p.x, static_cast<const uint16_t *>(p.codes),
+                               p.cb, p.y, p.bias, p.M, p.K, p.N, p.vec, p.entries, p.rows_per_cb);
+        return hipGetLastError();
+    }
     dim3 block(64, 4);
     dim3 grid((p.N + 63) / 64, (unsigned)(((p.M + 3) / 4) < 32768 ? (p.M + 3) / 4 : 32768));
     if (p.code_bits == 8)

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
                                                               half_t *__restrict__ y,
                                                               const half_t *__restrict__ bias, int M, int K, int N,
                                                               int n_begin, int ldn, int entries, int rows_per_cb,
-                                                              int tiles_m, int tiles_n, int cb_lds_count)
+                                                              int tiles_m, int tiles_n, int cb_lds_count, int gated)
 {
     // The launch covers the W rows (columns of Y) [n_begin, N) of a problem with ldn rows in all:
     // ldn is the row stride of Y and counts the codebooks, N bounds the rows that are touched.
@@ -481,6 +481,12 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
             }
         }
     };
+    if (gated) {
+        // gate and up rows of W interleaved in groups of 16: a lane holds both factors of its outputs
+        if (bias) store_gated<NP, MP, true>(acc, y, bias, M, N, ldn, m0 + wm * WM, n0 + wn * WN, r16, kg);
+        else store_gated<NP, MP, false>(acc, y, bias, M, N, ldn, m0 + wm * WM, n0 + wn * WN, r16, kg);
+        return;
+    }
     if (bias) epilogue(std::true_type{});
     else epilogue(std::false_type{});
 }
@@ -506,7 +512,7 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
                                                                      const half_t *__restrict__ bias, int M, int K,
                                                                      int N, int n_begin, int ldn, int entries,
                                                                      int rows_per_cb, int tiles_m, int tiles_n,
-                                                                     int cb_lds_count)
+                                                                     int cb_lds_count, int gated)
 {
     typedef PrefillCfg<VEC, CodeT> C;
     constexpr int NS = 4, D = NS - 1;
@@ -790,6 +796,11 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_narrow_kernel(const half_
             }
         }
     };
+    if (gated) {
+        if (bias) store_gated<NPN, MP, true>(acc, y, bias, M, N, ldn, m0 + wm * WM, n0 + wn * WNN, r16, kg);
+        else store_gated<NPN, MP, false>(acc, y, bias, M, N, ldn, m0 + wm * WM, n0 + wn * WNN, r16, kg);
+        return;
+    }
     if (bias) epilogue(std::true_type{});
     else epilogue(std::false_type{});
 }
@@ -885,7 +896,7 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
                            static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, n_split, 0, p.N, p.entries,
-                           p.rows_per_cb, tiles_m, tiles_n, n_cb);
+                           p.rows_per_cb, tiles_m, tiles_n, n_cb, p.gated ? 1 : 0);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -901,7 +912,7 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
                            static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, n_split, p.N, p.entries,
-                           p.rows_per_cb, tiles_m, tiles_n, codebooks_per_tile(p, BNN));
+                           p.rows_per_cb, tiles_m, tiles_n, codebooks_per_tile(p, BNN), p.gated ? 1 : 0);
         return hipGetLastError();
     }
     return hipSuccess;

@@ -51,6 +51,45 @@ __device__ __forceinline__ half4_t round4(const float4_t &a, const float (&b)[4]
         return half4_t{(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]};
 }
 
+// The gated epilogue of a wave tile of MPC x NPC pieces: pieces 2q and 2q+1 along N are the gate and the up
+// rows of output piece q (the rows of W are interleaved in groups of 16), so a lane holds both factors of its
+// four outputs: out = silu(gate + bias) * (up + bias) in fp32, rounded once.  The lane holds rows
+// i*16 + r16 and columns 4*kg .. 4*kg+3 of every piece; m_wave / n_wave are the tile's first row of Y and
+// first (interleaved) row of W.  The rows of W are a multiple of 32 (pairs are whole), so the 8-byte stores are aligned.
+template <int NPC, int MPC, bool HAS_BIAS>
+__device__ __forceinline__ void store_gated(const float4_t (&acc)[NPC][MPC], half_t *__restrict__ y,
+                                            const half_t *__restrict__ bias, int M, int n_limit, int n_rows_w,
+                                            int m_wave, int n_wave, int r16, int kg)
+{
+    // n_rows_w: rows of the whole W (y has half as many columns); n_limit: the launch's last row of W + 1
+    static_assert(NPC % 2 == 0, "whole pairs of pieces");
+    const int ldy = n_rows_w / 2;
+#pragma unroll
+    for (int i = 0; i < MPC; i++) {
+        const int m = m_wave + i * 16 + r16;
+        if (m >= M) continue;
+#pragma unroll
+        for (int q = 0; q < NPC / 2; q++) {
+            const int n = n_wave + 32 * q;  // the gate piece's first row of W
+            if (n >= n_limit) continue;
+            float4_t g = acc[2 * q][i], u = acc[2 * q + 1][i];
+            if constexpr (HAS_BIAS) {
+                const half4_t bg = *reinterpret_cast<const half4_t *>(bias + n + 4 * kg);
+                const half4_t bu = *reinterpret_cast<const half4_t *>(bias + n + 16 + 4 * kg);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    g[e] += (float)bg[e];
+                    u[e] += (float)bu[e];
+                }
+            }
+            half4_t h;
+#pragma unroll
+            for (int e = 0; e < 4; e++) h[e] = (half_t)(silu_f32(g[e]) * u[e]);
+            *reinterpret_cast<half4_t *>(y + (int64_t)m * ldy + n / 2 + 4 * kg) = h;
+        }
+    }
+}
+
 // floor(x / d) for 0 <= x and a quotient small enough that float rounding stays within one
 // (here: x < d + 256); `rcp` = 1.0f / d.
 __device__ __forceinline__ int small_div(int x, int d, float rcp)

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                                                                     half_t *__restrict__ y,
                                                                     const half_t *__restrict__ bias, int M, int K,
                                                                     int N, int entries, int rows_per_cb, int tiles_m,
-                                                                    int tiles_n, int cb_lds_count)
+                                                                    int tiles_n, int cb_lds_count, int gated)
 {
     typedef PrefillCfg<VEC, CodeT> C;
     constexpr int D = NS - 1;                 // loads run D stages ahead
@@ -329,6 +329,12 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
             }
         }
     };
+    if (gated) {
+        // gate and up rows of W interleaved in groups of 16: a lane holds both factors of its outputs
+        if (bias) store_gated<SNP, SMP, true>(acc, y, bias, M, N, N, m0 + wm * SWM, n0 + wn * SWN, r16, kg);
+        else store_gated<SNP, SMP, false>(acc, y, bias, M, N, N, m0 + wm * SWM, n0 + wn * SWN, r16, kg);
+        return;
+    }
     if (bias) epilogue(std::true_type{});
     else epilogue(std::false_type{});
 }
@@ -364,7 +370,7 @@ hipError_t launch_small_typed(const ProblemB &p, hipStream_t s)
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), smem, s, p.x,
                        static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
-                       tiles_m, tiles_n, codebooks_per_tile(p, SBN));
+                       tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0);
     return hipGetLastError();
 }
 

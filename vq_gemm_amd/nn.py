@@ -12,7 +12,7 @@ import torch
 
 from . import cabi
 from .quantize import kmeans_quantize, residual_quantize
-from .torch_ops import silu_mul, vq_linear, vq_linear_packed
+from .torch_ops import silu_mul, vq_gated_linear, vq_linear, vq_linear_packed
 
 
 class VQLinear(torch.nn.Module):
@@ -108,17 +108,37 @@ class VQLinear(torch.nn.Module):
 class VQGatedMLP(torch.nn.Module):
     """down(silu(x @ Wg.T) * (x @ Wu.T)) with all three weights vector-quantised.
 
-    `gate_up` holds the gate rows of W stacked on the up rows ([2*H, K] as codes): one fused VQ GEMM
-    gives both products, an element-wise kernel applies silu(gate) * up, `down` ([K_out, H]) follows.
+    `gate_up` holds the gate rows and the up rows of the pair as one [2*H, K] weight.  With `interleaved=True`
+    (what `from_float` builds) they alternate in groups of 16 rows (`vq_gemm_amd.quantize.interleave_gate_up`) and one
+    fused VQ GEMM with the gated epilogue gives silu(gate) * up directly: the [M, 2*H] product never exists in
+    memory.  With `interleaved=False` the gate rows are stacked on the up rows: the plain fused GEMM writes both
+    products and an element-wise kernel follows.  `down` ([K_out, H]) is an ordinary `VQLinear`.
     """
 
-    def __init__(self, gate_up: VQLinear, down: VQLinear):
+    def __init__(self, gate_up: VQLinear, down: VQLinear, interleaved: bool = False):
         super().__init__()
         if gate_up.out_features % 2 != 0 or gate_up.out_features // 2 != down.in_features:
             raise ValueError("gate_up must have twice as many output features as down has input features")
+        if interleaved and (gate_up.out_features % 32 != 0 or gate_up.k_repeat != 1):
+            raise ValueError("the interleaved layout needs a multiple of 32 gate_up rows and a single quantisation stage")
         self.gate_up = gate_up
         self.down = down
+        self.interleaved = interleaved
+
+    @classmethod
+    def from_float(cls, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, vec: int = 8, entries: int = 256,
+                   n_codebooks: int = 1, iters: int = 10, seed: int = 0) -> "VQGatedMLP":
+        """Quantise fp16 weights gate [H, K], up [H, K], down [K_out, H]; the pair is interleaved for the gated epilogue."""
+        from .quantize import interleave_gate_up
+        gu = VQLinear.from_float(interleave_gate_up(gate.to(torch.float16), up.to(torch.float16)), vec, entries, n_codebooks,
+                                 None, iters, seed)
+        return cls(gu, VQLinear.from_float(down, vec, entries, n_codebooks, None, iters, seed + 1), interleaved=True)
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.interleaved:
+            gu = self.gate_up
+            if x.dtype != torch.float16 or x.shape[-1] != gu.in_features:
+                raise ValueError(f"expected an fp16 input with {gu.in_features} features")
+            return self.down(vq_gated_linear(x, gu.codes, gu.codebook, gu.bias))
         return self.down(silu_mul(self.gate_up(x)))

@@ -100,3 +100,15 @@ def residual_quantize(w, vec: int, entries: int, stages: int = 2, n_codebooks: i
     # (not every build converts to uint16 directly: narrow to int16, same bits)
     merged = merged.to(torch.int16).view(torch.uint16) if wide else merged.to(torch.uint8)
     return merged.contiguous(), torch.cat(all_books, dim=1).contiguous(), history
+
+
+def interleave_gate_up(gate, up):
+    """Rows of a gate/up projection pair in the order the gated epilogue expects (`vqgemm_e2e_gemm_b_gated`):
+    rows 32g .. 32g+15 of the result are gate rows 16g .. 16g+15, rows 32g+16 .. 32g+31 the up rows of the same
+    numbers.  Works on weights (before quantising), on codes, and on biases; both need a multiple of 16 rows."""
+    import torch
+    if gate.shape != up.shape or gate.shape[0] % 16 != 0:
+        raise ValueError("gate and up must have the same shape and a multiple of 16 rows")
+    h = gate.shape[0]
+    rest = gate.shape[1:]
+    return torch.stack([gate.reshape(h // 16, 16, *rest), up.reshape(h // 16, 16, *rest)], dim=1).reshape(2 * h, *rest).contiguous()
