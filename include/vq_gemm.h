@@ -228,6 +228,23 @@ int vqgemm_gemm_f16(const void *x, const void *w, void *y, int64_t M, int64_t K,
 int vqgemm_select_variant_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
                             int32_t n_codebooks, int32_t code_bits);
 
+/*
+ * The constants of the cost models behind VQGEMM_VARIANT_AUTO (host only).  The compiled-in values were fitted
+ * to measurements on one 256-CU MI355X; `python -m vq_gemm_amd.tune --fit` measures the box at hand and writes
+ * a flat JSON object {"name": number, ...} that vqgemm_tuning_load reads (and that the library reads by itself,
+ * once, from the file named by the environment variable VQGEMM_TUNING_FILE).  Names: vqgemm_tuning_name(i) for
+ * 0 <= i < vqgemm_tuning_count(): per-tile and per-stage microseconds of the prefill tiles, per-tile
+ * microseconds of the batched decode kernel, the limits between the GEMV kernels.  set/get return
+ * VQGEMM_E_VARIANT for an unknown name; load returns the number of constants it set, or VQGEMM_E_NULL when the
+ * file cannot be read.  No counterpart in the reference, whose tiling is compile-time macros
+ * (strategy_1/src.cu:12-47).  Set them before launching from other threads.
+ */
+int vqgemm_tuning_count(void);
+const char *vqgemm_tuning_name(int index);
+int vqgemm_tuning_get(const char *name, double *value);
+int vqgemm_tuning_set(const char *name, double value);
+int vqgemm_tuning_load(const char *path);
+
 /* Host string for a return code of this library (static storage). */
 const char *vqgemm_error_string(int code);
 

@@ -872,6 +872,25 @@ def test_tune_reports_every_variant_and_the_automatic_choice():
     assert r["auto_over_fastest"] > 0
 
 
+def test_tune_fit_measures_plausible_constants_and_the_library_takes_them():
+    from vq_gemm_amd import tune
+    before = cabi.tuning()
+    fitted = tune.fit(verbose=False)
+    assert set(fitted) == set(before)
+    # plausible for any MI355X: microseconds per stage and per tile, neither zero nor wild
+    assert 0.2 <= fitted["prefill_stage_us_256x256"] <= 4.0 and 0.1 <= fitted["prefill_stage_us_256x128"] <= 3.0
+    assert 0.1 <= fitted["prefill_small_stage_us_idle"] <= fitted["prefill_small_stage_us_busy"] <= 3.0
+    assert 0.1 <= fitted["decode_tile_us"] <= 5.0
+    try:
+        cabi.set_tuning(**fitted)
+        assert cabi.tuning()["decode_tile_us"] == fitted["decode_tile_us"]
+        # the measured configurations keep their kernels under the refitted constants
+        assert cabi.select_variant_b(4096, 4096, 4096, 8, 256, 32, 8) == cabi.VARIANT_PREFILL
+        assert cabi.select_variant_b(16, 4096, 11008, 4, 4096, 1, 16) == cabi.VARIANT_DECODE
+    finally:
+        cabi.set_tuning(**before)
+
+
 # shapes the tiled kernel takes (K a multiple of 64, N of 8): few tiles -> 128x128
 # tiles (the first three and the fifth), about one 256x128 tile per compute unit -> those (the seventh and eighth),
 # more -> 256x256 tiles (the fourth and the sixth); ragged M and N

@@ -142,3 +142,27 @@ def test_ctypes_wrappers_refuse_host_tensors():
         cabi.e2e_gemm_b(x, codes, cb)
     with pytest.raises(ValueError):
         cabi.dequant_b(codes, cb)
+
+
+def test_tuning_constants_can_be_read_set_and_loaded_from_a_file(tmp_path):
+    import json
+    from vq_gemm_amd import cabi
+    before = cabi.tuning()
+    assert {"prefill_stage_us_256x256", "decode_tile_us", "gemv_max_tiles_per_cu", "gemv_wide_min_rows_per_wave"} <= set(before)
+    try:
+        # the choice between the four-wave GEMV kernel and the K-sliced kernel follows the constant
+        dims = (1, 4096, 16 * 256 * 2, 4, 256, 1, 8)   # one row of X, 4-vectors: two tiles per unit on a 256-CU device
+        cabi.set_tuning(gemv_max_tiles_per_cu=4)
+        assert cabi.select_variant_b(*dims) == cabi.VARIANT_DECODE_GEMV
+        cabi.set_tuning(gemv_max_tiles_per_cu=1)
+        assert cabi.select_variant_b(*dims) == cabi.VARIANT_DECODE
+        path = tmp_path / "t.json"
+        path.write_text(json.dumps({"device": "some name: 3", "gemv_max_tiles_per_cu": 8, "decode_tile_us": 0.5, "not_a_constant": 1}))
+        assert cabi.lib().vqgemm_tuning_load(str(path).encode()) == 2
+        assert cabi.tuning()["decode_tile_us"] == 0.5 and cabi.select_variant_b(*dims) == cabi.VARIANT_DECODE_GEMV
+        assert cabi.lib().vqgemm_tuning_load(b"/nonexistent/file.json") == -1
+        assert cabi.lib().vqgemm_tuning_set(b"no_such_constant", 1.0) == -4
+        assert cabi.lib().vqgemm_tuning_set(b"decode_tile_us", -1.0) == -2
+    finally:
+        cabi.set_tuning(**before)
+    assert cabi.tuning() == before

@@ -36,6 +36,11 @@ _SIGNATURES = {
     "vqgemm_max_code": (ctypes.c_int, [_P, _I64, _I32, _P, _P]),
     "vqgemm_select_variant_b": (ctypes.c_int, [_I64, _I64, _I64, _I32, _I32, _I32, _I32]),
     "vqgemm_select_variant_a": (ctypes.c_int, [_I64, _I64, _I64, _I32]),
+    "vqgemm_tuning_count": (ctypes.c_int, []),
+    "vqgemm_tuning_name": (ctypes.c_char_p, [ctypes.c_int]),
+    "vqgemm_tuning_get": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double)]),
+    "vqgemm_tuning_set": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_double]),
+    "vqgemm_tuning_load": (ctypes.c_int, [ctypes.c_char_p]),
     "vqgemm_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "vqgemm_version": (ctypes.c_int, []),
 }
@@ -70,11 +75,36 @@ def _load(name, sigs):
     return lib
 
 
+TUNING_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning.json")
+
+
 def lib():
+    """The C-ABI library.  When `vq_gemm_amd/tuning.json` exists (written by `python -m vq_gemm_amd.tune --fit`) and
+    VQGEMM_TUNING_FILE is not set, the library is pointed at it before its first use."""
     global _lib
     if _lib is None:
+        if "VQGEMM_TUNING_FILE" not in os.environ and os.path.exists(TUNING_FILE):
+            os.environ["VQGEMM_TUNING_FILE"] = TUNING_FILE
         _lib = _load("libvqgemm.so", _SIGNATURES)
     return _lib
+
+
+def tuning() -> dict:
+    """The cost-model constants the automatic kernel choice currently uses."""
+    out = {}
+    v = ctypes.c_double(0)
+    for i in range(lib().vqgemm_tuning_count()):
+        name = lib().vqgemm_tuning_name(i)
+        if lib().vqgemm_tuning_get(name, ctypes.byref(v)) == 0:
+            out[name.decode()] = v.value
+    return out
+
+
+def set_tuning(**constants) -> None:
+    for name, value in constants.items():
+        rc = lib().vqgemm_tuning_set(name.encode(), float(value))
+        if rc != 0:
+            raise VqGemmError(rc, f"vqgemm_tuning_set({name})")
 
 
 def ref_lib():

@@ -4,9 +4,13 @@
 #include "vq_common.h"
 
 #include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <limits.h>
 #include <map>
 #include <mutex>
+#include <string>
 #include <utility>
 
 namespace vq {
@@ -42,6 +46,77 @@ hipError_t ensure_dynamic_lds(const void *kernel, size_t bytes)
 }
 
 namespace {
+
+struct TuningEntry {
+    const char *name;
+    double Tuning::*field;
+};
+const TuningEntry kTuningEntries[] = {
+    {"prefill_tile_fixed_us", &Tuning::prefill_tile_fixed_us},
+    {"prefill_stage_us_256x256", &Tuning::prefill_stage_us_256x256},
+    {"prefill_stage_us_256x128", &Tuning::prefill_stage_us_256x128},
+    {"prefill_full_device_factor", &Tuning::prefill_full_device_factor},
+    {"prefill_small_tile_fixed_us", &Tuning::prefill_small_tile_fixed_us},
+    {"prefill_small_stage_us_idle", &Tuning::prefill_small_stage_us_idle},
+    {"prefill_small_stage_us_busy", &Tuning::prefill_small_stage_us_busy},
+    {"decode_prologue_us", &Tuning::decode_prologue_us},
+    {"decode_prologue_shared_cu_us", &Tuning::decode_prologue_shared_cu_us},
+    {"decode_tile_us", &Tuning::decode_tile_us},
+    {"decode_tile_chunked_us", &Tuning::decode_tile_chunked_us},
+    {"decode_pass_change_us", &Tuning::decode_pass_change_us},
+    {"gemv_max_tiles_per_cu", &Tuning::gemv_max_tiles_per_cu},
+    {"gemv_max_k", &Tuning::gemv_max_k},
+    {"gemv_wide_min_rows_per_wave", &Tuning::gemv_wide_min_rows_per_wave},
+};
+constexpr int kTuningCount = (int)(sizeof(kTuningEntries) / sizeof(kTuningEntries[0]));
+
+std::mutex g_tuning_mu;
+Tuning g_tuning;             // written under the mutex; read without it (plain doubles, set before the launches that use them)
+bool g_tuning_file_read = false;
+
+const TuningEntry *find_tuning(const char *name)
+{
+    if (!name) return nullptr;
+    for (const TuningEntry &e : kTuningEntries)
+        if (std::strcmp(e.name, name) == 0) return &e;
+    return nullptr;
+}
+
+// A flat JSON object of numbers, {"name": value, ...}: names this library does not know are skipped, and so
+// is everything that is no number (a "device" string, for instance).  Returns how many constants were set.
+int read_tuning_file(const char *path)
+{
+    FILE *f = std::fopen(path, "rb");
+    if (!f) return -1;
+    std::string text;
+    char buf[4096];
+    size_t n;
+    while ((n = std::fread(buf, 1, sizeof(buf), f)) > 0) text.append(buf, n);
+    std::fclose(f);
+    int set = 0;
+    size_t pos = 0;
+    while ((pos = text.find('"', pos)) != std::string::npos) {
+        const size_t end = text.find('"', pos + 1);
+        if (end == std::string::npos) break;
+        const std::string key = text.substr(pos + 1, end - pos - 1);
+        size_t q = end + 1;
+        while (q < text.size() && (text[q] == ' ' || text[q] == '\t' || text[q] == '\n' || text[q] == '\r')) q++;
+        pos = end + 1;
+        if (q >= text.size() || text[q] != ':') continue;   // a string value, not a key
+        q++;
+        while (q < text.size() && (text[q] == ' ' || text[q] == '\t' || text[q] == '\n' || text[q] == '\r')) q++;
+        char *stop = nullptr;
+        const double v = std::strtod(text.c_str() + q, &stop);
+        if (stop == text.c_str() + q) { pos = q; continue; }  // no number behind the key
+        pos = (size_t)(stop - text.c_str());
+        const TuningEntry *e = find_tuning(key.c_str());
+        if (e && v == v && v >= 0.0 && v < 1e9) {
+            g_tuning.*(e->field) = v;
+            set++;
+        }
+    }
+    return set;
+}
 
 bool aligned(const void *p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
@@ -98,13 +173,61 @@ int select_b(const ProblemB &p, bool all_aligned16)
 }
 
 }  // namespace
+
+const Tuning &tuning()
+{
+    // the file named by VQGEMM_TUNING_FILE is read once, at the first question
+    if (!g_tuning_file_read) {
+        std::lock_guard<std::mutex> lock(g_tuning_mu);
+        if (!g_tuning_file_read) {
+            const char *path = std::getenv("VQGEMM_TUNING_FILE");
+            if (path && path[0]) read_tuning_file(path);
+            g_tuning_file_read = true;
+        }
+    }
+    return g_tuning;
+}
+
 }  // namespace vq
 
 using namespace vq;
 
 extern "C" {
 
-int vqgemm_version(void) { return 100; }
+int vqgemm_version(void) { return 200; }
+
+int vqgemm_tuning_count(void) { return kTuningCount; }
+
+const char *vqgemm_tuning_name(int index) { return index >= 0 && index < kTuningCount ? kTuningEntries[index].name : nullptr; }
+
+int vqgemm_tuning_get(const char *name, double *value)
+{
+    const TuningEntry *e = find_tuning(name);
+    if (!e) return VQGEMM_E_VARIANT;
+    if (!value) return VQGEMM_E_NULL;
+    *value = tuning().*(e->field);
+    return VQGEMM_OK;
+}
+
+int vqgemm_tuning_set(const char *name, double value)
+{
+    const TuningEntry *e = find_tuning(name);
+    if (!e) return VQGEMM_E_VARIANT;
+    if (!(value >= 0.0) || value >= 1e9) return VQGEMM_E_SHAPE;
+    (void)tuning();  // (a file is read before, not after, an explicit setting)
+    std::lock_guard<std::mutex> lock(g_tuning_mu);
+    g_tuning.*(e->field) = value;
+    return VQGEMM_OK;
+}
+
+int vqgemm_tuning_load(const char *path)
+{
+    if (!path) return VQGEMM_E_NULL;
+    (void)tuning();
+    std::lock_guard<std::mutex> lock(g_tuning_mu);
+    const int n = read_tuning_file(path);
+    return n < 0 ? VQGEMM_E_NULL : n;
+}
 
 const char *vqgemm_error_string(int code)
 {

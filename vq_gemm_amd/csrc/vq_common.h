@@ -147,6 +147,33 @@ hipError_t launch_max_code(const void *codes, int64_t count, int code_bits, uint
 
 int device_cu_count();
 
+// The constants of the cost models behind the automatic kernel choice.  The compiled-in values were fitted to
+// measurements on one 256-CU MI355X; vqgemm_tuning_set / a file named by VQGEMM_TUNING_FILE (written by
+// `python -m vq_gemm_amd.tune --fit`) replace them with what the box at hand measures.
+struct Tuning {
+    // prefill kernels: microseconds per tile of prologue + epilogue, and per 64-k stage on an idle device; a
+    // full device holds a lower clock: the stage time grows by `prefill_full_device_factor` at one tile per unit
+    double prefill_tile_fixed_us = 5.0;
+    double prefill_stage_us_256x256 = 1.0;
+    double prefill_stage_us_256x128 = 0.56;
+    double prefill_full_device_factor = 1.6;
+    double prefill_small_tile_fixed_us = 4.0;
+    double prefill_small_stage_us_idle = 0.46;
+    double prefill_small_stage_us_busy = 0.56;
+    // batched decode kernel: per workgroup a prologue, then per tile of 16 rows and 4096 k
+    double decode_prologue_us = 3.0;
+    double decode_prologue_shared_cu_us = 8.0;
+    double decode_tile_us = 0.75;
+    double decode_tile_chunked_us = 1.25;
+    double decode_pass_change_us = 5.0;
+    // GEMV kernels: the four-wave kernel up to this many 16-row tiles per unit and this K; the wide form from this
+    // many rows per wave on
+    double gemv_max_tiles_per_cu = 4.0;
+    double gemv_max_k = 6144.0;
+    double gemv_wide_min_rows_per_wave = 1.0;
+};
+const Tuning &tuning();
+
 // Raises a kernel's dynamic-LDS limit when `bytes` needs it; remembers what was granted per
 // (device, kernel) so that steady-state launches make no attribute call.
 hipError_t ensure_dynamic_lds(const void *kernel, size_t bytes);

@@ -807,9 +807,11 @@ bool decode_preferred(const ProblemB &p)
     const int per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
     const int rounds_d = (per_slab * g.n_slabs + cus * g.per_cu - 1) / (cus * g.per_cu);
     const bool shared = g.per_cu > 1;
-    const double t_tile = (g.n_chunks == 1 ? 0.75 : 1.25) * g.n_waves / kMaxWaves * g.per_cu * (shared ? 1.35 : 1.0);
+    const Tuning &tn = tuning();
+    const double t_tile = (g.n_chunks == 1 ? tn.decode_tile_us : tn.decode_tile_chunked_us) * g.n_waves / kMaxWaves * g.per_cu * (shared ? 1.35 : 1.0);
     const int passes = g.books_per_wg * g.n_chunks;
-    const double t_decode = rounds_d * ((shared ? 8.0 : 3.0) + passes * g.tiles_per_wg * t_tile + (passes - 1) * 5.0);
+    const double t_decode = rounds_d * ((shared ? tn.decode_prologue_shared_cu_us : tn.decode_prologue_us) + passes * g.tiles_per_wg * t_tile +
+                                        (passes - 1) * tn.decode_pass_change_us);
     const double t_prefill = prefill_supports(p) ? 1.0 + prefill_cost_us(p) : 1e30;
     return t_decode <= t_prefill;
 }
@@ -824,11 +826,6 @@ bool decode_preferred(const ProblemB &p)
 // 6.0 -> 4.8, 4 tiles 7.5 -> 6.6, 8 tiles 11.1 -> 11.1; K = 8192 (x takes 64 registers, two waves per
 // SIMD) is a tie already at 2 tiles.  Two rows of X (every gathered codeword meets both): one tile per
 // unit 5.0 -> 4.8, two tiles a tie; three and four rows lose everywhere (5.1 -> 5.6 and 6.6 on one tile).
-#ifndef VQ_GEMV_MAX_TILES_PER_CU
-#define VQ_GEMV_MAX_TILES_PER_CU 4
-#endif
-constexpr int kGemvAutoMaxK = 6144;
-
 bool decode_gemv_preferred(const ProblemB &p)
 {
     if (decode_gemv_wide_preferred(p)) return true;
@@ -838,9 +835,10 @@ bool decode_gemv_preferred(const ProblemB &p)
     // 16-bit codes / 4096 entries N = 11008 9.9 -> 9.5; 8-vectors / 16-bit codes / 4096 entries 5.6 -> 5.9).
     const bool first_format = p.vec == 8 && p.code_bits == 8;
     if (!first_format && (p.M != 1 || (int64_t)p.entries * p.vec * 2 > 32 * 1024)) return false;
-    const int max_tiles_per_cu = p.M == 1 ? VQ_GEMV_MAX_TILES_PER_CU : (p.M == 2 ? 1 : 0);
-    if (!decode_gemv_supports(p) || p.N / kTileN > max_tiles_per_cu * device_cu_count()) return false;
-    return p.K <= kGemvAutoMaxK;
+    const Tuning &tn = tuning();
+    const double max_tiles_per_cu = p.M == 1 ? tn.gemv_max_tiles_per_cu : (p.M == 2 ? 1.0 : 0.0);
+    if (!decode_gemv_supports(p) || (double)(p.N / kTileN) > max_tiles_per_cu * device_cu_count()) return false;
+    return (double)p.K <= tn.gemv_max_k;
 }
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)

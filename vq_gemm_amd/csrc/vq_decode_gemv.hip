@@ -553,14 +553,13 @@ bool decode_gemv_plain_supports(const ProblemB &p)
 
 bool decode_gemv_supports(const ProblemB &p) { return decode_gemv_wide_preferred(p) || decode_gemv_plain_supports(p); }
 
-// From this many rows per wave of the wide form on (sixteen waves per compute unit), one row of X goes to it.
-#ifndef VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE
-#define VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE 1
-#endif
+// From Tuning::gemv_wide_min_rows_per_wave rows per wave of the wide form on (sixteen waves per compute unit), one row
+// of X goes to it.
 
 bool decode_gemv_wide_preferred(const ProblemB &p)
 {
-    return decode_gemv_wide_supports(p) && (p.gated ? p.N / 2 : p.N) >= VQ_GEMV_WIDE_MIN_ROWS_PER_WAVE * kWideWaves * device_cu_count();
+    return decode_gemv_wide_supports(p) &&
+           (double)(p.gated ? p.N / 2 : p.N) >= tuning().gemv_wide_min_rows_per_wave * kWideWaves * device_cu_count();
 }
 
 namespace {

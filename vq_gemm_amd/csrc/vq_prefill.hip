@@ -827,10 +827,11 @@ double tile_cost_us(const ProblemB &p, int bn, int cols)
 {
     const int64_t tiles = (int64_t)((p.M + BM - 1) / BM) * cols;
     const int cus = device_cu_count();
-    const double stages = p.K / 64.0 * (bn == BN ? 1.0 : 0.56);
+    const Tuning &tn = tuning();
+    const double stages = p.K / 64.0 * (bn == BN ? tn.prefill_stage_us_256x256 : tn.prefill_stage_us_256x128);
     const int64_t full = tiles / cus, rem = tiles % cus;
-    double t = (double)full * (5.0 + stages * 1.6);
-    if (rem) t += 5.0 + stages * (1.0 + 0.6 * (double)rem / cus);
+    double t = (double)full * (tn.prefill_tile_fixed_us + stages * tn.prefill_full_device_factor);
+    if (rem) t += tn.prefill_tile_fixed_us + stages * (1.0 + (tn.prefill_full_device_factor - 1.0) * (double)rem / cus);
     return t;
 }
 

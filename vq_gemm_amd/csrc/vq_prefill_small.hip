@@ -401,7 +401,9 @@ double prefill_small_cost_us(const ProblemB &p)
     const int64_t tiles = (int64_t)((p.M + SBM - 1) / SBM) * ((p.N + SBN - 1) / SBN);
     const int64_t rounds = (tiles + cus - 1) / cus, resident_rounds = (tiles + 2 * cus - 1) / (2 * cus);
     const double busy = tiles >= cus ? 1.0 : (double)tiles / cus;
-    return (double)resident_rounds * 4.0 + (double)rounds * (p.K / 64.0 * (0.46 + 0.10 * busy));
+    const Tuning &tn = tuning();
+    return (double)resident_rounds * tn.prefill_small_tile_fixed_us +
+           (double)rounds * (p.K / 64.0 * (tn.prefill_small_stage_us_idle + (tn.prefill_small_stage_us_busy - tn.prefill_small_stage_us_idle) * busy));
 }
 
 hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s)

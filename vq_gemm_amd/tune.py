@@ -2,6 +2,17 @@
 
     python -m vq_gemm_amd.tune M K N [vec entries codebooks code_bits]
 
+or measures the box at hand and refits the constants of the cost models behind the automatic choice:
+
+    python -m vq_gemm_amd.tune --fit [--write [PATH]]
+
+`--fit` times forced variants on a fixed set of shapes (per-stage and per-tile times come out of pairs of
+shapes that differ in K or in the number of tiles), prints the fitted constants next to the compiled-in
+ones, and with `--write` stores them as a flat JSON object (default: vq_gemm_amd/tuning.json) that
+`vq_gemm_amd.cabi` hands to the library at its next load (`VQGEMM_TUNING_FILE`, `vqgemm_tuning_load`).
+The same run under `rocprofv3 --kernel-trace --stats -- python3 -m vq_gemm_amd.tune --fit` gives the
+per-kernel durations behind every figure.
+
 The choice between the kernels rests on cost models fitted to measurements on one MI355X; this
 prints, for the box at hand, the time of each variant that accepts the shape (launches replayed
 from a HIP graph), the variant `VQGEMM_VARIANT_AUTO` resolves to, its distance from the fastest,
@@ -77,7 +88,103 @@ def tune(M: int, K: int, N: int, vec: int = 8, entries: int = 256, n_codebooks: 
     return result
 
 
+def _t(M, K, N, variant, vec=8, entries=256, n_codebooks=1, code_bits=8, device="cuda:0"):
+    """Microseconds of one forced variant on one shape (None when the variant refuses it)."""
+    spec = ProblemSpec("fit", GEOM_B, M, K, N, vec, entries, n_codebooks, code_bits)
+    x, codes, cb = make_problem(spec, seed=1, device=device)
+    y = torch.empty(M, N, dtype=torch.float16, device=device)
+    try:
+        return time_graph(lambda: cabi.e2e_gemm_b(x, codes, cb, out=y, variant=variant))
+    except cabi.VqGemmError as e:
+        if e.code != -4:
+            raise
+        return None
+
+
+def fit(device: str = "cuda:0", verbose: bool = True) -> dict:
+    """Measures forced variants on shape pairs and returns the cost-model constants they imply for this box.
+    Constants whose measurement fails (a variant that refuses the shape) keep their current value."""
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    cur = cabi.tuning()
+    out = dict(cur)
+    say = print if verbose else (lambda *a, **k: None)
+
+    def pair(variant, M, N, k1, k2, **kw):
+        """(fixed microseconds, microseconds per 64-k stage) out of two K."""
+        t1, t2 = _t(M, k1, N, variant, **kw), _t(M, k2, N, variant, **kw)
+        if t1 is None or t2 is None:
+            return None
+        stage = (t2 - t1) / ((k2 - k1) / 64.0)
+        return t1 - stage * k1 / 64.0, stage
+
+    # prefill, 256x256 tiles on a full device (one tile per unit): fixed part and per-stage time
+    n_side = 256 * int(cus ** 0.5)
+    r = pair(cabi.VARIANT_PREFILL, n_side, n_side, 2048, 4096, n_codebooks=n_side // 128)
+    if r:
+        fixed, stage_full = r
+        factor = cur["prefill_full_device_factor"]
+        out["prefill_tile_fixed_us"] = max(fixed, 0.5)
+        out["prefill_stage_us_256x256"] = stage_full / factor
+        say(f"prefill 256x256, {n_side}x{n_side}: fixed {fixed:.2f} us, stage {stage_full:.3f} us on a full device")
+    r = pair(cabi.VARIANT_PREFILL_NARROW, n_side, n_side // 2, 2048, 4096, n_codebooks=n_side // 256)
+    if r:
+        out["prefill_stage_us_256x128"] = r[1] / cur["prefill_full_device_factor"]
+        say(f"prefill 256x128: fixed {r[0]:.2f} us, stage {r[1]:.3f} us on a full device")
+    # 128x128 tiles: a busy device (one tile per unit) and an idle one (a sixteenth of that)
+    rb = pair(cabi.VARIANT_PREFILL_SMALL, 128 * int(cus ** 0.5), 128 * int(cus ** 0.5), 2048, 4096)
+    ri = pair(cabi.VARIANT_PREFILL_SMALL, 512, 512, 2048, 4096)
+    if rb and ri:
+        out["prefill_small_tile_fixed_us"] = max(0.5 * (rb[0] + ri[0]), 0.5)
+        out["prefill_small_stage_us_busy"] = rb[1]
+        out["prefill_small_stage_us_idle"] = min(ri[1], rb[1])
+        say(f"prefill 128x128: fixed {rb[0]:.2f} / {ri[0]:.2f} us, stage {rb[1]:.3f} us busy, {ri[1]:.3f} us idle")
+    # batched decode kernel, 16 rows of X: one and eight tiles of 16 rows per unit
+    t1 = _t(16, 4096, 16 * cus, cabi.VARIANT_DECODE)
+    t8 = _t(16, 4096, 128 * cus, cabi.VARIANT_DECODE)
+    if t1 and t8:
+        tile = (t8 - t1) / 7.0
+        out["decode_tile_us"] = tile
+        out["decode_prologue_us"] = max(t1 - tile, 0.5)
+        say(f"decode, K=4096: {t1:.2f} us at one tile per unit, {t8:.2f} us at eight: {tile:.3f} us per tile")
+    t1c = _t(16, 8192, 16 * cus, cabi.VARIANT_DECODE)
+    t8c = _t(16, 8192, 128 * cus, cabi.VARIANT_DECODE)
+    if t1c and t8c:
+        out["decode_tile_chunked_us"] = (t8c - t1c) / 7.0 / 2.0   # per 4096 k
+        say(f"decode, K=8192 (two chunks): {(t8c - t1c) / 7.0:.3f} us per tile")
+    # four-wave GEMV kernel against the batched kernel, one row of X in a format the wide form does not take
+    best = 0.0
+    for tiles in (1, 2, 4, 8, 16):
+        tg = _t(1, 4096, 16 * cus * tiles, cabi.VARIANT_DECODE_GEMV, vec=4)
+        td = _t(1, 4096, 16 * cus * tiles, cabi.VARIANT_DECODE, vec=4)
+        if tg is None or td is None:
+            break
+        say(f"one row of X, 4-vectors, {tiles} tile(s) per unit: GEMV {tg:.2f} us, batched {td:.2f} us")
+        if tg <= td:
+            best = float(tiles)
+        else:
+            break
+    out["gemv_max_tiles_per_cu"] = best
+    # (gemv_wide_min_rows_per_wave and gemv_max_k keep their values: the wide form wins its short launches on codes that
+    # come from HBM and loses them on cached ones - 3.3 against 3.5 us cold, 3.2 against 2.7 us warm on C2 - and this
+    # loop times warm launches; bench.py's rotating pool is the protocol that decides them.)
+    if verbose:
+        print("constant                          compiled-in / current -> fitted")
+        for k in out:
+            print(f"  {k:32s} {cur[k]:8.3f} -> {out[k]:8.3f}")
+    return out
+
+
 def main(argv) -> int:
+    if argv and argv[0] == "--fit":
+        import json
+        fitted = fit()
+        if "--write" in argv:
+            i = argv.index("--write")
+            path = argv[i + 1] if len(argv) > i + 1 else cabi.TUNING_FILE
+            with open(path, "w") as f:
+                json.dump({"device": torch.cuda.get_device_name(0), **fitted}, f, indent=1)
+            print("wrote", path)
+        return 0
     if len(argv) not in (3, 7):
         print(__doc__)
         return 2
