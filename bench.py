@@ -61,6 +61,15 @@ def parse_args():
                          "device copy as a counter yardstick; prints no JSON")
     ap.add_argument("--probe-variant", type=int, default=0,
                     help="with --probe on a geometry-B shape: the VQGEMM_VARIANT_* value to launch (0 = automatic choice)")
+    ap.add_argument("--probe-skew", type=float, default=1.0,
+                    help="with --probe on a geometry-B shape: codes = floor(entries * u^P) for uniform u; 1 = uniform codes (the "
+                         "measured configurations), larger P concentrates the codes on few 'hot' entries (P = 4: half of all "
+                         "codes fall on 6 %% of the entries) - for counter runs on what a skewed code distribution does to the gathers")
+    ap.add_argument("--study", choices=["gated", "split-k", "code-usage"], default=None,
+                    help="print one JSON report instead of the benchmark line: 'gated' times gate/up projection pairs as the "
+                         "plain product + element-wise pass and as the gated entry point; 'split-k' times C3 whole and as "
+                         "K slices with a summing pass behind them; 'code-usage' quantises Gaussian and heavy-tailed "
+                         "weights with the package's k-means and reports how unevenly the entries are used")
     ap.add_argument("--launch-floor", action="store_true",
                     help="run the empty-kernel launch probe (vq_gemm_amd/lib/launch_floor): what one launch of a replayed "
                          "HIP graph costs on this device when the kernel does nothing; prints no JSON")
@@ -147,8 +156,12 @@ def main():
             return
         n_bufs = max(1, min(512, POOL_BYTES // spec.code_bytes)) if spec.M <= 16 else 1
         gen = torch.Generator(device=dev).manual_seed(1234)
-        pool = [codes] + [torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev,
-                                        dtype=torch.int32).to(spec.code_dtype) for _ in range(n_bufs - 1)]
+        def draw_codes():
+            if args.probe_skew == 1.0:
+                return torch.randint(0, spec.entries, spec.codes_shape, generator=gen, device=dev, dtype=torch.int32).to(spec.code_dtype)
+            u = torch.rand(spec.codes_shape, generator=gen, device=dev)
+            return (u.pow(args.probe_skew) * spec.entries).to(torch.int32).clamp_(0, spec.entries - 1).to(spec.code_dtype)
+        pool = [codes if args.probe_skew == 1.0 else draw_codes()] + [draw_codes() for _ in range(n_bufs - 1)]
         if args.probe_variant == cabi.VARIANT_DECODE_PACKED:   # that variant reads code matrices re-laid offline
             pool = [cabi.pack_codes_b(c, spec.vec) for c in pool]
         y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
@@ -281,6 +294,87 @@ def main():
         del pool, wpool
         torch.cuda.empty_cache()
         return res, (x, codes, cb, y0)
+
+    if args.study == "gated":
+        # A gate/up pair of an MLP, H outputs each: before = one product [M, 2H] written to HBM, then the element-wise
+        # pass reads it back; after = the gated entry point (epilogue inside the GEMM kernel where one applies).
+        report = {}
+        for name, M, K, H, G in (("prefill_m2048_k8192_h14336", 2048, 8192, 14336, 56), ("prefill_m2048_k4096_h11008", 2048, 4096, 11008, 43),
+                                 ("prefill_m512_k4096_h11008", 512, 4096, 11008, 43), ("decode_m16_k4096_h11008", 16, 4096, 11008, 1),
+                                 ("decode_m1_k4096_h14336", 1, 4096, 14336, 1), ("decode_m1_k8192_h14336", 1, 8192, 14336, 1),
+                                 ("decode_m1_k4096_h11008", 1, 4096, 11008, 1)):
+            spec = ProblemSpec(name, GEOM_B, M, K, 2 * H, 8, 256, G, 8)
+            x, codes, cb = make_problem(spec, seed=42, device=dev)
+            cold = M <= 16
+            n_bufs = max(1, min(512, POOL_BYTES // spec.code_bytes)) if cold else 1
+            gen = torch.Generator(device=dev).manual_seed(1234)
+            pool = [codes] + [torch.randint(0, 256, spec.codes_shape, generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+                              for _ in range(n_bufs - 1)]
+            prod = torch.empty(M, 2 * H, dtype=torch.float16, device=dev)
+            y = torch.empty(M, H, dtype=torch.float16, device=dev)
+            steps, warm, min_l = (200, 20, MIN_TIMED_LAUNCHES) if cold else (10, 3, 1)
+            t_before = time_launches(lambda i: (cabi.e2e_gemm_b(x, pool[i], cb, out=prod), cabi.silu_mul(prod, out=y)),
+                                     n_bufs, steps, warm, min_launches=min_l)[0]
+            t_plain = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[i], cb, out=prod), n_bufs, steps, warm, min_launches=min_l)[0]
+            t_after = time_launches(lambda i: cabi.e2e_gemm_b_gated(x, pool[i], cb, out=y, workspace=prod), n_bufs, steps, warm,
+                                    min_launches=min_l)[0]
+            report[name] = {"M": M, "K": K, "H": H, "n_codebooks": G,
+                            "product_then_elementwise_us": t_before * 1e6, "product_alone_us": t_plain * 1e6,
+                            "gated_entry_point_us": t_after * 1e6, "speedup": t_before / t_after,
+                            "plain_variant": cabi.VARIANT_NAMES[cabi.select_variant_b(M, K, 2 * H, 8, 256, G, 8)],
+                            "cold_code_buffers": n_bufs}
+            del pool, prod, y
+            torch.cuda.empty_cache()
+        print(json.dumps({"study": "gated", "shapes": report}))
+        return
+
+    if args.study == "split-k":
+        # Would splitting K across workgroups pay on C3?  A split-K launch of S slices reads the same code bytes, gives every
+        # workgroup 1/S of X to pull, and leaves S partial products to sum.  The slices are timed as what they are to the kernel,
+        # an [M, K/S] x [S*N, K/S] problem (same code bytes, same number of row tiles x S), plus the summing pass over [S, M, N].
+        spec = CONFIGS["C3"]
+        report = {}
+        for S in (1, 2, 4):
+            sspec = ProblemSpec(f"C3/{S}", GEOM_B, spec.M, spec.K // S, spec.N * S, spec.vec, spec.entries, 1, spec.code_bits)
+            x, codes, cb = make_problem(sspec, seed=42, device=dev)
+            n_bufs = max(1, min(512, POOL_BYTES // sspec.code_bytes))
+            gen = torch.Generator(device=dev).manual_seed(1234)
+            pool = [codes] + [torch.randint(0, spec.entries, sspec.codes_shape, generator=gen, device=dev, dtype=torch.int32).to(sspec.code_dtype)
+                              for _ in range(n_bufs - 1)]
+            part = torch.empty(spec.M, spec.N * S, dtype=torch.float16, device=dev)
+            ysum = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
+            t_prod = time_launches(lambda i: cabi.e2e_gemm_b(x, pool[i], cb, out=part), n_bufs, 200, 20)[0]
+            if S > 1:
+                view = part.view(spec.M, S, spec.N)
+                t_both = time_launches(lambda i: (cabi.e2e_gemm_b(x, pool[i], cb, out=part), torch.sum(view, dim=1, out=ysum)),
+                                       n_bufs, 200, 20)[0]
+            else:
+                t_both = t_prod
+            report[f"slices_{S}"] = {"K_per_slice": spec.K // S, "rows": spec.N * S, "product_us": t_prod * 1e6,
+                                     "with_summing_pass_us": t_both * 1e6,
+                                     "variant": cabi.VARIANT_NAMES[cabi.select_variant_b(spec.M, spec.K // S, spec.N * S, spec.vec,
+                                                                                         spec.entries, 1, spec.code_bits)]}
+            del pool, part, ysum
+            torch.cuda.empty_cache()
+        print(json.dumps({"study": "split-k", "config": "C3", "slices": report}))
+        return
+
+    if args.study == "code-usage":
+        # How unevenly does a trained codebook use its entries?  A "hot entry" table only pays when few entries carry most codes.
+        import numpy as np
+
+        from vq_gemm_amd.quantize import kmeans_quantize
+        torch.manual_seed(0)
+        report = {}
+        for name, w in (("gaussian", torch.randn(1024, 4096)),
+                        ("student_t_3dof", torch.distributions.StudentT(3.0).sample((1024, 4096)))):
+            q = kmeans_quantize(w.half().to(dev), 8, 256, 1, iters=10)
+            h = np.bincount(q[0].cpu().numpy().astype(np.int64).ravel(), minlength=256).astype(np.float64)
+            h = np.sort(h)[::-1] / h.sum()
+            report[name] = {"share_of_16_most_used": h[:16].sum(), "share_of_32": h[:32].sum(), "share_of_64": h[:64].sum(),
+                            "most_used_over_mean": h[0] * 256, "entropy_bits": float(-(h[h > 0] * np.log2(h[h > 0])).sum())}
+        print(json.dumps({"study": "code-usage", "format": "8-vectors, 256 entries, 1024x4096 weights", "weights": report}))
+        return
 
     # ---- headline: decode GEMV ---------------------------------------------------------------
     main_name = "C2"

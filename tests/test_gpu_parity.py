@@ -1249,8 +1249,14 @@ GATED_B = [
     ("gemv_wide", 1, 4096, 8192, 8, 256, 8, 1),                  # one row of X: one output per group of two code rows
     ("gemv_wide_ragged_two_books", 1, 2048, 8192 + 64, 8, 200, 8, 2),
     ("gemv_wide_many_books", 1, 4096, 16384, 8, 256, 8, 16),
-    ("decode_shape", 16, 1024, 2048, 4, 4096, 16, 1),           # the K-sliced kernels have no gated epilogue
+    ("gemv_wide_k8192", 1, 8192, 16384, 8, 256, 8, 1),           # gate row and up row as two groups of one row in turn
+    ("gemv_wide_k6144_books", 1, 6144, 3 * 2752, 8, 256, 8, 3),
+    ("decode_shape", 16, 1024, 2048, 4, 4096, 16, 1),           # batched K-sliced kernel: gate and up tiles summed in pairs
     ("decode_shape_m2", 2, 4096, 4096, 8, 256, 8, 1),
+    ("decode_books_ragged_units", 16, 4096, 4 * 1056, 8, 256, 8, 4),   # 33 pairs per codebook: short last batches
+    ("decode_chunked_k", 9, 8192, 1024, 8, 256, 8, 1),           # K in two chunks: gate and up sums carried in the LDS
+    ("decode_two_slabs_u8v4", 40, 2048, 1536, 4, 256, 8, 2),
+    ("decode_v2_u16_no_pairs", 16, 1024, 512, 2, 4096, 16, 1),   # batches of one tile: no gated form, two passes
     ("odd_k_scalar_only", 5, 72, 64, 8, 256, 8, 1),
 ]
 
@@ -1284,7 +1290,9 @@ def test_gated_epilogue_against_the_oracle(row):
             _say(f"    rel_err(floor)={e1:.3e} max/max={e2:.3e}")
             assert e2 <= TOL and e1 <= 2 * TOL, (name, variant, e1, e2)
             ran.append(variant)
-    assert cabi.VARIANT_DECODE not in ran and cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran
+    assert cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran
+    if name.startswith("decode_"):
+        assert (cabi.VARIANT_DECODE in ran) == (name != "decode_v2_u16_no_pairs")
     if name.startswith("gemv_wide"):
         assert cabi.VARIANT_DECODE_GEMV in ran
     if name.endswith("_tile") or "tile_" in name:

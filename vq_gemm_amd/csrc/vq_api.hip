@@ -349,12 +349,15 @@ int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebo
         if (K == 0 || !a16) variant = VQGEMM_VARIANT_GENERIC;
         else if (decode_gemv_wide_preferred(p)) variant = VQGEMM_VARIANT_DECODE_GEMV;
         else {
-            // What the plain product would run on decides: the prefill kernels carry the gated epilogue themselves;
-            // where a decode kernel would be chosen, the product goes to the workspace and the element-wise pass
-            // follows (two launches), or - without a workspace - the prefill kernels take it after all.
+            // What the plain product would run on decides: the prefill kernels and the batched K-sliced decode kernel
+            // carry the gated epilogue themselves; where another decode kernel would be chosen (the four-wave GEMV, the
+            // general K-sliced kernel), the product goes to the workspace and the element-wise pass follows (two
+            // launches), or - without a workspace - the batched decode or the prefill kernels take it after all.
             const int plain_variant = select_b(plain, true);
             const bool decode_like = plain_variant == VQGEMM_VARIANT_DECODE || plain_variant == VQGEMM_VARIANT_DECODE_GEMV;
-            if (decode_like && workspace) variant = VQGEMM_VARIANT_TWOPASS;
+            if (plain_variant == VQGEMM_VARIANT_DECODE && decode_gated_supports(p)) variant = VQGEMM_VARIANT_DECODE;
+            else if (decode_like && workspace) variant = VQGEMM_VARIANT_TWOPASS;
+            else if (decode_like && decode_gated_supports(p)) variant = VQGEMM_VARIANT_DECODE;
             else if (prefill_supports(plain)) variant = VQGEMM_VARIANT_PREFILL;
             else variant = VQGEMM_VARIANT_GENERIC;
         }
@@ -368,6 +371,11 @@ int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebo
         if (!a16) return VQGEMM_E_ALIGN;
         if (K == 0 || !decode_gemv_wide_preferred(p)) return VQGEMM_E_VARIANT;
         e = launch_decode_gemv(p, s);
+        break;
+    case VQGEMM_VARIANT_DECODE:
+        if (!a16) return VQGEMM_E_ALIGN;
+        if (K == 0 || !decode_gated_supports(p)) return VQGEMM_E_VARIANT;
+        e = launch_decode_b(p, s);
         break;
     case VQGEMM_VARIANT_PREFILL:
         if (!a16) return VQGEMM_E_ALIGN;
@@ -394,7 +402,7 @@ int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebo
         break;
     }
     default:
-        return VQGEMM_E_VARIANT;  // the K-sliced decode kernels have no gated epilogue
+        return VQGEMM_E_VARIANT;
     }
     return static_cast<int>(e);
 }

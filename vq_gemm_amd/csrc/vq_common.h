@@ -107,8 +107,8 @@ bool decode_gemv_preferred(const ProblemB &p);
 bool decode_general_supports(const ProblemB &p);
 hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);
 
-// whether some fused kernel takes the shape with p.gated set (the prefill kernels, the wide GEMV kernel, the scalar kernel)
-bool gated_supports(const ProblemB &p);
+// whether the batched K-sliced decode kernel takes the shape with its gated epilogue (p.gated set)
+bool decode_gated_supports(const ProblemB &p);
 
 bool prefill_supports(const ProblemB &p);
 // whether the 256x128 tile of the prefill kernel can serve the shape (a subset of prefill_supports)

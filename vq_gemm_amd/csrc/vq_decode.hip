@@ -233,7 +233,12 @@ constexpr int kStageOverTable = 1, kStageOverSlots = 2;
 __device__ __forceinline__ const half_t *bias_of() { return nullptr; }
 __device__ __forceinline__ const half_t *bias_of(const half_t *b) { return b; }
 
-template <int VEC, typename CodeT, bool REPL, int TB, bool PACKED, typename... Bias>
+//
+// GATED: the epilogue of a gate/up pair.  The rows of W are gate and up rows interleaved in groups of 16, so an
+// even tile holds gate rows and the tile behind it the up rows of the same 16 outputs: workgroups are dealt whole
+// pairs of tiles (tiles_q and tiles_r then count pairs), TB is even, and a reducing lane sums the gate slot and the
+// matching up slot and stores silu(gate) * up into Y [m_total, N/2].
+template <int VEC, typename CodeT, bool REPL, int TB, bool PACKED, bool GATED, typename... Bias>
 __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__restrict__ x,
                                                                const CodeT *__restrict__ codes,
                                                                const half_t *__restrict__ cb,
@@ -260,7 +265,10 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     const int M = min(kTileN, m_total - slab_row);
     const int recip_m = M == kTileN ? 65536 / kTileN : recip_tail;
     x += (int64_t)slab_row * K;
-    y += (int64_t)slab_row * N;
+    static_assert(!GATED || TB % 2 == 0, "gate and up tiles come in pairs");
+    constexpr int kDeal = GATED ? 2 : 1;  // tiles per unit that is dealt to the workgroups
+    const int ldy = GATED ? N / 2 : N;
+    y += (int64_t)slab_row * ldy;
     constexpr int kPieces = Operand<VEC>::kPieces;
     constexpr int kEntryBytes = VEC * 2;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -286,8 +294,8 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     const int book_end = min(n_books, book_begin + books_per_wg);
     const int wg = wgs_per_cb > 1 ? (int)blockIdx.x - book_begin * wgs_per_cb : 0;
     int book = book_begin;
-    int tile_begin = book * tiles_per_cb + wg * tiles_q + min(wg, tiles_r);
-    int tile_end = tile_begin + tiles_q + (wg < tiles_r ? 1 : 0);
+    int tile_begin = book * tiles_per_cb + kDeal * (wg * tiles_q + min(wg, tiles_r));
+    int tile_end = tile_begin + kDeal * (tiles_q + (wg < tiles_r ? 1 : 0));
     if (book >= book_end || tile_begin >= tile_end) return;
     cb += (int64_t)book * entries * VEC;
     int n_units = (tile_end - tile_begin + TB - 1) / TB;
@@ -412,7 +420,8 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     const uint32_t wr_addr = red_base + (uint32_t)(kq * M + r16) * kSlotPitch + w * 16;
     const uint32_t wr_stride = (uint32_t)(4 * M) * kSlotPitch;
     const int n_slots = TB * 4 * M;
-    const int n_passes = (n_slots + 63) >> 6;
+    const int n_out_slots = n_slots / kDeal;  // what the reducing lanes are dealt: slots, or pairs of a gate and an up slot
+    const int n_passes = (n_out_slots + 63) >> 6;
     int turn = 0;  // the wave that takes the next reduction pass
 
     auto process_unit = [&](int q, Codes (&cur)[TB]) {
@@ -479,23 +488,25 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
         // first (`locate`), the sum and the store follow (`finish`).
         struct Target { uint32_t src, carry; half_t *dst; int n; bool live; };  // LDS offsets, output address, first W row
         auto locate = [&](int pass) {
-            const int slot = pass * 64 + opaque(lane);
-            const int jq = (slot * recip_m) >> 16;  // slot / M = j*4 + kq
-            const int m = slot - jq * M;
-            const int tile = tile_begin + q * TB + (jq >> 2);
+            const int out = pass * 64 + opaque(lane);
+            const int jq = (out * recip_m) >> 16;  // out / M = j*4 + kq (GATED: j counts pairs of tiles)
+            const int m = out - jq * M;
+            const int j = kDeal * (jq >> 2);       // tile of the unit (GATED: the gate tile)
+            const int tile = tile_begin + q * TB + j;
+            const int slot = GATED ? (j * 4 + (jq & 3)) * M + m : out;
             Target t;
             t.src = red_base + slot * kSlotPitch;
             // with several chunks the sums are carried from chunk to chunk in the LDS, one entry per slot of the range
             t.carry = (uint32_t)acc_off + (uint32_t)(q * n_slots + slot) * 16u;
             // D[i][j] of the tile: the slot holds rows i = 4*kq .. 4*kq+3 of column j = m.
             t.n = tile * kTileN + 4 * (jq & 3);
-            t.dst = y + (int64_t)m * N + t.n;
-            t.live = pass < n_passes && slot < n_slots && tile < tile_end;
+            t.dst = GATED ? y + (int64_t)m * ldy + (tile >> 1) * kTileN + 4 * (jq & 3) : y + (int64_t)m * N + t.n;
+            t.live = pass < n_passes && out < n_out_slots && tile < tile_end;
             return t;
         };
-        auto finish = [&](const Target &t) {
-            if (!t.live) return;
-            const float4_t *src = reinterpret_cast<const float4_t *>(smem + t.src);
+        // the sum over the waves of one slot, carried across the chunks of K; `last` = this was the last chunk
+        auto sum_slot = [&](uint32_t src_off, uint32_t carry_off, int n_bias, bool &last) {
+            const float4_t *src = reinterpret_cast<const float4_t *>(smem + src_off);
             float4_t sum;
             if (n_act == kMaxWaves) {
                 // four interleaved chains, to keep the run of dependent additions short
@@ -509,15 +520,28 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
                 sum = src[0];
                 for (int i = 1; i < n_act; i++) sum += src[i];
             }
-            float4_t *carry = reinterpret_cast<float4_t *>(smem + t.carry);
+            float4_t *carry = reinterpret_cast<float4_t *>(smem + carry_off);
             if (chunk > 0) sum += *carry;
-            if (chunk < n_chunks - 1) {
+            last = chunk >= n_chunks - 1;
+            if (!last) {
                 *carry = sum;
-            } else {
-                if constexpr (kHasBias) {
-                    const half4_t b = *reinterpret_cast<const half4_t *>(bias + t.n);
-                    sum += float4_t{(float)b[0], (float)b[1], (float)b[2], (float)b[3]};
-                }
+            } else if constexpr (kHasBias) {
+                const half4_t b = *reinterpret_cast<const half4_t *>(bias + n_bias);
+                sum += float4_t{(float)b[0], (float)b[1], (float)b[2], (float)b[3]};
+            }
+            return sum;
+        };
+        auto finish = [&](const Target &t) {
+            if (!t.live) return;
+            bool last;
+            float4_t sum = sum_slot(t.src, t.carry, t.n, last);
+            if constexpr (GATED) {
+                // the up slot of the same outputs: one tile (4*M slots) further on
+                const float4_t up = sum_slot(t.src + (uint32_t)(4 * M) * kSlotPitch, t.carry + (uint32_t)(4 * M) * 16u, t.n + kTileN, last);
+#pragma unroll
+                for (int e = 0; e < 4; e++) sum[e] = silu_f32(sum[e]) * up[e];
+            }
+            if (last) {
                 half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
                 *reinterpret_cast<half4_t *>(t.dst) = h;
             }
@@ -605,6 +629,10 @@ BatchedPlan plan_batched(const ProblemB &p)
     typedef DecodeCfg<VEC, CodeT> C;
     BatchedPlan g = {};
     if (p.K % kSliceK != 0 || p.N % kTileN != 0 || p.rows_per_cb % kTileN != 0) return g;
+    // gated: whole pairs of a gate and an up tile per codebook, dealt to the workgroups as pairs, in batches of an even
+    // number of tiles; the packed code layout is not read
+    const int deal = p.gated ? 2 : 1;
+    if (p.gated && (p.rows_per_cb % (2 * kTileN) != 0 || C::TB % 2 != 0 || p.packed)) return g;
     const int slices = p.K / kSliceK;
     g.n_chunks = (slices + kMaxWaves - 1) / kMaxWaves;
     g.n_waves = (slices + g.n_chunks - 1) / g.n_chunks;
@@ -620,7 +648,7 @@ BatchedPlan plan_batched(const ProblemB &p)
     if (per_slab < 1) per_slab = 1;
     if (per_slab >= p.n_codebooks) {
         const int per_cb = per_slab / p.n_codebooks;
-        g.wgs_per_cb = per_cb < g.tiles_per_cb ? per_cb : g.tiles_per_cb;
+        g.wgs_per_cb = per_cb < g.tiles_per_cb / deal ? per_cb : g.tiles_per_cb / deal;
         g.books_per_wg = 1;
     } else {
         g.wgs_per_cb = 1;
@@ -631,7 +659,7 @@ BatchedPlan plan_batched(const ProblemB &p)
     const size_t slot_bytes = (size_t)4 * m_slab * kSlotPitch;  // per tile of a batch
     const size_t carry_bytes = (size_t)4 * m_slab * 16;         // per tile of the workgroup's range
     for (;;) {
-        g.tiles_per_wg = (g.tiles_per_cb + g.wgs_per_cb - 1) / g.wgs_per_cb;
+        g.tiles_per_wg = deal * ((g.tiles_per_cb / deal + g.wgs_per_cb - 1) / g.wgs_per_cb);
         g.full = g.tiles_per_wg >= 2;
         const int tb = g.full ? C::TB : 1;
         const size_t slots = tb * slot_bytes;
@@ -669,9 +697,9 @@ BatchedPlan plan_batched(const ProblemB &p)
             }
         }
         // Too many carried sums: fewer tiles per workgroup (more workgroups than are resident).
-        if (g.n_chunks == 1 || g.wgs_per_cb >= g.tiles_per_cb) return g;
+        if (g.n_chunks == 1 || g.wgs_per_cb >= g.tiles_per_cb / deal) return g;
         if (g.books_per_wg > 1) g.books_per_wg = 1;  // one codebook per workgroup first
-        else g.wgs_per_cb = g.wgs_per_cb * 2 < g.tiles_per_cb ? g.wgs_per_cb * 2 : g.tiles_per_cb;
+        else g.wgs_per_cb = g.wgs_per_cb * 2 < g.tiles_per_cb / deal ? g.wgs_per_cb * 2 : g.tiles_per_cb / deal;
     }
 }
 
@@ -693,29 +721,39 @@ hipError_t launch_decode_batched(const ProblemB &p, hipStream_t s)
     if (!g.ok) return hipErrorInvalidValue;
     g.per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
     const int tail_rows = p.M - (g.n_slabs - 1) * kTileN;
+    const int dealt = p.gated ? g.tiles_per_cb / 2 : g.tiles_per_cb;  // what the workgroups of a codebook share: tiles, or pairs
     // the same launch for the instantiation with a bias argument and the one without
     auto launch = [&](auto kern, auto... bias) {
         hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), g.smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(g.per_slab, g.n_slabs), dim3(g.n_waves * 64), g.smem, s, p.x,
                            static_cast<const CodeT *>(p.codes), p.cb, p.y, p.M, p.K, p.N, p.entries, p.n_codebooks,
-                           g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, g.tiles_per_cb / g.wgs_per_cb,
-                           g.tiles_per_cb % g.wgs_per_cb, g.n_chunks, g.red_off, g.stage_off, g.stage_over, g.acc_off,
+                           g.wgs_per_cb, g.books_per_wg, g.tiles_per_cb, dealt / g.wgs_per_cb,
+                           dealt % g.wgs_per_cb, g.n_chunks, g.red_off, g.stage_off, g.stage_over, g.acc_off,
                            (65536 + tail_rows - 1) / tail_rows, bias...);
         return hipGetLastError();
     };
     // a full batch of one tile is the only case with a replicated table and TB = 1
     const int tb = g.full ? C::TB : 1;
-    if (p.bias) {
-        if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, PACKED, const half_t *>, p.bias)
-                                   : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, PACKED, const half_t *>, p.bias);
-        return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, PACKED, const half_t *>, p.bias)
-                       : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, PACKED, const half_t *>, p.bias);
+    if constexpr (!PACKED && C::TB % 2 == 0) {
+        if (p.gated) {
+            if (p.bias) return g.repl ? launch(decode_batched_kernel<VEC, CodeT, true, C::TB, false, true, const half_t *>, p.bias)
+                                      : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, false, true, const half_t *>, p.bias);
+            return g.repl ? launch(decode_batched_kernel<VEC, CodeT, true, C::TB, false, true>)
+                          : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, false, true>);
+        }
     }
-    if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, PACKED>)
-                               : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, PACKED>);
-    return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, PACKED>)
-                   : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, PACKED>);
+    if (p.gated) return hipErrorInvalidValue;
+    if (p.bias) {
+        if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, PACKED, false, const half_t *>, p.bias)
+                                   : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, PACKED, false, const half_t *>, p.bias);
+        return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, PACKED, false, const half_t *>, p.bias)
+                       : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, PACKED, false, const half_t *>, p.bias);
+    }
+    if (g.repl) return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, true, 1, PACKED, false>)
+                               : launch(decode_batched_kernel<VEC, CodeT, true, C::TB, PACKED, false>);
+    return tb == 1 ? launch(decode_batched_kernel<VEC, CodeT, false, 1, PACKED, false>)
+                   : launch(decode_batched_kernel<VEC, CodeT, false, C::TB, PACKED, false>);
 }
 
 // ---- packed code layout ---------------------------------------------------------------------
@@ -784,6 +822,12 @@ hipError_t launch_pack_codes(const void *src, void *dst, int64_t N, int64_t K, i
     }
 }
 
+// the gated epilogue: the batched kernel only
+bool decode_gated_supports(const ProblemB &p)
+{
+    return p.gated && p.M >= 1 && p.M <= kBatchedMaxM && decode_general_supports(p) && batched_supports(p);
+}
+
 bool decode_supports(const ProblemB &p)
 {
     if (p.M < 1 || !decode_general_supports(p)) return false;
@@ -843,8 +887,9 @@ bool decode_gemv_preferred(const ProblemB &p)
 
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
-    if (p.gated || !decode_supports(p)) return hipErrorInvalidValue;  // (the K-sliced kernels have no gated epilogue)
+    if (!decode_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
+    if (p.gated && !batched_supports(p)) return hipErrorInvalidValue;  // (the general kernel has no gated epilogue)
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension
         if (p.packed) {

@@ -277,7 +277,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 {
     // gated: the epilogue of a gate/up pair.  The rows of W are gate and up rows interleaved in groups of 16; what
     // is dealt out to the waves (rows_q, rows_r, n_total) are then the N/2 outputs, a wave's code rows are the gate
-    // and the up row of each of its outputs in turn, and a group of two rows is one output (G = 2).
+    // and the up row of each of its outputs in turn; a group of two rows is one output (G = 2), or the gate row and the
+    // up row are two groups in turn (G = 1).
     constexpr bool TWO = BOOKS == 2;
     constexpr int kXChunks = RUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
@@ -400,6 +401,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     const uint32_t copy_base = (lane & (kWideCopies - 1)) * 16u;
     const uint8_t *tbl = reinterpret_cast<const uint8_t *>(table);
     float res = 0.f;  // lane i: the sum of the wave's row i
+    float gate_sum = 0.f;  // gated, G = 1: the gate row's sum (wave-uniform) until the up row's group has run
     // rows [g*G, g*G + R) of the wave, R <= G (a compile-time count: the last group may be short)
     auto multiply_rows = [&](int g, const uint32_t (&cur)[G][RUNS], auto r_const) {
         constexpr int R = decltype(r_const)::value;
@@ -437,6 +439,18 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
             const float sg = wave_sum_to_uniform(acc[0]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), g));
             const float su = wave_sum_to_uniform(acc[R - 1]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), g));
             res = (int)lane == g ? silu_f32(sg) * su : res;
+            return;
+        }
+        if (G == 1 && gated) {
+            // even groups are gate rows, odd groups the up rows of the same output
+            const int o = g >> 1;
+            const float s = wave_sum_to_uniform(acc[0]);
+            if ((g & 1) == 0) {
+                gate_sum = s + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), o));
+            } else {
+                const float su = s + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), o));
+                res = (int)lane == o ? silu_f32(gate_sum) * su : res;
+            }
             return;
         }
 #pragma unroll
@@ -490,8 +504,9 @@ bool decode_gemv_wide_supports(const ProblemB &p)
     if (p.K < kRunK || p.K % kRunK != 0 || p.K / kRunK > kGemvMaxRuns || p.N < 1) return false;
     const int waves = device_cu_count() * kWideWaves;
     if (p.gated) {
-        // two code rows per output, one output per group of two rows: K up to 4096 (the instantiations with G = 2)
-        if (p.N % 32 != 0 || p.K / kRunK > 2 || VQ_GEMV_WIDE_G != 2) return false;
+        // two code rows per output: one group of two rows, or two groups of one
+        const int g = p.K / kRunK > 2 ? VQ_GEMV_WIDE_G4 : VQ_GEMV_WIDE_G;
+        if (p.N % 32 != 0 || g > 2) return false;
         const int outs_per_wave = (p.N / 2 + waves - 1) / waves;
         if (outs_per_wave > 32) return false;
         // a workgroup's rows of W: its outputs' gate and up rows, in whole groups of 32
