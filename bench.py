@@ -70,6 +70,10 @@ def parse_args():
                          "plain product + element-wise pass and as the gated entry point; 'split-k' times C3 whole and as "
                          "K slices with a summing pass behind them; 'code-usage' quantises Gaussian and heavy-tailed "
                          "weights with the package's k-means and reports how unevenly the entries are used")
+    ap.add_argument("--probe-flat-codebook", action="store_true",
+                    help="with --probe on a geometry-B shape: every entry of a codebook is a copy of its first entry, so that W is "
+                         "constant whatever the codes are (the control for --probe-skew 1000: same W, but the gathers still go to "
+                         "random entries)")
     ap.add_argument("--launch-floor", action="store_true",
                     help="run the empty-kernel launch probe (vq_gemm_amd/lib/launch_floor): what one launch of a replayed "
                          "HIP graph costs on this device when the kernel does nothing; prints no JSON")
@@ -146,6 +150,9 @@ def main():
             m, k, n, vec, entries, bits = (int(v) for v in args.probe.split(","))
             spec = ProblemSpec("probe", GEOM_B, m, k, n, vec, entries, 1, bits)
         x, codes, cb = make_problem(spec, seed=42, device=dev)
+        if args.probe_flat_codebook and spec.geometry == GEOM_B:
+            cb3 = cb.view(-1, spec.entries, spec.vec)
+            cb3.copy_(cb3[:, :1, :].expand_as(cb3).clone())
         if spec.geometry == GEOM_A:
             y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
             barrier()

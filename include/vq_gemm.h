@@ -50,15 +50,17 @@ extern "C" {
                                             in the order the kernel's lanes load it (never chosen by AUTO: the
                                             layout is a property of the caller's data); the K-sliced MFMA kernel
                                             whatever the shape, same results as on the plain matrix bit for bit */
-#define VQGEMM_VARIANT_DECODE_GEMV 8     /* the GEMV kernel: M <= 4 for 8-vectors with 8-bit codes, M <= 2 for 4-vectors,
-                                            8-vectors with 16-bit codes and 2-vectors with 8-bit codes; at most 256
-                                            resp. 4096 entries, entries * vec a multiple of 8; K a multiple of 2048
-                                            with (K / 2048) * M <= 8, N and N / n_codebooks multiples of 16; whole
-                                            rows of W per wave, no matrix core.  AUTO takes it where it was measured
-                                            faster (M == 1: at most 4 tiles of 16 rows per compute unit, 16 with a
-                                            single codebook of 8-vectors; M == 2: at most one; K <= 6144, K = 8192
-                                            between 4 and 8 tiles per unit) and VQGEMM_VARIANT_DECODE, the K-sliced
-                                            MFMA kernels, otherwise */
+#define VQGEMM_VARIANT_DECODE_GEMV 8     /* the GEMV kernels: whole rows of W per wave, no matrix core.  One row of X,
+                                            8-vectors with 8-bit codes, at most 256 entries, K a multiple of 2048 up
+                                            to 8192, at most 64 rows of W per wave of a 16-wave workgroup per compute
+                                            unit and at most two codebooks per workgroup: the wide form (AUTO takes it
+                                            from one row per wave on).  Otherwise the four-wave form: M <= 4 for that
+                                            format, M <= 2 for 4-vectors, 8-vectors with 16-bit codes and 2-vectors
+                                            with 8-bit codes; at most 256 resp. 4096 entries, entries * vec a multiple
+                                            of 8; K a multiple of 2048 with (K / 2048) * M <= 8, N and N / n_codebooks
+                                            multiples of 16.  AUTO takes it where it was measured faster than
+                                            VQGEMM_VARIANT_DECODE, the K-sliced MFMA kernels (the limits are constants
+                                            of the tuning table below) */
 
 /*
  * Fused VQ GEMM, geometry B.
@@ -92,11 +94,13 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
  *     y[m, 16g + r] = silu(P[m, 32g + r]) * P[m, 32g + 16 + r],   P = X . W^T (+ bias[n], indexed like the rows of W),
  * silu(t) = t / (1 + exp(-t)), everything in fp32 with one rounding to fp16: y is [M, N/2] and the [M, N] product
  * never exists in memory.  N % 32 == 0.  No counterpart in the reference (its storeC has no epilogue,
- * strategy_2/bsz128/src.cu:163-177).  The prefill kernels (variants 3, 5, 6), the wide GEMV kernel (variant 8: one
- * row of X) and the scalar kernel (variant 1) carry the epilogue; the K-sliced decode kernels do not:
- * VQGEMM_VARIANT_TWOPASS here means the plain product into `workspace` ([M, N] fp16) followed by the element-wise
- * pass, and VQGEMM_VARIANT_AUTO takes that route where the plain product would run a decode kernel and a
- * workspace is given (NULL: the prefill kernels or the scalar kernel take the shape after all).
+ * strategy_2/bsz128/src.cu:163-177).  The prefill kernels (variants 3, 5, 6), the batched K-sliced decode kernel
+ * (variant 2: K % 256 == 0, (N / n_codebooks) % 32 == 0, not 2-vectors with 16-bit codes), the wide GEMV kernel
+ * (variant 8: one row of X) and the scalar kernel (variant 1) carry the epilogue; the four-wave GEMV kernel and the
+ * general K-sliced kernel do not: VQGEMM_VARIANT_TWOPASS here means the plain product into `workspace` ([M, N]
+ * fp16) followed by the element-wise pass, and VQGEMM_VARIANT_AUTO takes that route where the plain product would
+ * run one of those two and a workspace is given (NULL: the batched decode, prefill or scalar kernel takes the shape
+ * after all).
  */
 int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebook, const void *bias, void *y,
                             int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
