@@ -363,7 +363,29 @@ def main():
                                                                                          spec.entries, 1, spec.code_bits)]}
             del pool, part, ysum
             torch.cuda.empty_cache()
-        print(json.dumps({"study": "split-k", "config": "C3", "slices": report}))
+        # The tiles of medium M: split K is built there (vqgemm_e2e_gemm_b_ws: 128x128 tiles, 2-8 workgroups per tile, the
+        # last one sums the partial products).  The automatic choice without and with a workspace, and the baselines.
+        tiles = {}
+        for M, K, N, G in ((256, 4096, 4096, 32), (384, 4096, 4096, 32), (512, 4096, 4096, 32), (768, 4096, 4096, 32),
+                           (256, 8192, 8192, 1), (512, 8192, 8192, 1), (256, 11008, 4096, 1), (2048, 4096, 1024, 8),
+                           (128, 8192, 4096, 1), (512, 4096, 11008, 1)):
+            tspec = ProblemSpec(f"m{M}_k{K}_n{N}", GEOM_B, M, K, N, 8, 256, G, 8)
+            x, codes, cb = make_problem(tspec, seed=42, device=dev)
+            y = torch.empty(M, N, dtype=torch.float16, device=dev)
+            need = cabi.workspace_bytes_b(M, K, N, 8, 256, G, 8)
+            ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+            wd = cabi.dequant_b(codes, cb)
+            t_plain = time_launches(lambda i: cabi.e2e_gemm_b(x, codes, cb, out=y), 1, 40, 10, min_launches=1)[0]
+            t_ws = time_launches(lambda i: cabi.e2e_gemm_b_ws(x, codes, cb, out=y, workspace=ws), 1, 40, 10, min_launches=1)[0]
+            t_blas = time_launches(lambda i: cabi.ref_gemm_f16(x, wd, w_is_nk=True, out=y), 1, 40, 10, min_launches=1)[0]
+            t_torch = time_launches(lambda i: torch.nn.functional.linear(x, wd), 1, 40, 10, min_launches=1)[0]
+            tiles[tspec.name] = {"n_codebooks": G, "without_workspace_us": t_plain * 1e6,
+                                 "without_workspace_variant": cabi.VARIANT_NAMES[cabi.select_variant_b(M, K, N, 8, 256, G, 8)],
+                                 "workspace_bytes_wanted": need, "with_workspace_us": t_ws * 1e6,
+                                 "hipblaslt_us": t_blas * 1e6, "torch_linear_us": t_torch * 1e6}
+            del x, codes, cb, y, ws, wd
+            torch.cuda.empty_cache()
+        print(json.dumps({"study": "split-k", "decode_C3_emulated": report, "tiles_medium_m": tiles}))
         return
 
     if args.study == "code-usage":

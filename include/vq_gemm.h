@@ -32,7 +32,8 @@ extern "C" {
 #define VQGEMM_E_CODEBITS (-3)  /* code_bits not 8/16, or entries > 2^code_bits */
 #define VQGEMM_E_VARIANT (-4)   /* unknown variant, or the variant cannot serve this shape */
 #define VQGEMM_E_ALIGN (-5)     /* a pointer is not aligned to its element size */
-#define VQGEMM_E_SCRATCH (-6)   /* the problem needs more scratch than the library's fixed device array holds */
+#define VQGEMM_E_SCRATCH (-6)   /* the problem needs more scratch than the library's fixed device array, or the
+                                   workspace that was passed with its size, holds */
 
 /* kernel selection for the fused GEMM */
 #define VQGEMM_VARIANT_AUTO 0     /* pick by shape */
@@ -62,6 +63,11 @@ extern "C" {
                                             VQGEMM_VARIANT_DECODE, the K-sliced MFMA kernels (the limits are constants
                                             of the tuning table below) */
 
+#define VQGEMM_VARIANT_PREFILL_SPLITK 9  /* vqgemm_e2e_gemm_b_ws only: the 128x128 tiles with K split over 2, 4 or 8
+                                            workgroups per tile (as many as the cost model expects to be fastest);
+                                            medium M on few columns, where whole tiles are fewer than the compute
+                                            units; fp32 partial sums through the workspace */
+
 /*
  * Fused VQ GEMM, geometry B.
  * Replaces: torch::Tensor e2e_gemm(input, w, codebook) — reference bind.cpp:3,7 and the host
@@ -85,6 +91,25 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
                            int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
                            int32_t n_codebooks, int32_t code_bits, int32_t variant,
                            void *workspace, void *stream);
+
+/*
+ * vqgemm_e2e_gemm_b_bias with a workspace whose size the library is told, so that the automatic choice may use
+ * kernels that need scratch memory: today split K (VQGEMM_VARIANT_PREFILL_SPLITK), which VQGEMM_VARIANT_AUTO takes
+ * where its cost model expects at least 10 % over what it would launch otherwise and `workspace_bytes` suffices
+ * (a workspace that is too small, or NULL, is no error for AUTO: it does without).  vqgemm_workspace_bytes_b says
+ * how many bytes the given variant (AUTO, PREFILL_SPLITK, TWOPASS) wants for a shape: 0 when it uses none, a
+ * negative error for an invalid shape.  `workspace` must be 256-byte aligned device memory; its contents before the
+ * call do not matter and are undefined after it; two calls that overlap in time need a workspace each.  An explicit
+ * variant with too small a workspace returns VQGEMM_E_SCRATCH.  The partial sums of a tile are added in the order
+ * of the slices of K whichever workgroup finishes last: results are the same from run to run.  No counterpart in
+ * the reference (one workgroup per tile over all of K, strategy_2/bsz128/src.cu:179-253).
+ */
+int vqgemm_e2e_gemm_b_ws(const void *x, const void *codes, const void *codebook, const void *bias, void *y,
+                         int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                         int32_t n_codebooks, int32_t code_bits, int32_t variant,
+                         void *workspace, int64_t workspace_bytes, void *stream);
+int64_t vqgemm_workspace_bytes_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,
+                                 int32_t n_codebooks, int32_t code_bits, int32_t variant);
 
 /*
  * The fused VQ GEMM with a gated epilogue, for a gate/up projection pair (the MLP shapes among the measured

@@ -1347,3 +1347,82 @@ def test_gated_mlp_module_with_interleaved_rows():
         # the stacked layout with the element-wise kernel computes the same layer
         ys = stacked(x)
         assert ((y.float() - ys.float()).abs().max() / ys.float().abs().max()).item() <= 2 * TOL
+
+
+# ------------------------------------------------------------------ split K over the 128x128 tiles
+SPLITK_B = [
+    # name, M, K, N, vec, E, bits, G
+    ("mid_m_few_columns", 512, 4096, 4096, 8, 256, 8, 32),      # the shape the cost model was fitted on
+    ("ragged_m_and_n", 300, 2048, 1000, 8, 256, 8, 1),          # Y rows not 16-byte aligned: the plain epilogue
+    ("u16_v4_books", 200, 1024, 768, 4, 4096, 16, 3),
+    ("v2", 129, 512, 256, 2, 256, 8, 1),
+    ("one_tile", 64, 4096, 128, 8, 256, 8, 1),
+    ("many_tiles", 1024, 1024, 2048, 8, 256, 8, 16),            # more workgroups than fit the device at once
+]
+
+
+@pytest.mark.parametrize("row", SPLITK_B, ids=[r[0] for r in SPLITK_B])
+def test_split_k_against_the_oracle_and_from_run_to_run(row):
+    name, M, K, N, v, E, bits, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1), codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=61, device=DEV)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(62)) * 0.5).half().to(DEV)
+    # (the unrounded float64 product: the bias is added before the one rounding)
+    want = _np(x).astype(np.float64) @ vo.dequant_b(_np(codes), _np(cb)).astype(np.float64).T
+    need = cabi.workspace_bytes_b(M, K, N, v, E, G, bits, cabi.VARIANT_PREFILL_SPLITK)
+    assert need > 0, "every shape of this list has a split"
+    # the workspace's contents before the call do not matter: start from garbage
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV).random_()
+    for b, ref in ((None, want), (bias, want + _np(bias).astype(np.float64)[None, :])):
+        _say("split-k", name, "bias" if b is not None else "")
+        y = cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws, bias=b).clone()
+        torch.cuda.synchronize()
+        e1, e2 = vo.rel_err(_np(y), ref)
+        _say(f"    rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+        assert e1 <= TOL, (name, e1, e2)
+        # the partial sums are added in the order of the slices whoever finishes last: the same bits every time
+        for _ in range(4):
+            ws.random_()
+            assert torch.equal(cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws, bias=b), y)
+    # and close to the unsplit kernel (the same fp32 products, summed in another order)
+    y1 = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_PREFILL_SMALL)
+    y2 = cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws)
+    assert vo.rel_err(_np(y2), _np(y1).astype(np.float64))[0] <= 2e-3
+    # a workspace that is too small: an error for the explicit variant, no obstacle for the automatic choice
+    small = torch.empty(256, dtype=torch.uint8, device=DEV)
+    with pytest.raises(cabi.VqGemmError) as err:
+        cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=small)
+    assert err.value.code == -6
+    ya = cabi.e2e_gemm_b_ws(x, codes, cb, workspace=small)
+    assert vo.rel_err(_np(ya), want)[0] <= TOL
+
+
+def test_split_k_is_what_the_automatic_choice_takes_for_medium_m_on_few_columns_and_only_with_a_workspace():
+    M, K, N = 512, 4096, 4096
+    spec = ProblemSpec("auto_split", GEOM_B, M, K, N, 8, 256, 32, 8, codebook_3d=True, codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=63, device=DEV)
+    need = cabi.workspace_bytes_b(M, K, N, 8, 256, 32, 8)
+    assert need > 0
+    want = vo.vq_gemm_b(_np(x), _np(codes), _np(cb), acc=np.float64)
+    y_plain = cabi.e2e_gemm_b(x, codes, cb)                      # no workspace: the unsplit choice
+    y_split = cabi.e2e_gemm_b_ws(x, codes, cb)                   # allocates what workspace_bytes_b says
+    assert vo.rel_err(_np(y_plain), want)[0] <= TOL and vo.rel_err(_np(y_split), want)[0] <= TOL
+    # where a split cannot pay the automatic choice wants no workspace: one row of X, a full device of large tiles
+    assert cabi.workspace_bytes_b(1, 4096, 4096, 8, 256, 1, 8) == 0 and cabi.workspace_bytes_b(14, 512, 768, 8, 256, 3, 8) == 0
+    assert cabi.workspace_bytes_b(4096, 4096, 4096, 8, 256, 32, 8) == 0
+    # captured into a graph and replayed (the counters are cleared by a kernel, not a memset node)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        cabi.e2e_gemm_b_ws(x, codes, cb, workspace=ws, out=out)
+        st.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            cabi.e2e_gemm_b_ws(x, codes, cb, workspace=ws, out=out)
+        for _ in range(3):
+            out.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            st.synchronize()
+            assert torch.equal(out, y_split)

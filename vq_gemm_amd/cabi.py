@@ -14,9 +14,9 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 _INCLUDE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
 
 (VARIANT_AUTO, VARIANT_GENERIC, VARIANT_DECODE, VARIANT_PREFILL, VARIANT_TWOPASS, VARIANT_PREFILL_NARROW,
- VARIANT_PREFILL_SMALL, VARIANT_DECODE_PACKED, VARIANT_DECODE_GEMV) = range(9)
+ VARIANT_PREFILL_SMALL, VARIANT_DECODE_PACKED, VARIANT_DECODE_GEMV, VARIANT_PREFILL_SPLITK) = range(10)
 VARIANT_NAMES = {0: "auto", 1: "generic", 2: "decode", 3: "prefill", 4: "twopass", 5: "prefill_narrow", 6: "prefill_small",
-                 7: "decode_packed", 8: "decode_gemv"}
+                 7: "decode_packed", 8: "decode_gemv", 9: "prefill_splitk"}
 
 _I64, _I32, _P = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p
 
@@ -24,6 +24,8 @@ _SIGNATURES = {
     "vqgemm_e2e_gemm_b": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_b_bias": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "vqgemm_e2e_gemm_b_gated": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
+    "vqgemm_e2e_gemm_b_ws": (ctypes.c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _I64, _P]),
+    "vqgemm_workspace_bytes_b": (_I64, [_I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32]),
     "vqgemm_e2e_gemm_a": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _P]),
     "vqgemm_e2e_gemm_a_noalloc": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P]),
     "vqgemm_dequant_b": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _I32, _I32, _I32, _I32, _P]),
@@ -213,6 +215,47 @@ def e2e_gemm_b(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=Non
                                           bits, variant, _ptr(workspace), _stream())
     if rc != 0:
         raise VqGemmError(rc, "vqgemm_e2e_gemm_b")
+    return out
+
+
+def workspace_bytes_b(M, K, N, vec, entries, n_codebooks, code_bits, variant=VARIANT_AUTO) -> int:
+    """Bytes of workspace `e2e_gemm_b_ws` would use for the shape with `variant` (0: none)."""
+    n = lib().vqgemm_workspace_bytes_b(M, K, N, vec, entries, n_codebooks, code_bits, variant)
+    if n < 0:
+        raise VqGemmError(int(n), "vqgemm_workspace_bytes_b")
+    return int(n)
+
+
+def e2e_gemm_b_ws(x, codes, codebook, variant=VARIANT_AUTO, out=None, workspace=None, bias=None):
+    """The fused GEMM with a sized workspace (a uint8 device tensor, 256-byte aligned as torch allocates it): lets the
+    automatic choice split K over several workgroups per tile where that pays (medium M, few columns).  With
+    `workspace=None` one of `workspace_bytes_b(...)` bytes is allocated when the variant wants one."""
+    import torch
+    _require(x.dim() == 2 and codes.dim() == 2, "x must be [M, K] and codes [N, K/vec]")
+    G, E, v = _check_codebook(codebook)
+    bits = _code_bits(codes)
+    M, K = x.shape
+    N = codes.shape[0]
+    _check_f16(x, (M, K), "x")
+    _require(codes.shape[1] * v == K, f"codes have {codes.shape[1]} columns of {v}-vectors but x has K = {K}")
+    _require(N % G == 0, "rows of codes must be a multiple of the number of codebooks")
+    if workspace is None:
+        need = workspace_bytes_b(M, K, N, v, E, G, bits, variant) if variant in (VARIANT_AUTO, VARIANT_TWOPASS, VARIANT_PREFILL_SPLITK) else 0
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    else:
+        _require(workspace.dtype == torch.uint8 and workspace.is_contiguous(), "workspace must be a contiguous uint8 tensor")
+    _same_device(x, codes, codebook, out, workspace, bias)
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    else:
+        _check_f16(out, (M, N), "out")
+    if bias is not None:
+        _check_f16(bias, (N,), "bias")
+    rc = lib().vqgemm_e2e_gemm_b_ws(_ptr(x), _ptr(codes), _ptr(codebook), _ptr(bias), _ptr(out), M, K, N, v, E, G, bits, variant,
+                                    _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream())
+    if rc != 0:
+        raise VqGemmError(rc, "vqgemm_e2e_gemm_b_ws")
     return out
 
 

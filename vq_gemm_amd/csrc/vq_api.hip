@@ -67,6 +67,9 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_max_tiles_per_cu", &Tuning::gemv_max_tiles_per_cu},
     {"gemv_max_k", &Tuning::gemv_max_k},
     {"gemv_wide_min_rows_per_wave", &Tuning::gemv_wide_min_rows_per_wave},
+    {"splitk_fixed_us", &Tuning::splitk_fixed_us},
+    {"splitk_us_per_partial_mb", &Tuning::splitk_us_per_partial_mb},
+    {"splitk_force_splits", &Tuning::splitk_force_splits},
 };
 constexpr int kTuningCount = (int)(sizeof(kTuningEntries) / sizeof(kTuningEntries[0]));
 
@@ -238,7 +241,7 @@ const char *vqgemm_error_string(int code)
     case VQGEMM_E_CODEBITS: return "code_bits must be 8 or 16 and entries <= 2^code_bits";
     case VQGEMM_E_VARIANT: return "unknown kernel variant, or the variant cannot serve this shape";
     case VQGEMM_E_ALIGN: return "pointer not aligned as the selected kernel requires";
-    case VQGEMM_E_SCRATCH: return "the problem needs more scratch than the library's fixed device array holds";
+    case VQGEMM_E_SCRATCH: return "the problem needs more scratch than the library's fixed device array, or the workspace passed with its size, holds";
     default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -320,6 +323,75 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
         return VQGEMM_E_VARIANT;
     }
     return static_cast<int>(e);
+}
+
+namespace {
+
+// Split K with the cost model's number of slices when that is expected to beat what the automatic choice would
+// launch otherwise by a margin (and then at least two slices); 0: do not split.
+int splitk_auto(const ProblemB &p, bool all_aligned16)
+{
+    if (p.K == 0 || !all_aligned16 || p.gated) return 0;
+    const int plain = select_b(p, all_aligned16);
+    double t_plain;
+    if (plain == VQGEMM_VARIANT_PREFILL) t_plain = prefill_cost_us(p);
+    else if (plain == VQGEMM_VARIANT_DECODE) t_plain = decode_cost_us(p);
+    else return 0;
+    if (t_plain >= 1e29) return 0;  // (short X: the decode path is taken without a comparison, and stays)
+    double t_split = 1e30;
+    const int sp = prefill_splitk_choice(p, &t_split, 2);
+    return sp >= 2 && t_split < 0.9 * t_plain ? sp : 0;
+}
+
+}  // namespace
+
+int64_t vqgemm_workspace_bytes_b(int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks,
+                                 int32_t code_bits, int32_t variant)
+{
+    const int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (M == 0 || N == 0 || K == 0) return 0;
+    const ProblemB p = make_b(nullptr, nullptr, nullptr, nullptr, M, K, N, vec, entries, n_codebooks, code_bits);
+    if (variant == VQGEMM_VARIANT_TWOPASS) return N * K * 2;
+    int sp = 0;
+    if (variant == VQGEMM_VARIANT_AUTO) sp = splitk_auto(p, true);
+    else if (variant == VQGEMM_VARIANT_PREFILL_SPLITK) sp = prefill_splitk_choice(p, nullptr, 2);
+    return sp >= 2 ? (int64_t)prefill_splitk_workspace_bytes(p, sp) : 0;
+}
+
+int vqgemm_e2e_gemm_b_ws(const void *x, const void *codes, const void *codebook, const void *bias, void *y, int64_t M,
+                         int64_t K, int64_t N, int32_t vec, int32_t entries, int32_t n_codebooks, int32_t code_bits,
+                         int32_t variant, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return VQGEMM_E_NULL;
+    if (variant == VQGEMM_VARIANT_TWOPASS) {
+        if (workspace_bytes < N * K * 2) return VQGEMM_E_SCRATCH;
+        return vqgemm_e2e_gemm_b_bias(x, codes, codebook, bias, y, M, K, N, vec, entries, n_codebooks, code_bits, variant, workspace, stream);
+    }
+    if (variant != VQGEMM_VARIANT_AUTO && variant != VQGEMM_VARIANT_PREFILL_SPLITK)
+        return vqgemm_e2e_gemm_b_bias(x, codes, codebook, bias, y, M, K, N, vec, entries, n_codebooks, code_bits, variant, nullptr, stream);
+    int rc = check_b(M, K, N, vec, entries, n_codebooks, code_bits);
+    if (rc != VQGEMM_OK) return rc;
+    if (M == 0 || N == 0) return VQGEMM_OK;
+    if (!y || !codebook || (K > 0 && (!x || !codes))) return VQGEMM_E_NULL;
+    const bool a16 = aligned(x, 16) && aligned(y, 16) && aligned(codebook, 16) && aligned(codes, 16) && aligned(bias, 8) &&
+                     aligned(workspace, 256);
+    ProblemB p = make_b(x, codes, codebook, y, M, K, N, vec, entries, n_codebooks, code_bits);
+    p.bias = static_cast<const half_t *>(bias);
+    int sp;
+    if (variant == VQGEMM_VARIANT_PREFILL_SPLITK) {
+        if (!a16) return VQGEMM_E_ALIGN;
+        sp = K > 0 ? prefill_splitk_choice(p, nullptr, 2) : 0;
+        if (sp < 2) return VQGEMM_E_VARIANT;
+        if ((int64_t)prefill_splitk_workspace_bytes(p, sp) > workspace_bytes) return VQGEMM_E_SCRATCH;
+    } else {
+        sp = splitk_auto(p, a16);
+        // (a workspace that is too small is not an error for the automatic choice: it does without)
+        if (sp < 2 || (int64_t)prefill_splitk_workspace_bytes(p, sp) > workspace_bytes)
+            return vqgemm_e2e_gemm_b_bias(x, codes, codebook, bias, y, M, K, N, vec, entries, n_codebooks, code_bits, VQGEMM_VARIANT_AUTO,
+                                          nullptr, stream);
+    }
+    return static_cast<int>(launch_prefill_small_b(p, static_cast<hipStream_t>(stream), sp, workspace));
 }
 
 int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebook, const void *bias, void *y, int64_t M,

@@ -12,6 +12,11 @@ namespace {
 
 __global__ __launch_bounds__(64) void clear_word_kernel(uint32_t *out) { if (threadIdx.x == 0) *out = 0u; }
 
+__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t *out, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) out[i] = 0u;
+}
+
 // 16-byte loads over the aligned body, scalar loads for the ragged head and tail.
 template <typename CodeT>
 __global__ __launch_bounds__(256) void max_code_kernel(const CodeT *__restrict__ codes, int64_t count, uint32_t *out)
@@ -43,6 +48,15 @@ __global__ __launch_bounds__(256) void max_code_kernel(const CodeT *__restrict__
 }
 
 }  // namespace
+
+hipError_t launch_clear_words(uint32_t *words, int64_t n, hipStream_t s)
+{
+    if (n <= 0) return hipSuccess;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 64) blocks = 64;
+    hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)blocks), dim3(256), 0, s, words, n);
+    return hipGetLastError();
+}
 
 hipError_t launch_max_code(const void *codes, int64_t count, int code_bits, uint32_t *out, hipStream_t s)
 {

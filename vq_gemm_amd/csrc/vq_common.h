@@ -109,6 +109,8 @@ hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);
 
 // whether the batched K-sliced decode kernel takes the shape with its gated epilogue (p.gated set)
 bool decode_gated_supports(const ProblemB &p);
+// expected microseconds of the batched decode kernel for tall X (more rows than the general kernel serves); 1e30 otherwise
+double decode_cost_us(const ProblemB &p);
 
 bool prefill_supports(const ProblemB &p);
 // whether the 256x128 tile of the prefill kernel can serve the shape (a subset of prefill_supports)
@@ -122,7 +124,14 @@ hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile = 0);
 // the prefill kernel with 128x128 tiles (vq_prefill_small.hip), for medium M
 bool prefill_small_supports(const ProblemB &p);
 double prefill_small_cost_us(const ProblemB &p);  // expected time, microseconds (1e30: not supported)
-hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s);
+// splits > 1: split K, `splits` workgroups per tile (workspace of prefill_splitk_workspace_bytes, device memory)
+hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s, int splits = 1, void *workspace = nullptr);
+bool prefill_splitk_supports(const ProblemB &p, int splits);
+size_t prefill_splitk_counter_bytes(int64_t tiles);
+size_t prefill_splitk_workspace_bytes(const ProblemB &p, int splits);
+// slices of K the cost model expects to be fastest with 128x128 tiles and the time it expects (min_splits 1: none is a
+// candidate; 2: the best split); 0 when no split applies
+int prefill_splitk_choice(const ProblemB &p, double *cost_us, int min_splits = 1);
 
 // o[M,N] = x[M,K] . w[K,N]
 hipError_t launch_gemm_nn(const half_t *x, const half_t *w, half_t *y, int M, int K, int N, hipStream_t s);
@@ -144,6 +153,8 @@ hipError_t launch_silu_mul(const half_t *a, half_t *out, int64_t M, int64_t N, h
 
 // out[0] = the largest code of codes[0 .. count) (0 when count == 0); out is device memory
 hipError_t launch_max_code(const void *codes, int64_t count, int code_bits, uint32_t *out, hipStream_t s);
+// words[0 .. n) = 0, by a kernel (a launch that may be captured into a graph records no memset)
+hipError_t launch_clear_words(uint32_t *words, int64_t n, hipStream_t s);
 
 int device_cu_count();
 
@@ -171,6 +182,12 @@ struct Tuning {
     double gemv_max_tiles_per_cu = 4.0;
     double gemv_max_k = 6144.0;
     double gemv_wide_min_rows_per_wave = 1.0;
+    // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums
+    // written and read once (microseconds per MB of partial sums)
+    double splitk_fixed_us = 2.0;
+    double splitk_us_per_partial_mb = 0.25;
+    // 2, 4 or 8: VQGEMM_VARIANT_PREFILL_SPLITK takes this many slices where the shape allows (for measurements); 0: the cost model's
+    double splitk_force_splits = 0.0;
 };
 const Tuning &tuning();
 

@@ -842,10 +842,10 @@ bool decode_supports(const ProblemB &p)
 //                 resident run in further rounds.  With K of 2048 or less two workgroups share a
 //                 compute unit: prologue 8, and a tile then costs each of them 1.0 us per 2048 k;
 //   prefill       the prefill kernels' own estimate for the tiles they would choose.
-bool decode_preferred(const ProblemB &p)
+// microseconds the batched decode kernel is expected to take on a shape it supports (M above what the general
+// kernel serves: below that the decode path is taken without a comparison)
+static double batched_cost_us(const ProblemB &p)
 {
-    if (!decode_supports(p)) return false;
-    if (p.M <= kGeneralMaxM) return true;
     const BatchedPlan g = plan_batched(p);
     const int cus = device_cu_count();
     const int per_slab = g.books_per_wg > 1 ? (p.n_codebooks + g.books_per_wg - 1) / g.books_per_wg : g.wgs_per_cb * p.n_codebooks;
@@ -854,10 +854,22 @@ bool decode_preferred(const ProblemB &p)
     const Tuning &tn = tuning();
     const double t_tile = (g.n_chunks == 1 ? tn.decode_tile_us : tn.decode_tile_chunked_us) * g.n_waves / kMaxWaves * g.per_cu * (shared ? 1.35 : 1.0);
     const int passes = g.books_per_wg * g.n_chunks;
-    const double t_decode = rounds_d * ((shared ? tn.decode_prologue_shared_cu_us : tn.decode_prologue_us) + passes * g.tiles_per_wg * t_tile +
-                                        (passes - 1) * tn.decode_pass_change_us);
+    return rounds_d * ((shared ? tn.decode_prologue_shared_cu_us : tn.decode_prologue_us) + passes * g.tiles_per_wg * t_tile +
+                       (passes - 1) * tn.decode_pass_change_us);
+}
+
+bool decode_preferred(const ProblemB &p)
+{
+    if (!decode_supports(p)) return false;
+    if (p.M <= kGeneralMaxM) return true;
     const double t_prefill = prefill_supports(p) ? 1.0 + prefill_cost_us(p) : 1e30;
-    return t_decode <= t_prefill;
+    return batched_cost_us(p) <= t_prefill;
+}
+
+double decode_cost_us(const ProblemB &p)
+{
+    if (!decode_supports(p) || p.M <= kGeneralMaxM || !batched_supports(p)) return 1e30;
+    return batched_cost_us(p);
 }
 
 // The GEMV kernels have no work shared between their waves.  One row of X in the first format

@@ -17,6 +17,12 @@
 // the buffer of stage-1, into which the loads of stage+3 go.
 //
 // K must be a multiple of the k one code tile covers (64, or 128 for 8-vectors with 8-bit codes).
+//
+// Split K.  Where even these tiles are fewer than the compute units, `splits` workgroups share a tile, each
+// multiplying k_len = K / splits of K.  Nothing waits for anything: a workgroup writes its fp32 sums to a partial
+// buffer with device-scope stores, waits for them, and counts itself in on the tile's counter; the one that
+// finds itself last adds the partial sums up in the order of the slices and runs the epilogue.  The sum is the same whoever comes last, so
+// results do not depend on the order in which the workgroups finish.
 #include "vq_prefill_common.h"
 
 #include <type_traits>
@@ -46,7 +52,9 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                                                                     half_t *__restrict__ y,
                                                                     const half_t *__restrict__ bias, int M, int K,
                                                                     int N, int entries, int rows_per_cb, int tiles_m,
-                                                                    int tiles_n, int cb_lds_count, int gated)
+                                                                    int tiles_n, int cb_lds_count, int gated, int k_len,
+                                                                    int splits, float4_t *__restrict__ partials,
+                                                                    unsigned int *__restrict__ counters)
 {
     typedef PrefillCfg<VEC, CodeT> C;
     constexpr int D = NS - 1;                 // loads run D stages ahead
@@ -65,12 +73,14 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
 
     // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: re-number them so
     // that an XCD works on consecutive tiles of the row-band-major order.
-    int wg = blockIdx.x;
+    // (with split K the slices of a tile lie n_wg workgroup ids apart: a multiple of 8 whenever the re-numbering applies)
     const int n_wg = tiles_m * tiles_n;
+    const int split = (int)blockIdx.x / n_wg;
+    int wg = (int)blockIdx.x - split * n_wg;
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
     const int tm = wg / tiles_n, tn = wg % tiles_n;
     const int m0 = tm * SBM, n0 = tn * SBN;
-    const int n_stage = K / kStageK;
+    const int n_stage = k_len / kStageK;
     const int n_super = n_stage / C::STAGES;
 
     // ---- per-lane codebook bases ------------------------------------------------------------
@@ -98,14 +108,14 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
         const int row = 2 * bank_row + (v >> 3), cc = v & 7;
         x_voff[i] = (uint32_t)(((int64_t)(min(m0 + row, M - 1) - m0) * K + cc * 8) * 2);
     }
-    const half_t *x_tile = x + (int64_t)m0 * K;
+    const half_t *x_tile = x + (int64_t)m0 * K + (int64_t)split * k_len;
     // X load i (0..3) of a stage that starts at `xb` into buffer `buf`.
     auto issue_x = [&](int i, int buf, const half_t *xb) {
         load_to_lds_16(buf * kSmallStage + (4 * i + wave) * 1024, x_voff[i], xb);
     };
     // The code tile has 128 rows, two waves' worth: the waves of the lower half of the tile load
     // the same chunks to the same place again, which keeps every wave's load count the same.
-    const uint8_t *code_tile = reinterpret_cast<const uint8_t *>(codes + (int64_t)n0 * J);
+    const uint8_t *code_tile = reinterpret_cast<const uint8_t *>(codes + (int64_t)n0 * J + (int64_t)split * (k_len / VEC));
     uint32_t code_voff[C::CH];
 #pragma unroll
     for (int c = 0; c < C::CH; c++) code_voff[c] = (uint32_t)(min(wn * 64 + lane, N - 1 - n0) * J * C::CSZ) + c * 16;
@@ -280,6 +290,55 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
     // the last MFMAs must have left the pipe before the accumulators are read
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
+    // ---- split K: partial sums out, and the workgroup that comes last adds them up -------------------
+    // The partial sums are written and read with device-scope memory instructions (sc1: through the L2 of the
+    // XCD, which is not coherent with the other seven), and the waits are written out: a release / acquire fence
+    // of device scope would write back and invalidate the whole L2 under the workgroups that are still multiplying
+    // (measured: 3 us per MB of partial sums).  A store is complete, and visible device-wide, when the counter
+    // has counted it; the count itself is a relaxed device-scope atomic; the loads of the last workgroup are issued
+    // behind the barrier that follows its count.
+    if (splits > 1) {
+        // partial sums of (tile, slice): half h (two floats) of accumulator (j, i) of thread tid at
+        // [((j * SMP + i) * 2 + h) * 256 + tid], moved as 64-bit words (the widest scoped access there is)
+        constexpr int kPartial = SNP * SMP * 2 * kThreads;  // 64-bit words per tile and slice
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        uint64_t *tile_partials = reinterpret_cast<uint64_t *>(partials) + (int64_t)wg * splits * kPartial;
+        uint64_t *mine = tile_partials + (int64_t)split * kPartial + tid;
+#pragma unroll
+        for (int j = 0; j < SNP; j++)
+#pragma unroll
+            for (int i = 0; i < SMP; i++)
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    __hip_atomic_store(mine + ((j * SMP + i) * 2 + h) * kThreads,
+                                       __builtin_bit_cast(uint64_t, float2_t{acc[j][i][2 * h], acc[j][i][2 * h + 1]}), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        uint32_t *flag = reinterpret_cast<uint32_t *>(smem);
+        if (tid == 0) *flag = __hip_atomic_fetch_add(counters + wg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const bool last = *flag == (uint32_t)(splits - 1);
+        __syncthreads();  // the flag's word belongs to the epilogue's staging area again
+        if (!last) return;
+        // The sum in the order of the slices, whoever is last - this workgroup's own sums are read back like the
+        // others' (the same bits it wrote; its registers are free for the loads that way).
+        for (int sl = 0; sl < splits; sl++) {
+            const uint64_t *src = tile_partials + (int64_t)sl * kPartial + tid;
+#pragma unroll
+            for (int j = 0; j < SNP; j++)
+#pragma unroll
+                for (int i = 0; i < SMP; i++)
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const float2_t v = __builtin_bit_cast(
+                            float2_t, __hip_atomic_load(src + ((j * SMP + i) * 2 + h) * kThreads, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                        acc[j][i][2 * h] = sl == 0 ? v[0] : acc[j][i][2 * h] + v[0];
+                        acc[j][i][2 * h + 1] = sl == 0 ? v[1] : acc[j][i][2 * h + 1] + v[1];
+                    }
+        }
+    }
+
     // ---- epilogue: lane holds Y[m = i*16 + r16][n = j*16 + 4*kg + 0..3] of its 64x64 wave tile ----
     auto epilogue = [&](auto has_bias_const) {
         constexpr bool HB = decltype(has_bias_const)::value;
@@ -356,11 +415,25 @@ bool small_cfg_supports(const ProblemB &p)
            (int64_t)SBM * p.K * 2 < ((int64_t)1 << 32);
 }
 
+// float4 slots of partial sums per tile and slice, and where the tiles' counters start inside the workspace
+constexpr size_t kPartialBytes = (size_t)SNP * SMP * kThreads * 16;  // 64 KB
+
 template <int VEC, typename CodeT>
-hipError_t launch_small_typed(const ProblemB &p, hipStream_t s)
+hipError_t launch_small_typed(const ProblemB &p, hipStream_t s, int splits, void *workspace)
 {
+    typedef PrefillCfg<VEC, CodeT> C;
     if (!small_cfg_supports<VEC, CodeT>(p)) return hipErrorInvalidValue;
+    if (splits < 1 || p.K % splits != 0 || (p.K / splits) % C::K_SUPER != 0 || (splits > 1 && !workspace)) return hipErrorInvalidValue;
     const int tiles_m = (p.M + SBM - 1) / SBM, tiles_n = (p.N + SBN - 1) / SBN;
+    // workspace: the tiles' counters (cleared here, by a kernel: the launch may be captured), then the partial sums
+    unsigned int *counters = static_cast<unsigned int *>(workspace);
+    float4_t *partials = nullptr;
+    if (splits > 1) {
+        const size_t counter_bytes = prefill_splitk_counter_bytes(tiles_m * tiles_n);
+        partials = reinterpret_cast<float4_t *>(static_cast<uint8_t *>(workspace) + counter_bytes);
+        const hipError_t e = launch_clear_words(counters, tiles_m * tiles_n, s);
+        if (e != hipSuccess) return e;
+    }
     const size_t smem = lds_bytes_small<VEC, CodeT>(p, 4);
     // the split codebook layout is built out of a copy in the last X buffer
     constexpr bool can_split = VEC == 8 && sizeof(CodeT) == 1;
@@ -368,9 +441,9 @@ hipError_t launch_small_typed(const ProblemB &p, hipStream_t s)
     auto kern = split ? prefill_small_kernel<VEC, CodeT, 4, can_split> : prefill_small_kernel<VEC, CodeT, 4, false>;
     const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), smem, s, p.x,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads), smem, s, p.x,
                        static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
-                       tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0);
+                       tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0, p.K / splits, splits, partials, counters);
     return hipGetLastError();
 }
 
@@ -406,15 +479,71 @@ double prefill_small_cost_us(const ProblemB &p)
            (double)rounds * (p.K / 64.0 * (tn.prefill_small_stage_us_idle + (tn.prefill_small_stage_us_busy - tn.prefill_small_stage_us_idle) * busy));
 }
 
-hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s)
+hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s, int splits, void *workspace)
 {
     if (!prefill_small_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
-    case 8: return u8 ? launch_small_typed<8, uint8_t>(p, s) : launch_small_typed<8, uint16_t>(p, s);
-    case 4: return u8 ? launch_small_typed<4, uint8_t>(p, s) : launch_small_typed<4, uint16_t>(p, s);
-    default: return launch_small_typed<2, uint8_t>(p, s);
+    case 8: return u8 ? launch_small_typed<8, uint8_t>(p, s, splits, workspace) : launch_small_typed<8, uint16_t>(p, s, splits, workspace);
+    case 4: return u8 ? launch_small_typed<4, uint8_t>(p, s, splits, workspace) : launch_small_typed<4, uint16_t>(p, s, splits, workspace);
+    default: return launch_small_typed<2, uint8_t>(p, s, splits, workspace);
     }
+}
+
+// the k one code tile of the format covers: a slice of K is whole code tiles
+static int small_k_super(const ProblemB &p)
+{
+    const int csz = p.code_bits / 8;
+    const int kc = (16 / csz) * p.vec;
+    return kc > kStageK ? kc : kStageK;
+}
+
+size_t prefill_splitk_counter_bytes(int64_t tiles) { return ((size_t)tiles * 4 + 255) & ~(size_t)255; }
+
+size_t prefill_splitk_workspace_bytes(const ProblemB &p, int splits)
+{
+    if (splits <= 1) return 0;
+    const int64_t tiles = (int64_t)((p.M + SBM - 1) / SBM) * ((p.N + SBN - 1) / SBN);
+    return prefill_splitk_counter_bytes(tiles) + (size_t)tiles * splits * kPartialBytes;
+}
+
+bool prefill_splitk_supports(const ProblemB &p, int splits)
+{
+    return splits >= 2 && splits <= 8 && prefill_small_supports(p) && p.K % splits == 0 && (p.K / splits) % small_k_super(p) == 0 &&
+           p.K / splits >= 2 * small_k_super(p);
+}
+
+// The number of slices of K (1: none) that the cost model expects to be fastest with 128x128 tiles, and its time.
+// A slice is a workgroup of its own: `splits` times the tiles, each over K / splits; on top of that the clearing launch
+// and, per tile, the partial sums written and read once (Tuning::splitk_fixed_us, splitk_us_per_partial_mb).
+int prefill_splitk_choice(const ProblemB &p, double *cost_us, int min_splits)
+{
+    int best = min_splits <= 1 ? 1 : 0;
+    double best_us = min_splits <= 1 ? prefill_small_cost_us(p) : 1e30;
+    const Tuning &tn = tuning();
+    const int64_t tiles = (int64_t)((p.M + SBM - 1) / SBM) * ((p.N + SBN - 1) / SBN);
+    if (min_splits >= 2 && tn.splitk_force_splits >= 2.0 && prefill_splitk_supports(p, (int)tn.splitk_force_splits)) {
+        if (cost_us) *cost_us = 0.0;
+        return (int)tn.splitk_force_splits;
+    }
+    for (int sp = 2; sp <= 8; sp *= 2) {
+        if (!prefill_splitk_supports(p, sp)) break;
+        ProblemB q = p;  // the slices as the kernel sees them: sp times the tiles over K / sp
+        q.K = p.K / sp;
+        const int cus = device_cu_count();
+        const int64_t wgs = tiles * sp;
+        const int64_t rounds = (wgs + cus - 1) / cus, resident_rounds = (wgs + 2 * cus - 1) / (2 * cus);
+        const double busy = wgs >= cus ? 1.0 : (double)wgs / cus;
+        const double main_us = (double)resident_rounds * tn.prefill_small_tile_fixed_us +
+                               (double)rounds * (q.K / 64.0 * (tn.prefill_small_stage_us_idle + (tn.prefill_small_stage_us_busy - tn.prefill_small_stage_us_idle) * busy));
+        const double fix_us = tn.splitk_fixed_us + tn.splitk_us_per_partial_mb * (double)(wgs * kPartialBytes) / 1e6;
+        if (main_us + fix_us < best_us) {
+            best_us = main_us + fix_us;
+            best = sp;
+        }
+    }
+    if (cost_us) *cost_us = best_us;
+    return best;
 }
 
 }  // namespace vq

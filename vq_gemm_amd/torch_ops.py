@@ -34,7 +34,8 @@ def vq_linear(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor,
     if x.dtype != torch.float16 or codebook.dtype != torch.float16:
         raise ValueError("vq_linear: x and codebook must be float16")
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
-    y = cabi.e2e_gemm_b(x2, codes.contiguous(), codebook.contiguous(), bias=None if bias is None else bias.contiguous())
+    # (the entry point with a sized workspace: allocated only for the shapes whose automatic choice wants one - split K)
+    y = cabi.e2e_gemm_b_ws(x2, codes.contiguous(), codebook.contiguous(), bias=None if bias is None else bias.contiguous())
     return y.view(shape)
 
 

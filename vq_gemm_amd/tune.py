@@ -70,11 +70,21 @@ def tune(M: int, K: int, N: int, vec: int = 8, entries: int = 256, n_codebooks: 
         except cabi.VqGemmError as e:
             if e.code != -4:   # anything but "this variant does not take the shape"
                 raise
+    # split K over the 128x128 tiles, and the automatic choice when it is given a workspace to split K with
+    need = cabi.workspace_bytes_b(M, K, N, vec, entries, n_codebooks, code_bits, cabi.VARIANT_PREFILL_SPLITK)
+    if need > 0:
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        times[cabi.VARIANT_PREFILL_SPLITK] = time_graph(
+            lambda: cabi.e2e_gemm_b_ws(x, codes, cb, out=y, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws))
+    auto_need = cabi.workspace_bytes_b(M, K, N, vec, entries, n_codebooks, code_bits)
     w = cabi.dequant_b(codes, cb)
     t_lib = time_graph(lambda: cabi.ref_gemm_f16(x, w, w_is_nk=True, out=y))
     picked = cabi.select_variant_b(M, K, N, vec, entries, n_codebooks, code_bits)
     forced = {v: t for v, t in times.items() if v != cabi.VARIANT_AUTO}
     fastest = min(forced, key=forced.get)
+    if auto_need > 0:   # with a workspace the automatic choice splits K here
+        picked = cabi.VARIANT_PREFILL_SPLITK
+        times[cabi.VARIANT_AUTO] = times[cabi.VARIANT_PREFILL_SPLITK]
     result = {"times_us": {cabi.VARIANT_NAMES[v]: t for v, t in times.items()}, "auto_picks": cabi.VARIANT_NAMES[picked],
               "fastest": cabi.VARIANT_NAMES[fastest], "auto_over_fastest": times[cabi.VARIANT_AUTO] / forced[fastest],
               "hipblaslt_us": t_lib}
