@@ -253,6 +253,10 @@ GEMV_B = [
     ("wide_128_row_books_straddled", 4096, 6144, 256, 48, 1),
     ("wide_128_row_books_aligned", 2048, 8192, 200, 64, 1),
     ("wide_four_runs_two_books", 8192, 4096 + 32, 256, 2, 1),
+    # the wide form on its plain table (a wave's rows are at most two runs of 2048 k): two tables, short codebooks, ragged rows
+    ("wide_plain_table_books_straddled", 2048, 3 * 2000, 256, 3, 1),
+    ("wide_plain_table_short_books", 4096, 4096, 77, 4, 1),
+    ("wide_plain_table_ragged", 2048, 7001, 256, 1, 1),
     ("many_tiles_three_runs_ragged_walk", 6144, 16 * 1500, 256, 1, 1),
     ("many_tiles_one_run", 2048, 65536, 77, 1, 1),
     ("two_rows_of_x", 4096, 4096, 256, 1, 2),

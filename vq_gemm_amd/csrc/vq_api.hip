@@ -67,6 +67,7 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_max_tiles_per_cu", &Tuning::gemv_max_tiles_per_cu},
     {"gemv_max_k", &Tuning::gemv_max_k},
     {"gemv_wide_min_rows_per_wave", &Tuning::gemv_wide_min_rows_per_wave},
+    {"gemv_wide_plain_table_max_runs", &Tuning::gemv_wide_plain_table_max_runs},
     {"splitk_fixed_us", &Tuning::splitk_fixed_us},
     {"splitk_us_per_partial_mb", &Tuning::splitk_us_per_partial_mb},
     {"splitk_force_splits", &Tuning::splitk_force_splits},

@@ -182,6 +182,9 @@ struct Tuning {
     double gemv_max_tiles_per_cu = 4.0;
     double gemv_max_k = 6144.0;
     double gemv_wide_min_rows_per_wave = 1.0;
+    // the wide form gathers from the plain 4 KB table while a wave's rows are at most this many runs of 2048 k, from the
+    // bank-replicated one (64 KB to fill) beyond
+    double gemv_wide_plain_table_max_runs = 2.0;
     // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums
     // written and read once (microseconds per MB of partial sums)
     double splitk_fixed_us = 2.0;

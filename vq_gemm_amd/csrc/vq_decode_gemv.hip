@@ -265,7 +265,10 @@ __device__ __forceinline__ int small_quotient(int x, int d, float rcp)
 // landed: the table entry and the piece of x (both out of the L2) go out first, the code loads right
 // behind them.  And a launch starts with a cold instruction cache, so every instruction ahead of these
 // loads delays the one wait that cannot be shortened: nothing is computed ahead of them that they do not need.
-template <int RUNS, int G, int NBUF, int BOOKS>
+//
+// COPIES: 16 = the bank-replicated table (conflict-free gathers; 64 KB to fill), 1 = the plain 4 KB table (a wave
+// with one or two rows gathers too little for the fill of the replicated table to pay).
+template <int RUNS, int G, int NBUF, int BOOKS, int COPIES>
 __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const half_t *__restrict__ x,
                                                                            const uint8_t *__restrict__ codes,
                                                                            const half_t *__restrict__ cb,
@@ -283,7 +286,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     constexpr int kXChunks = RUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
     // permute) | table of the second one (TWO) | x
-    constexpr int kTableSlots = (TWO ? 2 : 1) * 256 * kWideCopies;
+    static_assert(COPIES == kWideCopies || COPIES == 1, "replicated or plain table");
+    constexpr int kTableSlots = (TWO ? 2 : 1) * 256 * COPIES;
     __shared__ __align__(16) uint4_t lds[kTableSlots + kXChunks];
     uint4_t *table = lds, *xs = lds + kTableSlots;
     // All kernel arguments are fetched at once: left to first use, each pointer costs the prologue a
@@ -373,11 +377,17 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         // served together to sixteen different copies (bank groups).  Entries past a short codebook are zeros,
         // so any 8-bit code gathers a defined value.
         if (e >= entries) entry0 = entry1 = uint4_t{0u, 0u, 0u, 0u};
+        if constexpr (COPIES == 1) {
+            // (the plain table: the first table's entry from the thread's even twin, the second table's from the odd one)
+            if (half_of_copies == 0) table[e] = entry0;
+            else if (second_table) table[256 + e] = entry1;
+        } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) table[e * kWideCopies + half_of_copies * 8 + ((e + i) & 7)] = entry0;
-        if (second_table) {
+            for (int i = 0; i < 8; i++) table[e * kWideCopies + half_of_copies * 8 + ((e + i) & 7)] = entry0;
+            if (second_table) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) table[256 * kWideCopies + e * kWideCopies + half_of_copies * 8 + ((e + i) & 7)] = entry1;
+                for (int i = 0; i < 8; i++) table[256 * kWideCopies + e * kWideCopies + half_of_copies * 8 + ((e + i) & 7)] = entry1;
+            }
         }
     } else {
         // x: piece i = q*256 + 4*l + c (the 8 halves that code c of lane l's dword in run q meets) is kept at
@@ -410,7 +420,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
         for (int r = 0; r < R; r++) {
             acc[r] = 0.f;
-            base[r] = TWO ? copy_base | (code_row(g * G + r) >= second_book_row ? 0x10000u : 0u) : copy_base;
+            if constexpr (COPIES == 1) base[r] = TWO && code_row(g * G + r) >= second_book_row ? 4096u : 0u;
+            else base[r] = TWO ? copy_base | (code_row(g * G + r) >= second_book_row ? 0x10000u : 0u) : copy_base;
         }
 #pragma unroll
         for (int q = 0; q < RUNS; q++) {
@@ -421,7 +432,9 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
                     // result bytes: 0 = byte 0 of the base, 1 = byte c of the codes, 2 = byte 2 of the base, 3 = zero
-                    const uint32_t addr = __builtin_amdgcn_perm(cur[r][q], base[r], 0x0c020000u | ((4u + c) << 8));
+                    // (plain table: code * 16 behind the table's offset)
+                    const uint32_t addr = COPIES == 1 ? (((cur[r][q] >> (8 * c)) & 0xffu) << 4) + base[r]
+                                                      : __builtin_amdgcn_perm(cur[r][q], base[r], 0x0c020000u | ((4u + c) << 8));
                     w[r][c] = *reinterpret_cast<const uint4_t *>(tbl + addr);
                 }
 #pragma unroll
@@ -533,10 +546,18 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
                            p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, n_dealt, p.gated ? 1 : 0);
         return hipGetLastError();
     };
+    // The plain table while a wave gathers for at most Tuning::gemv_wide_plain_table_max_runs runs of 2048 k (8 gathers per
+    // lane and run): measured cold, plain -> replicated, K = 4096: one row per wave 3.29 -> 3.43 us, two rows
+    // 4.07 -> 3.89; K = 2048, one row 2.93 -> 3.12; K = 8192, one row 4.26 -> 4.02.
+    const int code_rows_per_wave = (int)((p.N + waves - 1) / waves);
+    const bool plain_table = (double)code_rows_per_wave * (double)(p.K / kRunK) <= tuning().gemv_wide_plain_table_max_runs;
     auto pick = [&](auto runs_c, auto g_c, auto nbuf_c) {
         constexpr int R = decltype(runs_c)::value, GG = decltype(g_c)::value, NB = decltype(nbuf_c)::value;
-        return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, NB, 0>)
-             : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1>) : launch(decode_gemv_wide_kernel<R, GG, NB, 2>);
+        if (plain_table)
+            return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, NB, 0, 1>)
+                 : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1, 1>) : launch(decode_gemv_wide_kernel<R, GG, NB, 2, 1>);
+        return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, NB, 0, kWideCopies>)
+             : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1, kWideCopies>) : launch(decode_gemv_wide_kernel<R, GG, NB, 2, kWideCopies>);
     };
     using std::integral_constant;
     switch (p.K / kRunK) {
