@@ -42,8 +42,8 @@ EVICT_BYTES = 512 << 20  # source and destination of the device copy that emptie
 MIN_TIMED_LAUNCHES = 200  # a microsecond-scale kernel is never timed over fewer launches than this
 # HBM bytes one cold decode launch moves: NOT measured by this program.  From rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE of `bench.py --probe C2`, scaled by a 256 MiB copy in the same run
-# (1108.6 KiB x 2.0 read + 8 KiB written); the summary and its command are in the file named here.
-PROFILED_C2_HBM_BYTES_PER_LAUNCH = 2_278_400
+# (1104.1 KiB x 2.0 read + 8 KiB written); the summary and its command are in the file named here.
+PROFILED_C2_HBM_BYTES_PER_LAUNCH = 2_269_389
 PROFILED_C2_TRAFFIC_SOURCE = "profiles/decode_gemv_wide_kernel_c2_decode_gemv.md"
 
 
