@@ -885,6 +885,8 @@ def test_tune_fit_measures_plausible_constants_and_the_library_takes_them():
     assert 0.2 <= fitted["prefill_stage_us_256x256"] <= 4.0 and 0.1 <= fitted["prefill_stage_us_256x128"] <= 3.0
     assert 0.1 <= fitted["prefill_small_stage_us_idle"] <= fitted["prefill_small_stage_us_busy"] <= 3.0
     assert 0.1 <= fitted["decode_tile_us"] <= 5.0
+    assert 0.05 <= fitted["splitk_us_per_partial_mb"] <= 3.0 and 0.5 <= fitted["splitk_fixed_us"] <= 20.0
+    assert fitted["splitk_force_splits"] == before["splitk_force_splits"] == 0.0
     try:
         cabi.set_tuning(**fitted)
         assert cabi.tuning()["decode_tile_us"] == fitted["decode_tile_us"]

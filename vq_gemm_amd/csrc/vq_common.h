@@ -187,8 +187,8 @@ struct Tuning {
     double gemv_wide_plain_table_max_runs = 2.0;
     // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums
     // written and read once (microseconds per MB of partial sums)
-    double splitk_fixed_us = 2.0;
-    double splitk_us_per_partial_mb = 0.25;
+    double splitk_fixed_us = 4.5;
+    double splitk_us_per_partial_mb = 0.15;
     // 2, 4 or 8: VQGEMM_VARIANT_PREFILL_SPLITK takes this many slices where the shape allows (for measurements); 0: the cost model's
     double splitk_force_splits = 0.0;
 };

@@ -174,7 +174,30 @@ def fit(device: str = "cuda:0", verbose: bool = True) -> dict:
         else:
             break
     out["gemv_max_tiles_per_cu"] = best
-    # (gemv_wide_min_rows_per_wave and gemv_max_k keep their values: the wide form wins its short launches on codes that
+    # split K over the 128x128 tiles: what two slices cost beyond their multiplying (the same tiles as an unsplit problem
+    # of half the K and twice the columns), at two sizes of partial sums
+    def split_extra(M, K, N):
+        cabi.set_tuning(splitk_force_splits=2)
+        try:
+            need = cabi.workspace_bytes_b(M, K, N, 8, 256, 1, 8, cabi.VARIANT_PREFILL_SPLITK)
+            if need <= 0:
+                return None
+            spec = ProblemSpec("fit", GEOM_B, M, K, N, 8, 256, 1, 8)
+            x, codes, cb = make_problem(spec, seed=1, device=device)
+            y = torch.empty(M, N, dtype=torch.float16, device=device)
+            ws = torch.empty(need, dtype=torch.uint8, device=device)
+            t_split = time_graph(lambda: cabi.e2e_gemm_b_ws(x, codes, cb, out=y, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws))
+        finally:
+            cabi.set_tuning(splitk_force_splits=cur["splitk_force_splits"])
+        t_main = _t(M, K // 2, 2 * N, cabi.VARIANT_PREFILL_SMALL)
+        return None if t_main is None else (t_split - t_main, need / 1e6)
+    small, large = split_extra(128, 4096, 4096), split_extra(512, 4096, 4096)
+    if small and large and large[1] > small[1]:
+        per_mb = max((large[0] - small[0]) / (large[1] - small[1]), 0.05)
+        out["splitk_us_per_partial_mb"] = per_mb
+        out["splitk_fixed_us"] = max(small[0] - per_mb * small[1], 0.5)
+        say(f"split K, two slices: {small[0]:.2f} us beyond the multiplying at {small[1]:.1f} MB of partial sums, {large[0]:.2f} us at {large[1]:.1f} MB")
+    # (gemv_wide_min_rows_per_wave, gemv_wide_plain_table_max_runs and gemv_max_k keep their values: the wide form wins its short launches on codes that
     # come from HBM and loses them on cached ones - 3.3 against 3.5 us cold, 3.2 against 2.7 us warm on C2 - and this
     # loop times warm launches; bench.py's rotating pool is the protocol that decides them.)
     if verbose:
