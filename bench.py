@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
     ap.add_argument("--probe", metavar="CONFIG", default=None,
-                    help="profiling aid: launch CONFIG (C1..C5, REF = the reference's own shape in its native layout, "
+                    help="profiling aid (BLAS,C4 = hipBLASLt on the dequantised weights of C4): launch CONFIG (C1..C5, REF = the reference's own shape in its native layout, "
                          "a geometry-B shape M,K,N,vec,entries,code_bits, or GEMM,M,K,N = the plain fp16 GEMM) "
                          "--steps times, cold-HBM rotation for the decode configs, followed by one 256 MiB "
                          "device copy as a counter yardstick; prints no JSON")
@@ -143,6 +143,19 @@ def main():
                 cabi.gemm_f16(xa, wa, out=ya)
             barrier()
             print(f"probe {args.probe}: {args.steps} launches of the plain GEMM", file=sys.stderr)
+            return
+        if args.probe.startswith("BLAS,"):
+            # the hipBLASLt baseline on the dequantised weights of a configuration, for counter runs beside the fused kernel
+            spec = CONFIGS[args.probe.split(",")[1]]
+            x, codes, cb = make_problem(spec, seed=42, device=dev)
+            wd = cabi.dequant_b(codes, cb)
+            y = torch.empty(spec.M, spec.N, dtype=torch.float16, device=dev)
+            cabi.ref_gemm_f16(x, wd, w_is_nk=True, out=y)   # (picks its algorithm)
+            barrier()
+            for _ in range(args.steps):
+                cabi.ref_gemm_f16(x, wd, w_is_nk=True, out=y)
+            barrier()
+            print(f"probe {args.probe}: {args.steps} launches of hipBLASLt on the dequantised weights", file=sys.stderr)
             return
         if args.probe in CONFIGS:
             spec = CONFIGS[args.probe]

@@ -169,11 +169,23 @@ __global__ __launch_bounds__(kThreads, 1) void prefill_kernel(const half_t *__re
         cr[set][j & 3] = read_codes<C::RB>(smem + code_rd + cbuf * C::kTileBytes + (pos / 16) * (BN * 16) + j * 256 + pos % 16);
     };
     // the two halves of W piece j from the codes read before
+    // 8-vectors out of the plain table: one 16-byte gather per operand.  (This kernel is bound by the energy it spends,
+    // not by issue slots or LDS cycles: half as many gather instructions took 1 % off C4 and C5, while the conflicts
+    // the split layout saves cost it nothing.  The smaller tiles, which the LDS does bound, gather in halves.)
+    constexpr bool kWholeGather = VEC == 8 && !SPLIT;
     auto load_w1 = [&](int set, int j, bool zero) {
-        wlo[j] = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[set][j & 3], 0, zero, zero_off);
+        if constexpr (kWholeGather) {
+            uint32_t a = book[j] + cr[set][j & 3] * 16u;
+            if (TAIL) a = zero ? zero_off : a;
+            const half8_t v = *reinterpret_cast<const half8_t *>(smem + a);
+            wlo[j] = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+            whi[j] = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+        } else {
+            wlo[j] = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[set][j & 3], 0, zero, zero_off);
+        }
     };
     auto load_w2 = [&](int set, int j, bool zero) {
-        whi[j] = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[set][j & 3], 1, zero, zero_off);
+        if constexpr (!kWholeGather) whi[j] = gather4<VEC, CodeT, TAIL, SPLIT>(smem, book[j], cr[set][j & 3], 1, zero, zero_off);
     };
     // MFMA f of group p of the 4x4 quadrant (jh, ih): a group is W piece p against the four X
     // pieces, or (x_outer) X piece p against the four W pieces
@@ -880,14 +892,11 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         // waits for its own loads) only so that very large codebooks still run.
         const int ns = lds_bytes<VEC, CodeT>(p, 4) <= kLdsLimit ? 4 : lds_bytes<VEC, CodeT>(p, 3) <= kLdsLimit ? 3 : 2;
         const size_t smem = lds_bytes<VEC, CodeT>(p, ns);
-        // the split codebook layout (8-vectors, 8-bit codes, 256 entries) is built out of a plain copy
-        // that waits in the unused part of an X buffer
-        constexpr bool can_split = VEC == 8 && sizeof(CodeT) == 1;
-        const bool split = can_split && split_layout_applies(p, n_cb, kStageBytes - kWideSplitSkip);
+        // (the 256x256 tile takes its codebooks plain and gathers whole entries; the split layout is the narrow tile's)
         auto pick = [&](auto tail_c, auto ns_c) {
             constexpr bool T = decltype(tail_c)::value;
             constexpr int S = decltype(ns_c)::value;
-            return split ? prefill_kernel<VEC, CodeT, T, S, can_split> : prefill_kernel<VEC, CodeT, T, S, false>;
+            return prefill_kernel<VEC, CodeT, T, S, false>;
         };
         using std::integral_constant;
         auto kern = ns == 4   ? (tail ? pick(std::true_type{}, integral_constant<int, 4>{}) : pick(std::false_type{}, integral_constant<int, 4>{}))
