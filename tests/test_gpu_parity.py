@@ -1432,3 +1432,43 @@ def test_split_k_is_what_the_automatic_choice_takes_for_medium_m_on_few_columns_
             g.replay()
             st.synchronize()
             assert torch.equal(out, y_split)
+
+
+def test_split_k_calls_on_two_streams_with_a_workspace_each_do_not_disturb_each_other():
+    M, K, N = 384, 4096, 4096
+    spec = ProblemSpec("two_streams", GEOM_B, M, K, N, 8, 256, 32, 8, codebook_3d=True, codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=71, device=DEV)
+    x2 = (x * 0.5).contiguous()
+    need = cabi.workspace_bytes_b(M, K, N, 8, 256, 32, 8, cabi.VARIANT_PREFILL_SPLITK)
+    ws = [torch.empty(need, dtype=torch.uint8, device=DEV).random_() for _ in range(2)]
+    want = [cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_GENERIC), cabi.e2e_gemm_b(x2, codes, cb, variant=cabi.VARIANT_GENERIC)]
+    ref = [cabi.e2e_gemm_b_ws(xx, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws[0]).clone() for xx in (x, x2)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]   # default priority
+    outs = [torch.empty(M, N, dtype=torch.float16, device=DEV) for _ in range(2)]
+    for _ in range(20):
+        for i, (st, xx) in enumerate(zip(streams, (x, x2))):
+            with torch.cuda.stream(st):
+                cabi.e2e_gemm_b_ws(xx, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws[i], out=outs[i])
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(outs[i], ref[i])
+        assert vo.rel_err(_np(outs[i]), _np(want[i]).astype(np.float64))[0] <= 2 * TOL
+
+
+def test_sized_workspace_entry_point_passes_the_other_variants_through():
+    spec = ProblemSpec("ws_passthrough", GEOM_B, 48, 512, 256, 8, 256, 1, 8, codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=72, device=DEV)
+    y0 = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
+    assert torch.equal(cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_DECODE), y0)
+    # the two-pass route takes its scratch from the sized workspace, and says so when it is too small
+    y2 = cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_TWOPASS)
+    assert vo.rel_err(_np(y2), _np(y0).astype(np.float64))[0] <= 2 * TOL
+    with pytest.raises(cabi.VqGemmError) as err:
+        cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_TWOPASS, workspace=torch.empty(1024, dtype=torch.uint8, device=DEV))
+    assert err.value.code == -6
+    # split K is refused where no slice of K is long enough
+    with pytest.raises(cabi.VqGemmError) as err:
+        cabi.e2e_gemm_b_ws(x[:, :128].contiguous(), codes[:, :16].contiguous(), cb, variant=cabi.VARIANT_PREFILL_SPLITK,
+                           workspace=torch.empty(1 << 20, dtype=torch.uint8, device=DEV))
+    assert err.value.code == -4
