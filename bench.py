@@ -70,6 +70,9 @@ def parse_args():
                          "plain product + element-wise pass and as the gated entry point; 'split-k' times C3 whole and as "
                          "K slices with a summing pass behind them; 'code-usage' quantises Gaussian and heavy-tailed "
                          "weights with the package's k-means and reports how unevenly the entries are used")
+    ap.add_argument("--probe-workspace", action="store_true",
+                    help="with --probe on a geometry-B shape: launch through the entry point with a sized workspace "
+                         "(vqgemm_e2e_gemm_b_ws), so that the automatic choice may split K")
     ap.add_argument("--probe-flat-codebook", action="store_true",
                     help="with --probe on a geometry-B shape: every entry of a codebook is a copy of its first entry, so that W is "
                          "constant whatever the codes are (the control for --probe-skew 1000: same W, but the gathers still go to "
@@ -160,8 +163,9 @@ def main():
         if args.probe in CONFIGS:
             spec = CONFIGS[args.probe]
         else:
-            m, k, n, vec, entries, bits = (int(v) for v in args.probe.split(","))
-            spec = ProblemSpec("probe", GEOM_B, m, k, n, vec, entries, 1, bits)
+            fields = [int(v) for v in args.probe.split(",")]
+            m, k, n, vec, entries, bits = fields[:6]
+            spec = ProblemSpec("probe", GEOM_B, m, k, n, vec, entries, fields[6] if len(fields) > 6 else 1, bits)
         x, codes, cb = make_problem(spec, seed=42, device=dev)
         if args.probe_flat_codebook and spec.geometry == GEOM_B:
             cb3 = cb.view(-1, spec.entries, spec.vec)
@@ -188,8 +192,15 @@ def main():
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
         barrier()
-        for i in range(args.steps):
-            cabi.e2e_gemm_b(x, pool[i % n_bufs], cb, out=y, variant=args.probe_variant)
+        if args.probe_workspace:
+            need = cabi.workspace_bytes_b(spec.M, spec.K, spec.N, spec.vec, spec.entries, spec.n_codebooks, spec.code_bits)
+            ws = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+            barrier()
+            for i in range(args.steps):
+                cabi.e2e_gemm_b_ws(x, pool[i % n_bufs], cb, out=y, workspace=ws)
+        else:
+            for i in range(args.steps):
+                cabi.e2e_gemm_b(x, pool[i % n_bufs], cb, out=y, variant=args.probe_variant)
         barrier()
         dst.copy_(src)   # yardstick: reads 256 MiB, writes 256 MiB
         barrier()
