@@ -550,6 +550,8 @@ def main():
         "prepacked_codes": main_res.get("prepacked_codes"),
         "other_configs": others,
         "reference_layout_and_control": native,
+        # the file of cost-model constants behind the automatic kernel choice (None: the compiled-in table)
+        "tuning_file": cabi.tuning_file(),
     }
     if others:
         # what the matrix cores sustain on this device with random operands (register-only MFMA loop):

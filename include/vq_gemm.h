@@ -159,8 +159,10 @@ int vqgemm_e2e_gemm_a(const void *x, const void *w, const void *codebook, void *
  * with VQGEMM_E_SCRATCH, whichever route they would take.  All calls on one GPU share that GPU's
  * array: calls that overlap in time on one GPU (different streams) race on it.  Nothing in it has to
  * be cleared between calls - the dequant pass overwrites every element the GEMM pass reads.  The
- * first call on a device looks the array's address up (which makes the runtime load the code object
- * that holds it); make that call outside stream capture.
+ * array used is the one of the device that owns `stream` (the current device for the default stream).
+ * The first call on a device looks the array's address up (which makes the runtime load the code object
+ * that holds it): make that call outside stream capture - under capture it is refused with
+ * hipErrorStreamCaptureUnsupported and nothing is recorded.
  */
 #define VQGEMM_NOALLOC_SCRATCH_BYTES (16 << 20)
 int vqgemm_e2e_gemm_a_noalloc(const void *x, const void *w, const void *codebook, void *out,

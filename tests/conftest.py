@@ -3,6 +3,10 @@ import sys
 
 import pytest
 
+# The tests assert kernel choices of the compiled-in cost-model table: a tuning.json left in the package by
+# `python -m vq_gemm_amd.tune --fit --write` is not handed to the library.
+os.environ.setdefault("VQGEMM_NO_PACKAGE_TUNING", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

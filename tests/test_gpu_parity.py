@@ -876,25 +876,28 @@ def test_tune_reports_every_variant_and_the_automatic_choice():
     assert r["auto_over_fastest"] > 0
 
 
-def test_tune_fit_measures_plausible_constants_and_the_library_takes_them():
+def test_tune_fit_returns_the_table_and_the_library_takes_it():
+    import math
     from vq_gemm_amd import tune
     before = cabi.tuning()
     fitted = tune.fit(verbose=False)
     assert set(fitted) == set(before)
-    # plausible for any MI355X: microseconds per stage and per tile, neither zero nor wild
-    assert 0.2 <= fitted["prefill_stage_us_256x256"] <= 4.0 and 0.1 <= fitted["prefill_stage_us_256x128"] <= 3.0
-    assert 0.1 <= fitted["prefill_small_stage_us_idle"] <= fitted["prefill_small_stage_us_busy"] <= 3.0
-    assert 0.1 <= fitted["decode_tile_us"] <= 5.0
-    assert 0.05 <= fitted["splitk_us_per_partial_mb"] <= 3.0 and 0.5 <= fitted["splitk_fixed_us"] <= 20.0
+    # (the fitted values are timings of the box at hand: printed, not asserted - only that they are numbers)
+    _say("  fitted: " + ", ".join(f"{k}={v:.3g}" for k, v in sorted(fitted.items())))
+    assert all(math.isfinite(v) for v in fitted.values())
     assert fitted["splitk_force_splits"] == before["splitk_force_splits"] == 0.0
     try:
         cabi.set_tuning(**fitted)
         assert cabi.tuning()["decode_tile_us"] == fitted["decode_tile_us"]
-        # the measured configurations keep their kernels under the refitted constants
-        assert cabi.select_variant_b(4096, 4096, 4096, 8, 256, 32, 8) == cabi.VARIANT_PREFILL
-        assert cabi.select_variant_b(16, 4096, 11008, 4, 4096, 1, 16) == cabi.VARIANT_DECODE
+        # the library answers for the measured configurations under the refitted table (which kernel it names is
+        # the fit's business; that it names one the shape can run is the library's)
+        assert cabi.select_variant_b(4096, 4096, 4096, 8, 256, 32, 8) > 0
+        assert cabi.select_variant_b(16, 4096, 11008, 4, 4096, 1, 16) > 0
     finally:
         cabi.set_tuning(**before)
+    # with the compiled-in table the measured configurations keep their kernels
+    assert cabi.select_variant_b(4096, 4096, 4096, 8, 256, 32, 8) == cabi.VARIANT_PREFILL
+    assert cabi.select_variant_b(16, 4096, 11008, 4, 4096, 1, 16) == cabi.VARIANT_DECODE
 
 
 # shapes the tiled kernel takes (K a multiple of 64, N of 8): few tiles -> 128x128
@@ -1131,6 +1134,32 @@ def test_modules_serve_reference_native_shapes_on_every_route(M, K, Nc, route):
     # the fused modules' result is what the C ABI's automatic choice gives with scratch at hand
     ws = torch.empty(K, 2 * Nc, dtype=torch.float16, device=DEV)
     assert torch.equal(ops.load_module("s2_128").e2e_gemm(x, w, cb), cabi.e2e_gemm_a(x, w, cb, workspace=ws))
+
+
+@pytest.mark.parametrize("M,K,Nc", [(2048, 4096, 640), (512, 4096, 640), (2048, 2048, 2048)])
+def test_fused_reference_layout_kernel_gives_the_same_bits_on_every_launch(M, K, Nc):
+    # The fused kernel waits for its hand-issued loads by count, and a count that does not match the order of the
+    # loads shows as a rare wrong element on a fast launch, not as a steady error.  The reference's own shape
+    # (128x128 tiles, 160 of them), a shorter X on it and a shape of 256x128 tiles: 50 launches each on fixed
+    # operands, every result equal to the first bit for bit, the first within the bar of the oracle on sampled rows.
+    spec = ProblemSpec("A", GEOM_A, M, K, 2 * Nc, 2, 256, Nc // 4, 8, codebook_std=1.0)
+    x, w, cb = make_problem(spec, seed=71, device=DEV)
+    _say("fused geometry A, 50 launches", M, K, Nc)
+    first = cabi.e2e_gemm_a(x, w, cb, variant=cabi.VARIANT_PREFILL).clone()
+    torch.cuda.synchronize()
+    rows = np.unique(np.concatenate([np.arange(0, M, max(1, M // 32)), [M - 1]]))
+    e1, e2 = vo.rel_err(_np(first)[rows], vo.vq_gemm_a(_np(x)[rows], _np(w), _np(cb), acc=np.float64))
+    _say(f"  rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+    assert e1 <= TOL, (e1, e2)
+    # back to back (the next launch's prologue runs beside the previous one's tail), then one at a time
+    outs = [cabi.e2e_gemm_a(x, w, cb, variant=cabi.VARIANT_PREFILL) for _ in range(25)]
+    torch.cuda.synchronize()
+    for i, y in enumerate(outs):
+        assert torch.equal(y, first), f"launch {i} differs"
+    for i in range(25):
+        y = cabi.e2e_gemm_a(x, w, cb, variant=cabi.VARIANT_PREFILL)
+        torch.cuda.synchronize()
+        assert torch.equal(y, first), f"synchronised launch {i} differs"
 
 
 def test_module_out_argument_receives_the_result():
@@ -1401,6 +1430,27 @@ def test_split_k_against_the_oracle_and_from_run_to_run(row):
     assert err.value.code == -6
     ya = cabi.e2e_gemm_b_ws(x, codes, cb, workspace=small)
     assert vo.rel_err(_np(ya), want)[0] <= TOL
+
+
+def test_split_k_scoped_accesses_equal_the_textbook_fences_bit_for_bit():
+    # The exchange moves partial sums with device-scope loads and stores and hand-written waits; the library also
+    # carries the release / acquire fences the memory model asks for, behind a switch of the tuning table.  Same
+    # partial sums, same order of addition: the two paths must agree bit for bit.
+    M, K, N = 512, 4096, 4096
+    spec = ProblemSpec("splitk_fences", GEOM_B, M, K, N, 8, 256, 32, 8, codebook_3d=True, codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=67, device=DEV)
+    need = cabi.workspace_bytes_b(M, K, N, 8, 256, 32, 8, cabi.VARIANT_PREFILL_SPLITK)
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV).random_()
+    fast = cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws).clone()
+    before = cabi.tuning()["splitk_validate_fences"]
+    try:
+        cabi.set_tuning(splitk_validate_fences=1)
+        for _ in range(3):
+            ws.random_()
+            fenced = cabi.e2e_gemm_b_ws(x, codes, cb, variant=cabi.VARIANT_PREFILL_SPLITK, workspace=ws)
+            assert torch.equal(fenced, fast)
+    finally:
+        cabi.set_tuning(splitk_validate_fences=before)
 
 
 def test_split_k_is_what_the_automatic_choice_takes_for_medium_m_on_few_columns_and_only_with_a_workspace():

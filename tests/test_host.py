@@ -166,3 +166,20 @@ def test_tuning_constants_can_be_read_set_and_loaded_from_a_file(tmp_path):
     finally:
         cabi.set_tuning(**before)
     assert cabi.tuning() == before
+
+
+def test_vqlinear_codes_key_works_on_inference_tensors():
+    # a module whose codes were made under torch.inference_mode(): such tensors keep no version counter
+    from vq_gemm_amd.nn import VQLinear
+    with torch.inference_mode():
+        codes = torch.zeros(32, 32, dtype=torch.uint8)
+        cb = torch.zeros(256, 8, dtype=torch.float16)
+        layer = VQLinear(codes, cb)
+        k1 = layer._codes_key()
+    assert layer.codes.is_inference()
+    assert layer._codes_key() == k1
+    # an ordinary tensor: the key follows in-place updates
+    layer2 = VQLinear(torch.zeros(32, 32, dtype=torch.uint8), cb.clone())
+    k2 = layer2._codes_key()
+    layer2.codes.add_(1)
+    assert layer2._codes_key() != k2

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import sys
 import re
 
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
@@ -80,15 +81,33 @@ def _load(name, sigs):
 TUNING_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning.json")
 
 
+_tuning_file = None  # the file of constants the library was handed at load, if any
+
+
 def lib():
-    """The C-ABI library.  When `vq_gemm_amd/tuning.json` exists (written by `python -m vq_gemm_amd.tune --fit`) and
-    VQGEMM_TUNING_FILE is not set, the library is pointed at it before its first use."""
-    global _lib
+    """The C-ABI library.  When `vq_gemm_amd/tuning.json` exists (written by `python -m vq_gemm_amd.tune --fit
+    --write`), VQGEMM_TUNING_FILE is not set (the library reads that one by itself) and VQGEMM_NO_PACKAGE_TUNING is not
+    set either, the file is handed to the library once, here, through `vqgemm_tuning_load`; `tuning_file()` says
+    which file, if any, is in force."""
+    global _lib, _tuning_file
     if _lib is None:
-        if "VQGEMM_TUNING_FILE" not in os.environ and os.path.exists(TUNING_FILE):
-            os.environ["VQGEMM_TUNING_FILE"] = TUNING_FILE
-        _lib = _load("libvqgemm.so", _SIGNATURES)
+        loaded = _load("libvqgemm.so", _SIGNATURES)
+        env = os.environ.get("VQGEMM_TUNING_FILE")
+        if env:
+            _tuning_file = env
+        elif not os.environ.get("VQGEMM_NO_PACKAGE_TUNING") and os.path.exists(TUNING_FILE):
+            if loaded.vqgemm_tuning_load(TUNING_FILE.encode()) >= 0:
+                _tuning_file = TUNING_FILE
+                print(f"vq_gemm_amd: cost-model constants from {TUNING_FILE}", file=sys.stderr)
+        _lib = loaded
     return _lib
+
+
+def tuning_file():
+    """Path of the file of cost-model constants in force (VQGEMM_TUNING_FILE, or the package's own tuning.json), or
+    None when the compiled-in table is."""
+    lib()
+    return _tuning_file
 
 
 def tuning() -> dict:

@@ -71,12 +71,13 @@ const TuningEntry kTuningEntries[] = {
     {"splitk_fixed_us", &Tuning::splitk_fixed_us},
     {"splitk_us_per_partial_mb", &Tuning::splitk_us_per_partial_mb},
     {"splitk_force_splits", &Tuning::splitk_force_splits},
+    {"splitk_validate_fences", &Tuning::splitk_validate_fences},
 };
 constexpr int kTuningCount = (int)(sizeof(kTuningEntries) / sizeof(kTuningEntries[0]));
 
 std::mutex g_tuning_mu;
 Tuning g_tuning;             // written under the mutex; read without it (plain doubles, set before the launches that use them)
-bool g_tuning_file_read = false;
+std::atomic<bool> g_tuning_file_read{false};  // (acquire/release: a reader that sees true also sees what the file set)
 
 const TuningEntry *find_tuning(const char *name)
 {
@@ -181,12 +182,12 @@ int select_b(const ProblemB &p, bool all_aligned16)
 const Tuning &tuning()
 {
     // the file named by VQGEMM_TUNING_FILE is read once, at the first question
-    if (!g_tuning_file_read) {
+    if (!g_tuning_file_read.load(std::memory_order_acquire)) {
         std::lock_guard<std::mutex> lock(g_tuning_mu);
-        if (!g_tuning_file_read) {
+        if (!g_tuning_file_read.load(std::memory_order_relaxed)) {
             const char *path = std::getenv("VQGEMM_TUNING_FILE");
             if (path && path[0]) read_tuning_file(path);
-            g_tuning_file_read = true;
+            g_tuning_file_read.store(true, std::memory_order_release);
         }
     }
     return g_tuning;

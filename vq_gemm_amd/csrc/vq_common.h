@@ -191,6 +191,7 @@ struct Tuning {
     double splitk_us_per_partial_mb = 0.15;
     // 2, 4 or 8: VQGEMM_VARIANT_PREFILL_SPLITK takes this many slices where the shape allows (for measurements); 0: the cost model's
     double splitk_force_splits = 0.0;
+    double splitk_validate_fences = 0.0;  // 1: release / acquire fences of device scope around the split-K count (validation)
 };
 const Tuning &tuning();
 

@@ -21,17 +21,30 @@ constexpr int kMaxDevices = 64;
 std::mutex g_mu;
 void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, looked up once
 
-// Device address of the current device's copy of `scratch`.
-hipError_t scratch_address(void **ptr)
+// Device address of the copy of `scratch` on the device that owns `stream` (the current device for the
+// default stream).  The first look-up on a device makes the runtime load the code object that holds the
+// array: it is refused while `stream` is capturing, where such work does not belong.
+hipError_t scratch_address(hipStream_t stream, void **ptr)
 {
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
+    int current = 0;
+    hipError_t e = hipGetDevice(&current);
     if (e != hipSuccess) return e;
+    int dev = current;
+    if (stream) {
+        e = hipStreamGetDevice(stream, &dev);
+        if (e != hipSuccess) return e;
+    }
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
     std::lock_guard<std::mutex> lock(g_mu);
     if (!g_scratch_ptr[dev]) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (stream && hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+            return hipErrorStreamCaptureUnsupported;
+        // (hipGetSymbolAddress answers for the current device)
+        if (dev != current && (e = hipSetDevice(dev)) != hipSuccess) return e;
         void *p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (dev != current) (void)hipSetDevice(current);
         if (e != hipSuccess) return e;
         if (!p) return hipErrorInvalidSymbol;
         g_scratch_ptr[dev] = p;
@@ -52,7 +65,7 @@ int vqgemm_e2e_gemm_a_noalloc(const void *x, const void *w, const void *codebook
     // does not depend on the kernel choice.
     if (K * 2 * Nc * 2 > (int64_t)VQGEMM_NOALLOC_SCRATCH_BYTES) return VQGEMM_E_SCRATCH;
     void *ptr = nullptr;
-    const hipError_t e = scratch_address(&ptr);
+    const hipError_t e = scratch_address(static_cast<hipStream_t>(stream), &ptr);
     if (e != hipSuccess) return static_cast<int>(e);
     return vqgemm_e2e_gemm_a(x, w, codebook, out, M, K, Nc, variant, ptr, stream);
 }

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                                                                     int N, int entries, int rows_per_cb, int tiles_m,
                                                                     int tiles_n, int cb_lds_count, int gated, int k_len,
                                                                     int splits, float4_t *__restrict__ partials,
-                                                                    unsigned int *__restrict__ counters)
+                                                                    unsigned int *__restrict__ counters, int fenced)
 {
     typedef PrefillCfg<VEC, CodeT> C;
     constexpr int D = NS - 1;                 // loads run D stages ahead
@@ -297,6 +297,12 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
     // (measured: 3 us per MB of partial sums).  A store is complete, and visible device-wide, when the counter
     // has counted it; the count itself is a relaxed device-scope atomic; the loads of the last workgroup are issued
     // behind the barrier that follows its count.
+#if !defined(__HIP_DEVICE_COMPILE__) || defined(__gfx942__) || defined(__gfx950__)
+    // (what "sc1" means for a store and a load, and that a counted store is visible device-wide, are properties of
+    // these two targets; another target has to re-establish them or build with the fences below)
+#else
+#error "the split-K exchange relies on the gfx942/gfx950 behaviour of device-scope (sc1) loads and stores"
+#endif
     if (splits > 1) {
         // partial sums of (tile, slice): half h (two floats) of accumulator (j, i) of thread tid at
         // [((j * SMP + i) * 2 + h) * 256 + tid], moved as 64-bit words (the widest scoped access there is)
@@ -313,7 +319,12 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                     __hip_atomic_store(mine + ((j * SMP + i) * 2 + h) * kThreads,
                                        __builtin_bit_cast(uint64_t, float2_t{acc[j][i][2 * h], acc[j][i][2 * h + 1]}), __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
+        // Every partial-sum store of this thread is complete (counted back) here, and the barrier extends that to the
+        // workgroup: nothing may be moved across this wait - not the stores above it, not the count below it.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // (validation path, Tuning::splitk_validate_fences: the textbook release / acquire pair of device scope around
+        // the count, as the memory model asks for; same results bit for bit, at the cost of the L2 write-backs)
+        if (fenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         __syncthreads();
         uint32_t *flag = reinterpret_cast<uint32_t *>(smem);
         if (tid == 0) *flag = __hip_atomic_fetch_add(counters + wg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -321,6 +332,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
         const bool last = *flag == (uint32_t)(splits - 1);
         __syncthreads();  // the flag's word belongs to the epilogue's staging area again
         if (!last) return;
+        if (fenced) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         // The sum in the order of the slices, whoever is last - this workgroup's own sums are read back like the
         // others' (the same bits it wrote; its registers are free for the loads that way).
         for (int sl = 0; sl < splits; sl++) {
@@ -443,7 +455,8 @@ hipError_t launch_small_typed(const ProblemB &p, hipStream_t s, int splits, void
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads), smem, s, p.x,
                        static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
-                       tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0, p.K / splits, splits, partials, counters);
+                       tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0, p.K / splits, splits, partials, counters,
+                       tuning().splitk_validate_fences >= 1.0 ? 1 : 0);
     return hipGetLastError();
 }
 

@@ -57,7 +57,11 @@ class VQLinear(torch.nn.Module):
         return self
 
     def _codes_key(self):
-        return (self.codes._version, self.codes.data_ptr())
+        # (a tensor made under torch.inference_mode() keeps no version counter and cannot be updated in
+        # place outside that mode: its address, shape and device identify its contents)
+        c = self.codes
+        version = -1 if c.is_inference() else c._version
+        return (version, c.data_ptr(), tuple(c.shape), str(c.device))
 
     def _fresh_packed_codes(self):
         """The packed copy, re-made first if `codes` changed since it was packed (`load_state_dict`,
