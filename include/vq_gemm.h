@@ -119,13 +119,12 @@ int64_t vqgemm_workspace_bytes_b(int64_t M, int64_t K, int64_t N, int32_t vec, i
  *     y[m, 16g + r] = silu(P[m, 32g + r]) * P[m, 32g + 16 + r],   P = X . W^T (+ bias[n], indexed like the rows of W),
  * silu(t) = t / (1 + exp(-t)), everything in fp32 with one rounding to fp16: y is [M, N/2] and the [M, N] product
  * never exists in memory.  N % 32 == 0.  No counterpart in the reference (its storeC has no epilogue,
- * strategy_2/bsz128/src.cu:163-177).  The prefill kernels (variants 3, 5, 6), the batched K-sliced decode kernel
- * (variant 2: K % 256 == 0, (N / n_codebooks) % 32 == 0, not 2-vectors with 16-bit codes), the wide GEMV kernel
- * (variant 8: one row of X) and the scalar kernel (variant 1) carry the epilogue; the four-wave GEMV kernel and the
- * general K-sliced kernel do not: VQGEMM_VARIANT_TWOPASS here means the plain product into `workspace` ([M, N]
- * fp16) followed by the element-wise pass, and VQGEMM_VARIANT_AUTO takes that route where the plain product would
- * run one of those two and a workspace is given (NULL: the batched decode, prefill or scalar kernel takes the shape
- * after all).
+ * strategy_2/bsz128/src.cu:163-177).  Every fused kernel carries the epilogue: the prefill tiles (variants 3, 5, 6),
+ * both K-sliced decode kernels (variant 2), both GEMV kernels (variant 8; the four-wave form and the batched K-sliced
+ * kernel want (N / n_codebooks) % 32 == 0) and the scalar kernel (variant 1); VQGEMM_VARIANT_AUTO follows the plain
+ * product's choice and needs no workspace.  VQGEMM_VARIANT_TWOPASS here means the plain product into `workspace`
+ * ([M, N] fp16) followed by the element-wise pass (vqgemm_silu_mul's interleaved form), kept as the control; the
+ * other variants ignore `workspace`.
  */
 int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebook, const void *bias, void *y,
                             int64_t M, int64_t K, int64_t N, int32_t vec, int32_t entries,

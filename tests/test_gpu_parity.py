@@ -1291,7 +1291,16 @@ GATED_B = [
     ("decode_books_ragged_units", 16, 4096, 4 * 1056, 8, 256, 8, 4),   # 33 pairs per codebook: short last batches
     ("decode_chunked_k", 9, 8192, 1024, 8, 256, 8, 1),           # K in two chunks: gate and up sums carried in the LDS
     ("decode_two_slabs_u8v4", 40, 2048, 1536, 4, 256, 8, 2),
-    ("decode_v2_u16_no_pairs", 16, 1024, 512, 2, 4096, 16, 1),   # batches of one tile: no gated form, two passes
+    ("decode_v2_u16_general", 16, 1024, 512, 2, 4096, 16, 1),    # batches of one tile in the batched kernel: the general kernel
+    ("decode_general_k640_ragged", 7, 640, 224, 8, 256, 8, 1),    # K not a multiple of 256: the general K-sliced kernel
+    ("decode_general_books_48_rows", 16, 1152, 480, 4, 4096, 16, 10),   # 48 rows per codebook: pairs that lie in two codebooks
+    ("decode_general_k8320_chunks_m33", 33, 8192 + 128, 96, 8, 256, 8, 1),   # three slabs of X, K in chunks
+    ("gemv4_c3_weights_m1", 1, 4096, 1376, 4, 4096, 16, 1),       # the four-wave GEMV kernel: 4-vectors, 16-bit codes, 4096 entries
+    ("gemv4_c3_weights_m2", 2, 4096, 1376, 4, 4096, 16, 1),
+    ("gemv4_v4_u8_m1", 1, 2048, 2048, 4, 256, 8, 4),
+    ("gemv4_v4_u8_m2", 2, 4096, 1024, 4, 256, 8, 1),
+    ("gemv4_v8_u8_few_rows_m2", 2, 4096, 2048, 8, 256, 8, 2),    # fewer rows than the wide form takes
+    ("gemv4_v2_u8_m1", 1, 2048, 512, 2, 256, 8, 1),
     ("odd_k_scalar_only", 5, 72, 64, 8, 256, 8, 1),
 ]
 
@@ -1327,12 +1336,16 @@ def test_gated_epilogue_against_the_oracle(row):
             ran.append(variant)
     assert cabi.VARIANT_AUTO in ran and cabi.VARIANT_GENERIC in ran
     if name.startswith("decode_"):
-        assert (cabi.VARIANT_DECODE in ran) == (name != "decode_v2_u16_no_pairs")
-    if name.startswith("gemv_wide"):
+        assert cabi.VARIANT_DECODE in ran
+    if name.startswith("gemv"):
         assert cabi.VARIANT_DECODE_GEMV in ran
+    if name.startswith("gemv4") or name.startswith("decode_general"):
+        # no gated call needs a workspace: the automatic choice without one is a decode kernel with its own epilogue
+        g, e, vv = cabi._cb_dims(cb)
+        assert cabi.select_variant_b(M, K, N, vv, e, g, bits) in (cabi.VARIANT_DECODE, cabi.VARIANT_DECODE_GEMV)
     if name.endswith("_tile") or "tile_" in name:
         assert cabi.VARIANT_PREFILL in ran
-    # without a workspace the automatic choice still answers (prefill or scalar kernel), and answers the same twice
+    # without a workspace the automatic choice answers the same way (no kernel needs one), and the same twice
     y0 = cabi.e2e_gemm_b_gated(x, codes, cb)
     e1, e2 = vo.rel_err(_np(y0), want)
     assert e2 <= TOL and e1 <= 2 * TOL and torch.equal(cabi.e2e_gemm_b_gated(x, codes, cb), y0)

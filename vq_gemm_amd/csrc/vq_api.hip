@@ -423,15 +423,13 @@ int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebo
         if (K == 0 || !a16) variant = VQGEMM_VARIANT_GENERIC;
         else if (decode_gemv_wide_preferred(p)) variant = VQGEMM_VARIANT_DECODE_GEMV;
         else {
-            // What the plain product would run on decides: the prefill kernels and the batched K-sliced decode kernel
-            // carry the gated epilogue themselves; where another decode kernel would be chosen (the four-wave GEMV, the
-            // general K-sliced kernel), the product goes to the workspace and the element-wise pass follows (two
-            // launches), or - without a workspace - the batched decode or the prefill kernels take it after all.
+            // What the plain product would run on decides: every tiled kernel carries the gated epilogue itself (the
+            // GEMV kernels and the K-sliced decode kernels want whole groups of 32 interleaved rows per codebook
+            // resp. per matrix; where one of them refuses, the next in line takes the shape).
             const int plain_variant = select_b(plain, true);
-            const bool decode_like = plain_variant == VQGEMM_VARIANT_DECODE || plain_variant == VQGEMM_VARIANT_DECODE_GEMV;
-            if (plain_variant == VQGEMM_VARIANT_DECODE && decode_gated_supports(p)) variant = VQGEMM_VARIANT_DECODE;
-            else if (decode_like && workspace) variant = VQGEMM_VARIANT_TWOPASS;
-            else if (decode_like && decode_gated_supports(p)) variant = VQGEMM_VARIANT_DECODE;
+            if (plain_variant == VQGEMM_VARIANT_DECODE_GEMV && decode_gemv_supports(p)) variant = VQGEMM_VARIANT_DECODE_GEMV;
+            else if ((plain_variant == VQGEMM_VARIANT_DECODE || plain_variant == VQGEMM_VARIANT_DECODE_GEMV) && decode_gated_supports(p))
+                variant = VQGEMM_VARIANT_DECODE;
             else if (prefill_supports(plain)) variant = VQGEMM_VARIANT_PREFILL;
             else variant = VQGEMM_VARIANT_GENERIC;
         }
@@ -443,7 +441,7 @@ int vqgemm_e2e_gemm_b_gated(const void *x, const void *codes, const void *codebo
         break;
     case VQGEMM_VARIANT_DECODE_GEMV:
         if (!a16) return VQGEMM_E_ALIGN;
-        if (K == 0 || !decode_gemv_wide_preferred(p)) return VQGEMM_E_VARIANT;
+        if (K == 0 || !decode_gemv_supports(p)) return VQGEMM_E_VARIANT;
         e = launch_decode_gemv(p, s);
         break;
     case VQGEMM_VARIANT_DECODE:

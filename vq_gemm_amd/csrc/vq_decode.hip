@@ -850,11 +850,8 @@ hipError_t launch_pack_codes(const void *src, void *dst, int64_t N, int64_t K, i
     }
 }
 
-// the gated epilogue: the batched kernel only
-bool decode_gated_supports(const ProblemB &p)
-{
-    return p.gated && p.M >= 1 && p.M <= kBatchedMaxM && decode_general_supports(p) && batched_supports(p);
-}
+// the gated epilogue: both K-sliced kernels carry it (as the plain product: the general kernel in slabs up to 64 rows of X)
+bool decode_gated_supports(const ProblemB &p) { return p.gated && decode_supports(p); }
 
 bool decode_supports(const ProblemB &p)
 {
@@ -929,7 +926,6 @@ hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
-    if (p.gated && !batched_supports(p)) return hipErrorInvalidValue;  // (the general kernel has no gated epilogue)
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension
         if (p.packed) {
@@ -952,7 +948,7 @@ hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
     for (int m0 = 0; m0 < p.M; m0 += 16) {
         ProblemB q = p;
         q.x = p.x + (int64_t)m0 * p.K;
-        q.y = p.y + (int64_t)m0 * p.N;
+        q.y = p.y + (int64_t)m0 * (p.gated ? p.N / 2 : p.N);
         q.M = p.M - m0 < 16 ? p.M - m0 : 16;
         const hipError_t e = launch_decode_general(q, s);
         if (e != hipSuccess) return e;

@@ -89,7 +89,11 @@ struct GemvCfg {
 };
 
 // RUNS: runs of 2048 k in a row of W; MX: rows of X (each gathered codeword meets MX shares of x).
-template <int VEC, typename CodeT, int RUNS, int MX>
+// GATED: the epilogue of a gate/up pair (rows of W interleaved in groups of 16: rows 32g .. 32g+15 gate, the
+// sixteen behind them the up rows of the same outputs).  A workgroup's sixteen code rows are then the gate and the
+// up rows of eight outputs, a wave's four the pairs of two outputs - rows 0 and 1 the gate rows, 2 and 3 the up
+// rows - and y is [M, N/2].
+template <int VEC, typename CodeT, int RUNS, int MX, bool GATED>
 __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half_t *__restrict__ x,
                                                                        const CodeT *__restrict__ codes,
                                                                        const half_t *__restrict__ cb,
@@ -97,18 +101,24 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
                                                                        const half_t *__restrict__ bias, int K,
                                                                        int N, int entries, int rows_per_cb)
 {
+    static_assert(!GATED || kGemvRows == 4, "a wave's rows are two gate/up pairs");
     typedef GemvCfg<VEC, CodeT> C;
     typedef uint32_t words_t __attribute__((ext_vector_type(C::CW)));
     __shared__ __align__(16) uint4_t table[C::kTableBytes / 16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int row0 = blockIdx.x * kGemvTile + wave * kGemvRows;
+    // plain: the wave's rows are row0 .. row0+3.  GATED: out0 is the first of its two outputs, its code rows the
+    // gate rows of out0 and out0+1 (neighbours inside one group of 16) and the up rows 16 further on.
+    const int out0 = blockIdx.x * (kGemvTile / 2) + wave * (kGemvRows / 2);
+    const int row0 = GATED ? 32 * (out0 >> 4) + (out0 & 15) : blockIdx.x * kGemvTile + wave * kGemvRows;
+    auto code_row = [&](int r) { return GATED ? row0 + (r & 1) + 16 * (r >> 1) : row0 + r; };
     constexpr int J = RUNS * 64 * C::CPR;  // codes per row
 
     // The table's load goes out first and is the first to be back (it comes out of the L2): its copy
     // into the LDS and the barrier then pass while the codes (HBM) and x are still on their way.
     // (no division in front of the first load when there is one codebook)
-    const int book = rows_per_cb >= N ? 0 : (blockIdx.x * kGemvTile) / rows_per_cb;
+    // (GATED: the workgroup's rows lie inside one group of 32, and a codebook holds whole groups)
+    const int book = rows_per_cb >= N ? 0 : (GATED ? 32 * ((blockIdx.x * (kGemvTile / 2)) >> 4) : blockIdx.x * kGemvTile) / rows_per_cb;
     // (entries * VEC * 2 is a multiple of 16, so every codebook starts on a 16-byte boundary)
     const int chunks = entries * VEC * 2 / 16;
     const uint4_t *tsrc = reinterpret_cast<const uint4_t *>(cb + (int64_t)book * entries * VEC);
@@ -119,7 +129,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     for (int r = 0; r < kGemvRows; r++)
 #pragma unroll
         for (int q = 0; q < RUNS; q++) {
-            const words_t v = *reinterpret_cast<const words_t *>(codes + (int64_t)(row0 + r) * J + (q * 64 + lane) * C::CPR);
+            const words_t v = *reinterpret_cast<const words_t *>(codes + (int64_t)code_row(r) * J + (q * 64 + lane) * C::CPR);
 #pragma unroll
             for (int i = 0; i < C::CW; i++) cw[r][q][i] = v[i];
         }
@@ -183,14 +193,24 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
             }
 #pragma unroll
     for (int m = 0; m < MX; m++) {
-        gemv_out_t out;
+        float sum[kGemvRows];
 #pragma unroll
         for (int r = 0; r < kGemvRows; r++) {
-            float s = wave_sum(acc[m][r]);
-            if (bias) s += (float)bias[row0 + r];
-            out[r] = (half_t)s;
+            sum[r] = wave_sum(acc[m][r]);
+            if (bias) sum[r] += (float)bias[code_row(r)];
         }
-        if (lane == 0) *reinterpret_cast<gemv_out_t *>(y + (int64_t)m * N + row0) = out;
+        if constexpr (GATED) {
+            // outputs out0 and out0+1: silu(gate) * up, one rounding
+            half2_t out;
+#pragma unroll
+            for (int j = 0; j < 2; j++) out[j] = (half_t)(silu_f32(sum[j]) * sum[2 + j]);
+            if (lane == 0) *reinterpret_cast<half2_t *>(y + (int64_t)m * (N / 2) + out0) = out;
+        } else {
+            gemv_out_t out;
+#pragma unroll
+            for (int r = 0; r < kGemvRows; r++) out[r] = (half_t)sum[r];
+            if (lane == 0) *reinterpret_cast<gemv_out_t *>(y + (int64_t)m * N + row0) = out;
+        }
     }
 }
 
@@ -581,6 +601,8 @@ bool decode_gemv_plain_supports(const ProblemB &p)
     if (p.entries > (u8 ? 256 : 4096) || (p.entries * p.vec * 2) % 16 != 0) return false;
     // two rows of X at most outside the first format (three and four never pay)
     const int max_m = (p.vec == 8 && u8) ? 4 : 2;
+    // gated: whole groups of 32 interleaved rows, per codebook too
+    if (p.gated && (p.N % 32 != 0 || p.rows_per_cb % 32 != 0)) return false;
     return p.M >= 1 && p.M <= max_m && (int)(p.K / kRunK) * p.M * 16 <= kGemvMaxXRegs && !p.packed && p.K >= kRunK &&
            p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns && p.N % kGemvTile == 0 && p.rows_per_cb % kGemvTile == 0;
 }
@@ -600,7 +622,7 @@ bool decode_gemv_wide_preferred(const ProblemB &p)
 
 namespace {
 
-template <int VEC, typename CodeT>
+template <int VEC, typename CodeT, bool GATED>
 hipError_t launch_gemv_format(const ProblemB &p, hipStream_t s)
 {
     const dim3 grid(p.N / kGemvTile), block(kGemvWaves * 64);
@@ -609,21 +631,21 @@ hipError_t launch_gemv_format(const ProblemB &p, hipStream_t s)
         hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.K, p.N, p.entries, p.rows_per_cb);
     };
     switch ((p.K / kRunK) * 10 + p.M) {
-    case 11: launch(decode_gemv_kernel<VEC, CodeT, 1, 1>); break;
-    case 12: launch(decode_gemv_kernel<VEC, CodeT, 1, 2>); break;
-    case 21: launch(decode_gemv_kernel<VEC, CodeT, 2, 1>); break;
-    case 22: launch(decode_gemv_kernel<VEC, CodeT, 2, 2>); break;
-    case 31: launch(decode_gemv_kernel<VEC, CodeT, 3, 1>); break;
-    case 32: launch(decode_gemv_kernel<VEC, CodeT, 3, 2>); break;
-    case 41: launch(decode_gemv_kernel<VEC, CodeT, 4, 1>); break;
-    case 42: launch(decode_gemv_kernel<VEC, CodeT, 4, 2>); break;
+    case 11: launch(decode_gemv_kernel<VEC, CodeT, 1, 1, GATED>); break;
+    case 12: launch(decode_gemv_kernel<VEC, CodeT, 1, 2, GATED>); break;
+    case 21: launch(decode_gemv_kernel<VEC, CodeT, 2, 1, GATED>); break;
+    case 22: launch(decode_gemv_kernel<VEC, CodeT, 2, 2, GATED>); break;
+    case 31: launch(decode_gemv_kernel<VEC, CodeT, 3, 1, GATED>); break;
+    case 32: launch(decode_gemv_kernel<VEC, CodeT, 3, 2, GATED>); break;
+    case 41: launch(decode_gemv_kernel<VEC, CodeT, 4, 1, GATED>); break;
+    case 42: launch(decode_gemv_kernel<VEC, CodeT, 4, 2, GATED>); break;
     default:
         if constexpr (VEC == 8 && sizeof(CodeT) == 1) {
             switch ((p.K / kRunK) * 10 + p.M) {
-            case 13: launch(decode_gemv_kernel<8, uint8_t, 1, 3>); break;
-            case 14: launch(decode_gemv_kernel<8, uint8_t, 1, 4>); break;
-            case 23: launch(decode_gemv_kernel<8, uint8_t, 2, 3>); break;
-            case 24: launch(decode_gemv_kernel<8, uint8_t, 2, 4>); break;
+            case 13: launch(decode_gemv_kernel<8, uint8_t, 1, 3, GATED>); break;
+            case 14: launch(decode_gemv_kernel<8, uint8_t, 1, 4, GATED>); break;
+            case 23: launch(decode_gemv_kernel<8, uint8_t, 2, 3, GATED>); break;
+            case 24: launch(decode_gemv_kernel<8, uint8_t, 2, 4, GATED>); break;
             default: return hipErrorInvalidValue;
             }
             break;
@@ -633,18 +655,24 @@ hipError_t launch_gemv_format(const ProblemB &p, hipStream_t s)
     return hipGetLastError();
 }
 
+template <bool GATED>
+hipError_t launch_gemv_any_format(const ProblemB &p, hipStream_t s)
+{
+    const bool u8 = p.code_bits == 8;
+    switch (p.vec) {
+    case 8: return u8 ? launch_gemv_format<8, uint8_t, GATED>(p, s) : launch_gemv_format<8, uint16_t, GATED>(p, s);
+    case 4: return u8 ? launch_gemv_format<4, uint8_t, GATED>(p, s) : launch_gemv_format<4, uint16_t, GATED>(p, s);
+    default: return launch_gemv_format<2, uint8_t, GATED>(p, s);
+    }
+}
+
 }  // namespace
 
 hipError_t launch_decode_gemv(const ProblemB &p, hipStream_t s)
 {
     if (decode_gemv_wide_preferred(p)) return launch_decode_gemv_wide(p, s);
-    if (p.gated || !decode_gemv_plain_supports(p)) return hipErrorInvalidValue;
-    const bool u8 = p.code_bits == 8;
-    switch (p.vec) {
-    case 8: return u8 ? launch_gemv_format<8, uint8_t>(p, s) : launch_gemv_format<8, uint16_t>(p, s);
-    case 4: return u8 ? launch_gemv_format<4, uint8_t>(p, s) : launch_gemv_format<4, uint16_t>(p, s);
-    default: return launch_gemv_format<2, uint8_t>(p, s);
-    }
+    if (!decode_gemv_plain_supports(p)) return hipErrorInvalidValue;
+    return p.gated ? launch_gemv_any_format<true>(p, s) : launch_gemv_any_format<false>(p, s);
 }
 
 }  // namespace vq

@@ -13,6 +13,11 @@
 //     in the same order.
 //   * Per tile the partial 16x16 fp32 results of the waves are summed through 1 KB LDS slots,
 //     and one wave converts and stores the tile.
+//   * The gated epilogue of a gate/up pair (rows of W interleaved in groups of 16, so an even tile
+//     holds gate rows and the tile behind it the up rows of the same sixteen outputs): the
+//     workgroups are dealt whole pairs of tiles, one wave sums both tiles of a pair - it keeps the
+//     gate sums in registers until the up tile has been multiplied - and stores silu(gate) * up
+//     into Y [M, N/2].
 //
 // M < 16 pads the X operand with zeros; fp32 accumulation throughout, one rounding to fp16.
 #include "vq_common.h"
@@ -105,7 +110,7 @@ __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__res
                                                       const half_t *__restrict__ bias, int M, int K, int N,
                                                       int entries, int rows_per_cb, int tiles_q,
                                                       int tiles_r, int n_chunks, int stage_off,
-                                                      int aliased)
+                                                      int aliased, int gated)
 {
     typedef DecodeCfg<VEC, CodeT, STEPS> C;
     constexpr int kSliceK = C::kSliceK;
@@ -129,9 +134,11 @@ __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__res
 
     // Balanced contiguous split of the tiles over the workgroups: tiles_q each, one more for the
     // first tiles_r (quotient and remainder of tiles / workgroups, computed by the host).
+    // (gated: tiles_q and tiles_r count pairs of a gate and an up tile)
     const int wg = blockIdx.x;
-    const int tile_begin = wg * tiles_q + min(wg, tiles_r);
-    const int tile_end = tile_begin + tiles_q + (wg < tiles_r ? 1 : 0);
+    const int deal = gated ? 2 : 1;
+    const int tile_begin = deal * (wg * tiles_q + min(wg, tiles_r));
+    const int tile_end = tile_begin + deal * (tiles_q + (wg < tiles_r ? 1 : 0));
     if (tile_begin >= tile_end) return;
 
     // k of MFMA step s for this lane inside a slice that starts at k0.
@@ -265,6 +272,7 @@ __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__res
     }
 
     int parity = 0;
+    float4_t gate_sum = {0.f, 0.f, 0.f, 0.f};  // gated: the gate tile's sums, in the wave that takes the pair, until the up tile is done
     // Four accumulators: consecutive MFMAs do not wait on each other's result.
     float4_t acc[4];
 #pragma unroll
@@ -304,7 +312,8 @@ __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__res
             // turns at adding up and storing a tile.
             red[(parity * n_waves + wave) * 64 + lane] = p;
             __syncthreads();
-            if (wave == (tile % n_waves)) {
+            // (gated: both tiles of a pair go to the same wave)
+            if (wave == ((gated ? tile >> 1 : tile) % n_waves)) {
                 float4_t sum = red[(parity * n_waves) * 64 + lane];
                 for (int w = 1; w < n_waves; w++) {
                     const float4_t v = red[(parity * n_waves + w) * 64 + lane];
@@ -317,7 +326,17 @@ __global__ __launch_bounds__(512) void decode_general_kernel(const half_t *__res
 #pragma unroll
                     for (int r = 0; r < 4; r++) sum[r] += n + r < N ? (float)bias[n + r] : 0.f;
                 }
-                if (m < M) {
+                if (gated) {
+                    if ((tile & 1) == 0) {
+                        gate_sum = sum;
+                    } else if (m < M) {
+                        // outputs (tile / 2) * 16 + 4*kq .. + 3 (N is a multiple of 32: no ragged edge)
+                        half4_t h;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) h[r] = (half_t)(silu_f32(gate_sum[r]) * sum[r]);
+                        *reinterpret_cast<half4_t *>(y + (int64_t)m * (N / 2) + (tile >> 1) * kTileN + 4 * kq) = h;
+                    }
+                } else if (m < M) {
                     half_t *dst = y + (int64_t)m * N + n;
                     if ((N & 3) == 0 && n + 3 < N) {
                         half4_t h = {(half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3]};
@@ -347,13 +366,14 @@ hipError_t launch_decode_steps(const ProblemB &p, hipStream_t s)
     const int n_waves = slices < kMaxWaves ? slices : kMaxWaves;
     const int n_chunks = (slices + n_waves - 1) / n_waves;
     const int n_tiles = (p.N + kTileN - 1) / kTileN;
+    const int n_dealt = p.gated ? n_tiles / 2 : n_tiles;  // what the workgroups share: tiles, or pairs of a gate and an up tile
     const int cb_bytes = p.entries * VEC * 2;
     // Workgroups resident per CU: the kernel needs 129+ registers per lane, i.e. at most 3 waves
     // per SIMD.
     int per_cu = 12 / n_waves > 0 ? 12 / n_waves : 1;
     const int cus = device_cu_count();
-    int grid = n_tiles < cus * per_cu ? n_tiles : cus * per_cu;
-    const int tiles_per_wg = (n_tiles + grid - 1) / grid;
+    int grid = n_dealt < cus * per_cu ? n_dealt : cus * per_cu;
+    const int tiles_per_wg = (p.gated ? 2 : 1) * ((n_dealt + grid - 1) / grid);
     // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time only
     // when the workgroup gathers from it for several tiles.
     const bool repl = p.entries <= 256 && tiles_per_wg >= 4;
@@ -376,13 +396,14 @@ hipError_t launch_decode_steps(const ProblemB &p, hipStream_t s)
     }
     if ((size_t)per_cu * smem > kDecodeLdsLimit) {
         per_cu = (int)(kDecodeLdsLimit / smem) > 0 ? (int)(kDecodeLdsLimit / smem) : 1;
-        grid = n_tiles < cus * per_cu ? n_tiles : cus * per_cu;
+        grid = n_dealt < cus * per_cu ? n_dealt : cus * per_cu;
     }
     auto kern = repl ? decode_general_kernel<VEC, CodeT, STEPS, true> : decode_general_kernel<VEC, CodeT, STEPS, false>;
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(n_waves * 64), smem, s, p.x, static_cast<const CodeT *>(p.codes), p.cb,
-                       p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb, n_tiles / grid, n_tiles % grid, n_chunks, stage_off, aliased);
+                       p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb, n_dealt / grid, n_dealt % grid, n_chunks, stage_off, aliased,
+                       p.gated ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -413,6 +434,8 @@ constexpr size_t kDecodeLdsBudget = 144 * 1024;  // codebook + reduction slots m
 bool decode_general_supports(const ProblemB &p)
 {
     if (p.M < 1 || p.N < 1 || p.K < 1) return false;
+    // gated: whole pairs of a gate and an up tile (a pair may lie in two codebooks: the table is picked per tile)
+    if (p.gated && p.N % (2 * kTileN) != 0) return false;
     if (p.vec != 2 && p.vec != 4 && p.vec != 8) return false;
     if (p.n_codebooks > 1 && p.rows_per_cb % kTileN != 0) return false;
     if ((size_t)p.entries * p.vec * 2 + 2 * kMaxWaves * 1024 > kDecodeLdsBudget) return false;

@@ -83,19 +83,15 @@ def _silu_mul_fake(gate_up):
 def vq_gated_linear(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor,
                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x @ Wg.T) * (x @ Wu.T) in one fused VQ GEMM: `codes` [2H, K/vec] hold the gate and the up rows
-    interleaved in groups of 16 (`vq_gemm_amd.quantize.interleave_gate_up`), the result is fp16 [..., H].  Short
-    inputs that the K-sliced decode kernels would take run as the plain product plus the element-wise pass."""
+    interleaved in groups of 16 (`vq_gemm_amd.quantize.interleave_gate_up`), the result is fp16 [..., H].  Every
+    fused kernel carries the epilogue, so no call allocates a workspace."""
     shape = _out_shape(x, codes, codebook)
     if x.dtype != torch.float16 or codebook.dtype != torch.float16:
         raise ValueError("vq_gated_linear: x and codebook must be float16")
     if codes.shape[0] % 32 != 0:
         raise ValueError("vq_gated_linear: the interleaved gate/up rows come in whole groups of 32")
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
-    workspace = None
-    if 1 < x2.shape[0] <= 64:   # where a decode kernel would run the plain product
-        workspace = torch.empty((x2.shape[0], codes.shape[0]), dtype=torch.float16, device=x.device)
-    y = cabi.e2e_gemm_b_gated(x2, codes.contiguous(), codebook.contiguous(), bias=None if bias is None else bias.contiguous(),
-                              workspace=workspace)
+    y = cabi.e2e_gemm_b_gated(x2, codes.contiguous(), codebook.contiguous(), bias=None if bias is None else bias.contiguous())
     return y.view(*shape[:-1], shape[-1] // 2)
 
 
