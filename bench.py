@@ -37,9 +37,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 FP16_MFMA_PEAK_TFLOPS = 2500.0
-POOL_BYTES = 640 << 20  # distinct code matrices rotated through by the bandwidth-bound configs
-EVICT_BYTES = 512 << 20  # source and destination of the device copy that empties the caches
-MIN_TIMED_LAUNCHES = 200  # a microsecond-scale kernel is never timed over fewer launches than this
+from vq_gemm_amd.timing import MIN_TIMED_LAUNCHES, POOL_BYTES  # the cold-HBM protocol's pool size and minimum count
 # HBM bytes one cold decode launch moves: NOT measured by this program.  From rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE of `bench.py --probe C2`, scaled by a 256 MiB copy in the same run
 # (1104.1 KiB x 2.0 read + 8 KiB written); the summary and its command are in the file named here.
@@ -61,6 +59,9 @@ def parse_args():
                          "device copy as a counter yardstick; prints no JSON")
     ap.add_argument("--probe-variant", type=int, default=0,
                     help="with --probe on a geometry-B shape: the VQGEMM_VARIANT_* value to launch (0 = automatic choice)")
+    ap.add_argument("--probe-set", action="append", default=[], metavar="NAME=VALUE",
+                    help="with --probe: set a constant of the tuning table first (a kernel parameter candidate, e.g. "
+                         "gemv_wide_groups_in_flight=3), for counter runs on one candidate")
     ap.add_argument("--probe-skew", type=float, default=1.0,
                     help="with --probe on a geometry-B shape: codes = floor(entries * u^P) for uniform u; 1 = uniform codes (the "
                          "measured configurations), larger P concentrates the codes on few 'hot' entries (P = 4: half of all "
@@ -135,6 +136,9 @@ def main():
 
     if args.probe:
         from vq_gemm_amd.problems import GEOM_A, GEOM_B, ProblemSpec
+        for item in args.probe_set:
+            name, value = item.split("=", 1)
+            cabi.set_tuning(**{name: float(value)})
         if args.probe.startswith("GEMM,"):
             m, k, n = (int(v) for v in args.probe.split(",")[1:])
             g = torch.Generator().manual_seed(42)
@@ -208,56 +212,8 @@ def main():
               file=sys.stderr)
         return
 
-    evict = {}
-
-    def evict_caches(stream):
-        """A device copy larger than L2 + Infinity Cache on `stream`: what was cached before it is gone after."""
-        if not evict:
-            evict["src"] = torch.empty(EVICT_BYTES, dtype=torch.uint8, device=dev).random_()
-            evict["dst"] = torch.empty(EVICT_BYTES, dtype=torch.uint8, device=dev)
-        with torch.cuda.stream(stream):
-            evict["dst"].copy_(evict["src"])
-
-    def time_launches(launch, n_bufs, steps, warmup, chunk=500, min_launches=MIN_TIMED_LAUNCHES):
-        """(average seconds per launch, launches timed) of `launch(i)`, i rotating over n_bufs buffers.
-
-        HIP graphs + events on the launch stream.  The timed region is `steps` launches repeated until it
-        covers two full rotations of the pool and at least `min_launches` launches, so that what is measured does
-        not depend on --steps; launch i always reads buffer i % n_bufs, so that two reads of a buffer lie a
-        whole pool apart.  Every graph is replayed once untimed (the first replay uploads it), then the
-        caches are emptied, then all graphs are replayed between two events.
-        """
-        n_timed = steps * max(1, -(-max(2 * n_bufs if n_bufs > 1 else 0, min_launches) // steps))
-        stream = torch.cuda.Stream()   # default priority
-        with torch.cuda.stream(stream):
-            for i in range(max(warmup, 1)):
-                launch(i % n_bufs)
-            stream.synchronize()
-            graphs = []
-            done = 0
-            while done < n_timed:
-                c = min(chunk, n_timed - done)
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g, stream=stream):
-                    for i in range(c):
-                        launch((done + i) % n_bufs)
-                graphs.append(g)
-                done += c
-            for g in graphs:            # first replay uploads a graph: keep it out of the timing
-                g.replay()
-            stream.synchronize()
-            if n_bufs > 1:
-                evict_caches(stream)
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            barrier()
-            e0.record(stream)
-            for g in graphs:
-                g.replay()
-            e1.record(stream)
-            e1.synchronize()
-            barrier()
-            return e0.elapsed_time(e1) * 1e-3 / n_timed, n_timed
+    # the cold-HBM timing protocol (rotating pool, graphs, events on the launch stream) lives in the package
+    from vq_gemm_amd.timing import time_launches
 
     def bench_config(name, steps, warmup, cold_pool):
         spec = CONFIGS[name] if isinstance(name, str) else name

@@ -900,6 +900,50 @@ def test_tune_fit_returns_the_table_and_the_library_takes_it():
     assert cabi.select_variant_b(16, 4096, 11008, 4, 4096, 1, 16) == cabi.VARIANT_DECODE
 
 
+def test_tune_search_tries_the_kernel_parameter_candidates_cold_and_the_library_takes_the_winners():
+    import math
+    from vq_gemm_amd import tune
+    before = cabi.tuning()
+    found = tune.search(verbose=False, quick=True)
+    assert set(found) == set(before) and all(math.isfinite(v) for v in found.values())
+    _say("  searched: " + ", ".join(f"{k}={found[k]:g}" for k in sorted(found) if found[k] != before[k]))
+    _say("  report:", tune.search.last_report)
+    # candidates stay inside what the kernels are built for
+    assert found["gemv_wide_rows_per_group"] in (1.0, 2.0) and found["gemv_wide_groups_in_flight"] in (2.0, 3.0)
+    assert found["gemv_wide_rows_per_group_long_k"] in (1.0, 2.0) and found["gemv_wide_groups_in_flight_long_k"] in (2.0, 3.0)
+    assert cabi.tuning() == before, "the search leaves the table as it found it"
+    # every candidate of the wide form's loop gives the same bits as the default (same sums in the same order per row)
+    spec = ProblemSpec("cand", GEOM_B, 1, 4096, 12288, 8, 256, 3, 8, codebook_3d=True)
+    x, codes, cb = make_problem(spec, seed=81, device=DEV)
+    want = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV).clone()
+    _check_gemm(want, x, codes, cb, what="wide GEMV, default loop")
+    try:
+        for g in (1, 2):
+            for nbuf in (2, 3):
+                for runs in (0, 1e6):
+                    cabi.set_tuning(gemv_wide_rows_per_group=g, gemv_wide_groups_in_flight=nbuf, gemv_wide_plain_table_max_runs=runs)
+                    assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), want), (g, nbuf, runs)
+        # beyond K = 4096, plain and gated (one group of two rows, or the gate and the up row as two groups in turn)
+        spec8 = ProblemSpec("cand8", GEOM_B, 1, 8192, 8192, 8, 256, 1, 8)
+        x8, codes8, cb8 = make_problem(spec8, seed=82, device=DEV)
+        want8 = vo.gated_gemm_b(_np(x8), _np(codes8), _np(cb8)).astype(np.float64)
+        plain8 = None
+        for g, nbuf in ((1, 2), (1, 3), (2, 2)):
+            cabi.set_tuning(gemv_wide_rows_per_group_long_k=g, gemv_wide_groups_in_flight_long_k=nbuf)
+            yp = cabi.e2e_gemm_b(x8, codes8, cb8, variant=cabi.VARIANT_DECODE_GEMV).clone()
+            plain8 = yp if plain8 is None else plain8
+            assert torch.equal(yp, plain8), (g, nbuf)
+            e1, e2 = vo.rel_err(_np(cabi.e2e_gemm_b_gated(x8, codes8, cb8, variant=cabi.VARIANT_DECODE_GEMV)), want8)
+            assert e2 <= TOL and e1 <= 2 * TOL, (g, nbuf, e1, e2)
+        _check_gemm(plain8, x8, codes8, cb8, what="wide GEMV, K=8192")
+        cabi.set_tuning(**found)
+        assert cabi.tuning() == found
+        y = cabi.e2e_gemm_b(x, codes, cb)
+        _check_gemm(y, x, codes, cb, what="automatic choice under the searched table")
+    finally:
+        cabi.set_tuning(**before)
+
+
 # shapes the tiled kernel takes (K a multiple of 64, N of 8): few tiles -> 128x128
 # tiles (the first three and the fifth), about one 256x128 tile per compute unit -> those (the seventh and eighth),
 # more -> 256x256 tiles (the fourth and the sixth); ragged M and N

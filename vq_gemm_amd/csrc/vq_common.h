@@ -180,11 +180,19 @@ struct Tuning {
     // GEMV kernels: the four-wave kernel up to this many 16-row tiles per unit and this K; the wide form from this
     // many rows per wave on
     double gemv_max_tiles_per_cu = 4.0;
-    double gemv_max_k = 6144.0;
-    double gemv_wide_min_rows_per_wave = 1.0;
+    double gemv_max_k = 8192.0;
+    double gemv_wide_min_rows_per_wave = 0.5;
     // the wide form gathers from the plain 4 KB table while a wave's rows are at most this many runs of 2048 k, from the
     // bank-replicated one (64 KB to fill) beyond
     double gemv_wide_plain_table_max_runs = 2.0;
+    // the wide form's loop: rows of W per group (1 or 2) and groups of codes in flight (2 or 3), for K up to 4096
+    // and beyond
+    double gemv_wide_rows_per_group = 2.0;
+    double gemv_wide_groups_in_flight = 2.0;
+    double gemv_wide_rows_per_group_long_k = 1.0;
+    double gemv_wide_groups_in_flight_long_k = 2.0;
+    // batched decode kernel: the bank-replicated table (64 KB to fill) from this many tiles per workgroup on
+    double decode_replicated_table_min_tiles = 2.0;
     // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums
     // written and read once (microseconds per MB of partial sums)
     double splitk_fixed_us = 4.5;

@@ -629,9 +629,6 @@ __global__ __launch_bounds__(1024) void decode_batched_kernel(const half_t *__re
     }
 }
 
-#ifndef VQ_REPL_MIN
-#define VQ_REPL_MIN 2
-#endif
 constexpr size_t kDecodeLdsLimit = 160 * 1024;
 constexpr size_t kDisjointBudget = 80 * 1024;  // keep two workgroups per CU when staging beside the codebook
 
@@ -695,7 +692,7 @@ BatchedPlan plan_batched(const ProblemB &p)
         const size_t carry = g.n_chunks > 1 ? (size_t)units * tb * carry_bytes : 0;
         // Replicated codebook (one 256-byte bank row per entry, <= 64 KB): worth its fill time as
         // soon as the workgroup gathers from it for more than one tile, where it fits.
-        for (int repl = (p.entries <= 256 && g.tiles_per_wg >= VQ_REPL_MIN) ? 1 : 0; repl >= 0; repl--) {
+        for (int repl = (p.entries <= 256 && (double)g.tiles_per_wg >= tuning().decode_replicated_table_min_tiles) ? 1 : 0; repl >= 0; repl--) {
             const size_t table = repl ? (size_t)p.entries * 256 : plain;
             g.repl = repl != 0;
             g.acc_off = g.n_chunks > 1 ? (int)table : -1;
@@ -899,7 +896,7 @@ double decode_cost_us(const ProblemB &p)
 
 // The GEMV kernels have no work shared between their waves.  One row of X in the first format
 // (8-vectors, 8-bit codes, at most two codebooks per workgroup's share of the rows) goes to the wide
-// form from one row per wave on (4096 rows on a 256-CU device): measured against the batched kernel
+// form from half a row per wave on (2048 rows on a 256-CU device; Tuning::gemv_wide_min_rows_per_wave): measured against the batched kernel
 // on a 256-CU MI355X, cold HBM, K = 4096: N = 4096 4.96 -> 3.4 us, N = 16384 7.5 -> 5.1, N = 28672
 // 9.9 -> 7.1, N = 65536 15.6 -> 12.4; K = 8192: N = 8192 8.3 -> 5.6, N = 28672 18.3 -> 10.8.
 // The four-wave kernel takes what is left where it was measured faster than the batched kernel

@@ -19,7 +19,7 @@
 // Four waves per workgroup, 16 rows of W: as many workgroups as the batched kernel has tiles.  It
 // serves two to four rows of X, the other code formats and launches with fewer rows than the device
 // has waves; one row of X in the first format goes to the wide form below (decode_gemv_wide_kernel)
-// from one row per wave on.
+// from half a row per wave on (Tuning::gemv_wide_min_rows_per_wave).
 #include "vq_common.h"
 
 #include <limits.h>
@@ -29,14 +29,8 @@ namespace vq {
 
 namespace {
 
-#ifndef VQ_GEMV_WAVES
-#define VQ_GEMV_WAVES 4
-#endif
-#ifndef VQ_GEMV_ROWS
-#define VQ_GEMV_ROWS 4
-#endif
-constexpr int kGemvWaves = VQ_GEMV_WAVES;
-constexpr int kGemvRows = VQ_GEMV_ROWS;                     // rows of W per wave
+constexpr int kGemvWaves = 4;
+constexpr int kGemvRows = 4;                                // rows of W per wave
 typedef _Float16 gemv_out_t __attribute__((ext_vector_type(kGemvRows)));
 constexpr int kGemvTile = kGemvWaves * kGemvRows;           // rows of W per workgroup
 constexpr int kRunCodes = 256;                              // codes of a row one wave load covers
@@ -214,7 +208,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     }
 }
 
-// ---- the wide form: long runs of rows, and every single-row launch of at least one row per wave -------
+// ---- the wide form: long runs of rows, and every single-row launch of at least half a row per wave -------
 // One workgroup of sixteen waves per compute unit over a bank-replicated table (64 KB: 16 copies of
 // each entry in one 256-byte bank row, lane l reading copy l % 16, so the gathers never collide):
 // four waves per SIMD cover the latency of each other's gathers.  One row of X, 8-vectors, 8-bit codes.
@@ -516,18 +510,19 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 
 }  // namespace
 
-#ifndef VQ_GEMV_WIDE_G
-#define VQ_GEMV_WIDE_G 2
-#endif
-#ifndef VQ_GEMV_WIDE_NBUF
-#define VQ_GEMV_WIDE_NBUF 2
-#endif
-#ifndef VQ_GEMV_WIDE_G4
-#define VQ_GEMV_WIDE_G4 1
-#endif
-#ifndef VQ_GEMV_WIDE_NBUF4
-#define VQ_GEMV_WIDE_NBUF4 2
-#endif
+// Rows per group (1 or 2) and groups of codes in flight (2 or 3) of the wide form are runtime choices out of the
+// tuning table, separately for K up to 4096 and beyond: `python -m vq_gemm_amd.tune --search` times the four
+// combinations on the box at hand, on codes that come from HBM.
+static int wide_rows_per_group(const ProblemB &p)
+{
+    const Tuning &tn = tuning();
+    return (p.K / kRunK > 2 ? tn.gemv_wide_rows_per_group_long_k : tn.gemv_wide_rows_per_group) >= 2.0 ? 2 : 1;
+}
+static int wide_groups_in_flight(const ProblemB &p)
+{
+    const Tuning &tn = tuning();
+    return (p.K / kRunK > 2 ? tn.gemv_wide_groups_in_flight_long_k : tn.gemv_wide_groups_in_flight) >= 3.0 ? 3 : 2;
+}
 
 // One row of X, 8-vectors, 8-bit codes, K a multiple of 2048 up to 8192, and no workgroup's share of
 // the rows reaching into more than two codebooks.
@@ -538,8 +533,7 @@ bool decode_gemv_wide_supports(const ProblemB &p)
     const int waves = device_cu_count() * kWideWaves;
     if (p.gated) {
         // two code rows per output: one group of two rows, or two groups of one
-        const int g = p.K / kRunK > 2 ? VQ_GEMV_WIDE_G4 : VQ_GEMV_WIDE_G;
-        if (p.N % 32 != 0 || g > 2) return false;
+        if (p.N % 32 != 0) return false;
         const int outs_per_wave = (p.N / 2 + waves - 1) / waves;
         if (outs_per_wave > 32) return false;
         // a workgroup's rows of W: its outputs' gate and up rows, in whole groups of 32
@@ -580,12 +574,25 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
              : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1, kWideCopies>) : launch(decode_gemv_wide_kernel<R, GG, NB, 2, kWideCopies>);
     };
     using std::integral_constant;
-    switch (p.K / kRunK) {
-    case 1: return pick(integral_constant<int, 1>{}, integral_constant<int, VQ_GEMV_WIDE_G>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF>{});
-    case 2: return pick(integral_constant<int, 2>{}, integral_constant<int, VQ_GEMV_WIDE_G>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF>{});
-    case 3: return pick(integral_constant<int, 3>{}, integral_constant<int, VQ_GEMV_WIDE_G4>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF4>{});
-    default: return pick(integral_constant<int, 4>{}, integral_constant<int, VQ_GEMV_WIDE_G4>{}, integral_constant<int, VQ_GEMV_WIDE_NBUF4>{});
-    }
+    auto pick_runs = [&](auto g_c, auto nbuf_c) {
+        switch (p.K / kRunK) {
+        case 1: return pick(integral_constant<int, 1>{}, g_c, nbuf_c);
+        case 2: return pick(integral_constant<int, 2>{}, g_c, nbuf_c);
+        default: break;
+        }
+        // (two rows per group with three groups in flight do not fit the registers beyond K = 4096: not built)
+        if constexpr (decltype(g_c)::value * decltype(nbuf_c)::value <= 4) {
+            if (p.K / kRunK == 3) return pick(integral_constant<int, 3>{}, g_c, nbuf_c);
+            return pick(integral_constant<int, 4>{}, g_c, nbuf_c);
+        }
+        return hipErrorInvalidValue;
+    };
+    const int g = wide_rows_per_group(p);
+    const int nbuf = (g == 2 && p.K / kRunK > 2) ? 2 : wide_groups_in_flight(p);
+    if (g == 2) return nbuf == 3 ? pick_runs(integral_constant<int, 2>{}, integral_constant<int, 3>{})
+                                 : pick_runs(integral_constant<int, 2>{}, integral_constant<int, 2>{});
+    return nbuf == 3 ? pick_runs(integral_constant<int, 1>{}, integral_constant<int, 3>{})
+                     : pick_runs(integral_constant<int, 1>{}, integral_constant<int, 2>{});
 }
 
 bool decode_gemv_wide_preferred(const ProblemB &p);

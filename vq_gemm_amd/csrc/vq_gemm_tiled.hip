@@ -644,9 +644,6 @@ hipError_t launch_gemm_tiled(const half_t *x, const half_t *w, half_t *y, int M,
                              int tile)
 {
     if (!gemm_tiled_supports(x, w, M, K, N, w_is_kn)) return hipErrorInvalidValue;
-#ifdef VQ_FORCE_TILE
-    tile = VQ_FORCE_TILE;   // measurement builds only
-#endif
     if (tile == 0) {
         // Rounds of tiles over the compute units.  A tile costs K/64 times a per-stage time that
         // grows with the share of the units at work (the clock drops under load): fitted to

@@ -164,9 +164,6 @@ __device__ __forceinline__ void split_codebooks(uint8_t *lds, uint32_t src, uint
 // whether a tile's codebooks can take the split layout, given the bytes free for the plain copy
 inline bool split_layout_applies(const ProblemB &p, int codebooks, size_t temp_bytes)
 {
-#ifdef VQ_NO_SPLIT
-    return false;
-#endif
     return p.vec == 8 && p.code_bits == 8 && p.entries == (int)kSplitEntries && (size_t)codebooks * 2 * kSplitHi <= temp_bytes;
 }
 

@@ -4,7 +4,15 @@
 
 or measures the box at hand and refits the constants of the cost models behind the automatic choice:
 
-    python -m vq_gemm_amd.tune --fit [--write [PATH]]
+    python -m vq_gemm_amd.tune --fit [--search] [--write [PATH]]
+    python -m vq_gemm_amd.tune --search [--write [PATH]]
+
+`--search` tries the candidates of the kernels' run-time parameters - rows per group and groups of codes in flight
+of the wide GEMV kernel, plain against bank-replicated table, the limits between the GEMV kernels and the K-sliced
+decode kernels, the tile count from which the batched decode kernel replicates its table - on codes that come from
+HBM (the rotating-pool protocol of `vq_gemm_amd.timing`, the one `bench.py` times with), and keeps the winners.
+A counter run on one candidate: `rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_WAIT_ANY -- python3 bench.py --probe
+M,K,N,vec,entries,bits --probe-set name=value` launches the shape with that constant set.
 
 `--fit` times forced variants on a fixed set of shapes (per-stage and per-tile times come out of pairs of
 shapes that differ in K or in the number of tiles), prints the fitted constants next to the compiled-in
@@ -197,9 +205,9 @@ def fit(device: str = "cuda:0", verbose: bool = True) -> dict:
         out["splitk_us_per_partial_mb"] = per_mb
         out["splitk_fixed_us"] = max(small[0] - per_mb * small[1], 0.5)
         say(f"split K, two slices: {small[0]:.2f} us beyond the multiplying at {small[1]:.1f} MB of partial sums, {large[0]:.2f} us at {large[1]:.1f} MB")
-    # (gemv_wide_min_rows_per_wave, gemv_wide_plain_table_max_runs and gemv_max_k keep their values: the wide form wins its short launches on codes that
-    # come from HBM and loses them on cached ones - 3.3 against 3.5 us cold, 3.2 against 2.7 us warm on C2 - and this
-    # loop times warm launches; bench.py's rotating pool is the protocol that decides them.)
+    # (the limits between the GEMV kernels and the kernels' run-time parameters are decided by launches on codes that
+    # come from HBM - the wide form wins its short launches cold and loses them warm - and this function times warm
+    # launches: `search` below covers them)
     if verbose:
         print("constant                          compiled-in / current -> fitted")
         for k in out:
@@ -207,10 +215,175 @@ def fit(device: str = "cuda:0", verbose: bool = True) -> dict:
     return out
 
 
+def _cold_us(M, K, N, variant=None, vec=8, entries=256, n_codebooks=1, code_bits=8, device="cuda:0", steps=50, repeats=3,
+             **constants):
+    """Microseconds per launch on codes from HBM (rotating pool; the median of `repeats` timed regions), with
+    `constants` set in the tuning table for the duration; None when the variant refuses the shape."""
+    from . import timing
+    variant = cabi.VARIANT_AUTO if variant is None else variant
+    spec = ProblemSpec("search", GEOM_B, M, K, N, vec, entries, n_codebooks, code_bits)
+    x, codes, cb = make_problem(spec, seed=1, device=device)
+    pool = timing.code_pool(spec, timing.pool_size(spec.code_bytes), first=codes, device=device)
+    y = torch.empty(M, N, dtype=torch.float16, device=device)
+    before = cabi.tuning()
+    try:
+        cabi.set_tuning(**constants)
+        try:
+            cabi.e2e_gemm_b(x, pool[0], cb, out=y, variant=variant)
+        except cabi.VqGemmError as e:
+            if e.code != -4:
+                raise
+            return None
+        ts = sorted(timing.time_launches(lambda i: cabi.e2e_gemm_b(x, pool[i], cb, out=y, variant=variant), len(pool), steps, 20,
+                                         device=device)[0] for _ in range(repeats))
+        return ts[len(ts) // 2] * 1e6
+    finally:
+        cabi.set_tuning(**{k: before[k] for k in constants})
+        del pool
+
+
+def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, margin: float = 0.02) -> dict:
+    """Times the candidates of the kernels' run-time parameters on cold code matrices and returns the table with the
+    winners in it.  `quick` leaves out the largest shapes (for tests).  A candidate replaces the value in force only
+    when it is ahead by more than `margin` (as a share of the time): differences inside the noise change nothing."""
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    waves = 16 * cus  # the wide GEMV kernel's waves on the device
+    cur = cabi.tuning()
+    out = dict(cur)
+    report = {}
+    say = print if verbose else (lambda *a, **k: None)
+    GEMV, DEC = cabi.VARIANT_DECODE_GEMV, cabi.VARIANT_DECODE
+    force_wide = dict(gemv_wide_min_rows_per_wave=0.0)
+
+    # 1. the wide form's loop: (rows per group, groups in flight), K up to 4096 and beyond
+    def loop_search(tag, names, shapes):
+        totals = {}
+        for g in (1, 2):
+            for nbuf in (2, 3):
+                if g * nbuf > 4 and any(K > 4096 for (K, _, _) in shapes):
+                    continue   # (not built: two rows per group with three groups in flight beyond K = 4096)
+                ts = [_cold_us(1, K, N, GEMV, n_codebooks=G, device=device, **force_wide, **{names[0]: g, names[1]: nbuf})
+                      for (K, N, G) in shapes]
+                if all(t is not None for t in ts):
+                    totals[(g, nbuf)] = ts
+        if not totals:
+            return
+        # each shape counts alike: sum of times relative to the shape's best candidate
+        best_of = [min(ts[i] for ts in totals.values()) for i in range(len(shapes))]
+        score = {c: sum(t / b for t, b in zip(ts, best_of)) for c, ts in totals.items()}
+        win = min(score, key=score.get)
+        now = (int(cur[names[0]]), int(cur[names[1]]))
+        if now in score and score[now] <= score[win] * (1.0 + margin):
+            win = now
+        out[names[0]], out[names[1]] = float(win[0]), float(win[1])
+        report[tag] = {f"g{c[0]}_nbuf{c[1]}": [round(t, 3) for t in ts] for c, ts in totals.items()}
+        say(f"wide GEMV loop, {tag}: " + "; ".join(f"G={c[0]} NBUF={c[1]}: " + "/".join(f"{t:.2f}" for t in ts) for c, ts in totals.items())
+            + f" us on {shapes} -> G={win[0]} NBUF={win[1]}")
+    loop_search("K<=4096", ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight"),
+                [(4096, waves, 1), (4096, 3 * waves, 3)] + ([] if quick else [(4096, 7 * waves, 1), (2048, 4 * waves, 1)]))
+    loop_search("K>4096", ("gemv_wide_rows_per_group_long_k", "gemv_wide_groups_in_flight_long_k"),
+                [(8192, 2 * waves, 1)] + ([] if quick else [(8192, 7 * waves, 1), (6144, 4 * waves, 1)]))
+    loop_now = {k: out[k] for k in ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight", "gemv_wide_rows_per_group_long_k",
+                                    "gemv_wide_groups_in_flight_long_k")}
+
+    # 2. plain against bank-replicated table: the threshold in gathers per lane (rows per wave x runs of 2048 k)
+    rows = []
+    for (K, N) in [(2048, waves), (4096, waves), (4096, 2 * waves), (8192, waves)] + ([] if quick else [(2048, 2 * waves), (8192, 2 * waves)]):
+        runs = (N // waves) * (K // 2048)
+        tp = _cold_us(1, K, N, GEMV, device=device, **force_wide, **loop_now, gemv_wide_plain_table_max_runs=1e6)
+        tr = _cold_us(1, K, N, GEMV, device=device, **force_wide, **loop_now, gemv_wide_plain_table_max_runs=0.0)
+        if tp is not None and tr is not None:
+            rows.append((runs, tp, tr))
+            say(f"wide GEMV table, K={K} N={N} ({runs} runs per wave): plain {tp:.2f} us, replicated {tr:.2f} us")
+    if rows:
+        cands = sorted({0.0} | {float(r[0]) for r in rows})
+        cost = {c: sum(tp if runs <= c else tr for runs, tp, tr in rows) for c in cands}
+        out["gemv_wide_plain_table_max_runs"] = min(cost, key=cost.get)
+        report["plain_table"] = [(r, round(a, 3), round(b, 3)) for r, a, b in rows]
+
+    # 3. wide form against the four-wave form: from how many rows per wave on the wide form wins
+    limit = None
+    fracs = (0.25, 0.5, 0.75, 1.0)
+    wins = []
+    for f in fracs:
+        N = int(waves * f) // 16 * 16
+        tw = _cold_us(1, 4096, N, GEMV, device=device, **loop_now, gemv_wide_plain_table_max_runs=out["gemv_wide_plain_table_max_runs"],
+                      gemv_wide_min_rows_per_wave=0.0)
+        t4 = _cold_us(1, 4096, N, GEMV, device=device, gemv_wide_min_rows_per_wave=1e6)
+        if tw is None or t4 is None:
+            continue
+        say(f"one row of X, K=4096, N={N} ({f} rows per wave): wide {tw:.2f} us, four-wave {t4:.2f} us")
+        wins.append((f, tw <= t4 * (1.0 - margin)))
+    for f, won in reversed(wins):   # the smallest share from which the wide form wins all the way up
+        if not won:
+            break
+        limit = f
+    if limit is not None:
+        out["gemv_wide_min_rows_per_wave"] = limit
+    report["wide_vs_four_wave"] = wins
+
+    # 4. four-wave GEMV against the batched K-sliced kernel in a format the wide form does not take: tiles per unit, K
+    best_tiles = 0.0
+    for tiles in (1, 2, 4, 8) if not quick else (1, 2):
+        tg = _cold_us(1, 4096, 16 * cus * tiles, GEMV, vec=4, device=device)
+        td = _cold_us(1, 4096, 16 * cus * tiles, DEC, vec=4, device=device)
+        if tg is None or td is None:
+            break
+        say(f"one row of X, 4-vectors, {tiles} tile(s) per unit: four-wave GEMV {tg:.2f} us, batched {td:.2f} us")
+        if tg > td:
+            break
+        best_tiles = float(tiles)
+    out["gemv_max_tiles_per_cu"] = best_tiles
+    best_k = 0.0
+    for K in (2048, 4096, 6144, 8192):
+        won = []
+        for tiles in (1, 2):
+            tg = _cold_us(1, K, 16 * cus * tiles, GEMV, vec=4, device=device)
+            td = _cold_us(1, K, 16 * cus * tiles, DEC, vec=4, device=device)
+            if tg is None or td is None:
+                continue
+            say(f"one row of X, 4-vectors, {tiles} tile(s) per unit, K={K}: four-wave GEMV {tg:.2f} us, batched {td:.2f} us")
+            won.append(tg <= td)
+        if won and all(won):
+            best_k = float(K)
+    if best_k:
+        out["gemv_max_k"] = best_k
+
+    # 5. batched decode kernel: from how many tiles per workgroup the replicated table pays (16 rows of X)
+    rows = []
+    for tiles in (1, 2, 3, 4):
+        tp = _cold_us(16, 4096, 16 * cus * tiles, DEC, device=device, decode_replicated_table_min_tiles=1e6)
+        tr = _cold_us(16, 4096, 16 * cus * tiles, DEC, device=device, decode_replicated_table_min_tiles=0.0)
+        if tp is None or tr is None:
+            continue
+        say(f"batched decode, {tiles} tile(s) per workgroup: plain table {tp:.2f} us, replicated {tr:.2f} us")
+        rows.append((tiles, tp, tr))
+    if rows:
+        cands = [1.0, 2.0, 3.0, 4.0, 5.0]
+        cost = {c: sum(tr if tiles >= c else tp for tiles, tp, tr in rows) for c in cands}
+        out["decode_replicated_table_min_tiles"] = min(cost, key=cost.get)
+        report["decode_table"] = [(t, round(a, 3), round(b, 3)) for t, a, b in rows]
+
+    if verbose:
+        print("constant                          current -> searched")
+        for k in out:
+            if out[k] != cur[k]:
+                print(f"  {k:36s} {cur[k]:8.3f} -> {out[k]:8.3f}")
+    out_report = dict(out)
+    search.last_report = report
+    return out_report
+
+
+search.last_report = {}
+
+
 def main(argv) -> int:
-    if argv and argv[0] == "--fit":
+    if argv and argv[0] in ("--fit", "--search"):
         import json
-        fitted = fit()
+        fitted = fit() if "--fit" in argv else cabi.tuning()
+        if "--search" in argv:
+            cabi.set_tuning(**fitted)
+            fitted = search()
         if "--write" in argv:
             i = argv.index("--write")
             path = argv[i + 1] if len(argv) > i + 1 else cabi.TUNING_FILE
