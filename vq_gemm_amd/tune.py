@@ -1,6 +1,9 @@
 """Times every kernel variant on one geometry-B shape and shows what the automatic choice picks:
 
-    python -m vq_gemm_amd.tune M K N [vec entries codebooks code_bits]
+    python -m vq_gemm_amd.tune [--cold] M K N [vec entries codebooks code_bits]
+
+(`--cold`: every launch reads a code matrix that comes from HBM - the rotating pool of `vq_gemm_amd.timing` - instead
+of one that sits in the caches)
 
 or measures the box at hand and refits the constants of the cost models behind the automatic choice:
 
@@ -59,6 +62,24 @@ def time_graph(fn, launches: int = 20, repeats: int = 3) -> float:
             e1.synchronize()
             best = min(best, e0.elapsed_time(e1) / launches * 1e3)
     return best
+
+
+def tune_cold(M: int, K: int, N: int, vec: int = 8, entries: int = 256, n_codebooks: int = 1, code_bits: int = 8,
+              device: str = "cuda:0", verbose: bool = True) -> dict:
+    """Microseconds per launch of every variant that takes the shape, on codes that come from HBM."""
+    times = {}
+    for variant in (cabi.VARIANT_AUTO, cabi.VARIANT_DECODE, cabi.VARIANT_DECODE_GEMV, cabi.VARIANT_PREFILL, cabi.VARIANT_PREFILL_NARROW,
+                    cabi.VARIANT_PREFILL_SMALL):
+        t = _cold_us(M, K, N, variant, vec=vec, entries=entries, n_codebooks=n_codebooks, code_bits=code_bits, device=device)
+        if t is not None:
+            times[cabi.VARIANT_NAMES[variant]] = t
+    picked = cabi.VARIANT_NAMES[cabi.select_variant_b(M, K, N, vec, entries, n_codebooks, code_bits)]
+    if verbose:
+        print(f"M={M} K={K} N={N} vec={vec} entries={entries} codebooks={n_codebooks} code_bits={code_bits}, cold code matrices")
+        for v, t in times.items():
+            print(f"  {v:15s} {t:9.2f} us")
+        print(f"  automatic choice: {picked}")
+    return {"times_us": times, "auto_picks": picked}
 
 
 def tune(M: int, K: int, N: int, vec: int = 8, entries: int = 256, n_codebooks: int = 1, code_bits: int = 8,
@@ -391,11 +412,13 @@ def main(argv) -> int:
                 json.dump({"device": torch.cuda.get_device_name(0), **fitted}, f, indent=1)
             print("wrote", path)
         return 0
+    cold = "--cold" in argv
+    argv = [a for a in argv if a != "--cold"]
     if len(argv) not in (3, 7):
         print(__doc__)
         return 2
     vals = [int(a) for a in argv]
-    tune(*vals)
+    (tune_cold if cold else tune)(*vals)
     return 0
 
 
