@@ -191,6 +191,8 @@ struct Tuning {
     double gemv_wide_groups_in_flight = 2.0;
     double gemv_wide_rows_per_group_long_k = 1.0;
     double gemv_wide_groups_in_flight_long_k = 2.0;
+    // the wide form's waves step their issue priority round with every group (1) or leave it alone (0)
+    double gemv_wide_rotate_priority = 1.0;
     // batched decode kernel: the bank-replicated table (64 KB to fill) from this many tiles per workgroup on
     double decode_replicated_table_min_tiles = 2.0;
     // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums

@@ -290,7 +290,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
                                                                            const half_t *__restrict__ bias, int entries,
                                                                            int rows_q, int rows_r, int rows_per_cb,
                                                                            float rcp_rows_per_cb, int n_books, int n_total,
-                                                                           int gated)
+                                                                           int gated, int rotate_priority)
 {
     // gated: the epilogue of a gate/up pair.  The rows of W are gate and up rows interleaved in groups of 16; what
     // is dealt out to the waves (rows_q, rows_r, n_total) are then the N/2 outputs, a wave's code rows are the gate
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     // All kernel arguments are fetched at once: left to first use, each pointer costs the prologue a
     // scalar-load round trip of its own.
     asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(bias), "s"(entries), "s"(rows_q), "s"(rows_r), "s"(rows_per_cb),
-                 "s"(rcp_rows_per_cb), "s"(n_books), "s"(n_total), "s"(gated));
+                 "s"(rcp_rows_per_cb), "s"(n_books), "s"(n_total), "s"(gated), "s"(rotate_priority));
     const int tid = threadIdx.x;
     constexpr int J = RUNS * kRunCodes;  // codes (bytes) per row
 
@@ -493,11 +493,29 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         else if (G > 2 && left == 2) multiply_rows(g, cur, std::integral_constant<int, (G > 2 ? 2 : 1)>{});
         else if (G > 3) multiply_rows(g, cur, std::integral_constant<int, (G > 3 ? 3 : 1)>{});
     };
+    // rotate_priority: a SIMD issues for its oldest wave first.  With equal shares the four waves of a SIMD therefore
+    // finish one after the other, and the youngest works through its last rows alone, with a single wave's loads in
+    // flight and nobody to cover its waits (time stamps inside the kernel, K = 8192, N = 28672, seven rows per wave: the
+    // four ages are done 5.7, 6.3, 7.4 and 8.9 us after they start; K = 4096: 3.6, 4.0, 4.7, 5.6).  The wave's issue
+    // priority (s_setprio, 0 to 3) therefore steps down by one with every group and wraps around, starting from its age
+    // class wave / 4: the four waves of a SIMD take turns at being served first (the same launches: 6.9, 8.0, 7.9, 7.6 us
+    // and 4.5, 4.9, 4.7, 4.4 us; the last wave ends 0.9 resp. 1.1 us earlier).  A hint to the arbiter: no result
+    // depends on it.
+    const int age = wave >> 2;
+    auto set_priority = [&](int v) {
+        switch (v & 3) {
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
+        }
+    };
     for (int g = 0; g < n_groups; g += NBUF) {
 #pragma unroll
         for (int u = 0; u < NBUF; u++) {
             // (unconditional: see the header; the group requested past the end is the last one again)
             load_group(min(g + u + NBUF - 1, n_groups - 1), cw[(u + NBUF - 1) % NBUF]);
+            if (rotate_priority) set_priority(age - (g + u));
             if (g + u < n_groups) multiply_group(g + u, cw[u]);
         }
     }
@@ -555,9 +573,13 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
     const bool straddle = p.n_codebooks > 1 && (p.gated || !(p.N % waves == 0 && p.rows_per_cb % (kWideWaves * (p.N / waves)) == 0));
     const int books = p.n_codebooks == 1 ? 0 : (straddle ? 2 : 1);
     const int n_dealt = p.gated ? p.N / 2 : p.N;  // what is dealt out to the waves: rows of W, or outputs
+    // the waves of a SIMD take turns at the issue priority (see the kernel) once they have two rows or more each: a
+    // single row per wave is over before a turn would come
+    const int rotate_priority = tuning().gemv_wide_rotate_priority >= 1.0 && (n_dealt + waves - 1) / waves >= 2 ? 1 : 0;
     auto launch = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.entries, n_dealt / waves, n_dealt % waves,
-                           p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, n_dealt, p.gated ? 1 : 0);
+                           p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, n_dealt, p.gated ? 1 : 0,
+                           rotate_priority);
         return hipGetLastError();
     };
     // The plain table while a wave gathers for at most Tuning::gemv_wide_plain_table_max_runs runs of 2048 k (8 gathers per

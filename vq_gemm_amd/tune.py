@@ -307,6 +307,21 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
     loop_now = {k: out[k] for k in ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight", "gemv_wide_rows_per_group_long_k",
                                     "gemv_wide_groups_in_flight_long_k")}
 
+    # 1b. the waves of a SIMD taking turns at the issue priority
+    rot_shapes = [(4096, 7 * waves), (8192, 7 * waves)] + ([] if quick else [(4096, 16 * waves), (2048, 8 * waves), (4096, 3 * waves)])
+    rot = {r: [_cold_us(1, K, N, GEMV, device=device, **force_wide, **loop_now, gemv_wide_rotate_priority=r) for (K, N) in rot_shapes] for r in (0, 1)}
+    if all(t is not None for ts in rot.values() for t in ts):
+        score = {r: sum(t / min(a, b) for t, a, b in zip(ts, rot[0], rot[1])) for r, ts in rot.items()}
+        now = int(cur["gemv_wide_rotate_priority"] >= 1.0)
+        win = min(score, key=score.get)
+        if score[now] <= score[win] * (1.0 + margin):
+            win = now
+        out["gemv_wide_rotate_priority"] = float(win)
+        report["rotate_priority"] = {r: [round(t, 3) for t in ts] for r, ts in rot.items()}
+        say("wide GEMV, issue priority: " + "; ".join(("rotating: " if r else "left alone: ") + "/".join(f"{t:.2f}" for t in ts) for r, ts in rot.items())
+            + f" us on {rot_shapes} -> {win}")
+    loop_now["gemv_wide_rotate_priority"] = out["gemv_wide_rotate_priority"]
+
     # 2. plain against bank-replicated table: the threshold in gathers per lane (rows per wave x runs of 2048 k)
     rows = []
     for (K, N) in [(2048, waves), (4096, waves), (4096, 2 * waves), (8192, waves)] + ([] if quick else [(2048, 2 * waves), (8192, 2 * waves)]):
