@@ -73,6 +73,7 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_wide_rows_per_group_long_k", &Tuning::gemv_wide_rows_per_group_long_k},
     {"gemv_wide_groups_in_flight_long_k", &Tuning::gemv_wide_groups_in_flight_long_k},
     {"gemv_wide_rotate_priority", &Tuning::gemv_wide_rotate_priority},
+    {"gemv_wide_min_units_share", &Tuning::gemv_wide_min_units_share},
     {"decode_replicated_table_min_tiles", &Tuning::decode_replicated_table_min_tiles},
     {"splitk_fixed_us", &Tuning::splitk_fixed_us},
     {"splitk_us_per_partial_mb", &Tuning::splitk_us_per_partial_mb},

@@ -191,6 +191,9 @@ struct Tuning {
     double gemv_wide_groups_in_flight = 2.0;
     double gemv_wide_rows_per_group_long_k = 1.0;
     double gemv_wide_groups_in_flight_long_k = 2.0;
+    // the wide form leaves up to this share of the compute units without a workgroup where that keeps every workgroup's
+    // rows inside one codebook
+    double gemv_wide_min_units_share = 0.7;
     // the wide form's waves step their issue priority round with every group (1) or leave it alone (0)
     double gemv_wide_rotate_priority = 1.0;
     // batched decode kernel: the bank-replicated table (64 KB to fill) from this many tiles per workgroup on

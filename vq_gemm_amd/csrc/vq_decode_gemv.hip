@@ -565,7 +565,21 @@ bool decode_gemv_wide_supports(const ProblemB &p)
 hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
 {
     if (!decode_gemv_wide_supports(p)) return hipErrorInvalidValue;
-    const int cus = device_cu_count();
+    // One workgroup per compute unit - or, with several codebooks, a few less where that makes every workgroup's rows
+    // fall inside one codebook: a workgroup whose rows cross a boundary fills two tables, and the launch ends with the
+    // slowest workgroup (the q, k and v projections of a layer as three codebooks of 4096 rows: 192 workgroups of 64 rows
+    // take 4.9 us cold where 256 workgroups of 48 rows take 5.25).  Not below Tuning::gemv_wide_min_units_share of the units.
+    int cus = device_cu_count();
+    if (p.n_codebooks > 1 && !p.gated) {
+        const int least = (int)(tuning().gemv_wide_min_units_share * cus);
+        for (int w = cus; w >= least && w >= 1; w--) {
+            const int per_wg = p.N / w;
+            if (p.N % w == 0 && per_wg % kWideWaves == 0 && per_wg / kWideWaves <= 64 && p.rows_per_cb % per_wg == 0) {
+                cus = w;
+                break;
+            }
+        }
+    }
     const int waves = cus * kWideWaves;
     const dim3 grid(cus), block(kWideWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);

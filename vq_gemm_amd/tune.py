@@ -322,6 +322,26 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
             + f" us on {rot_shapes} -> {win}")
     loop_now["gemv_wide_rotate_priority"] = out["gemv_wide_rotate_priority"]
 
+    # 1c. several codebooks: how many compute units may go without a workgroup so that no workgroup's rows cross a codebook
+    book_shapes = [(4096, 48 * cus, 3), (4096, 112 * cus, 56)] + ([] if quick else [(8192, 112 * cus, 56), (4096, 24 * cus, 3)])
+    shares = {}
+    for share in (1.0, 0.85, 0.7, 0.5):
+        ts = [_cold_us(1, K, N, GEMV, n_codebooks=G, device=device, **force_wide, **loop_now, gemv_wide_min_units_share=share)
+              for (K, N, G) in book_shapes]
+        if all(t is not None for t in ts):
+            shares[share] = ts
+    if shares:
+        best_of = [min(ts[i] for ts in shares.values()) for i in range(len(book_shapes))]
+        score = {c: sum(t / b for t, b in zip(ts, best_of)) for c, ts in shares.items()}
+        win = min(score, key=score.get)
+        now = cur["gemv_wide_min_units_share"]
+        if now in score and score[now] <= score[win] * (1.0 + margin):
+            win = now
+        out["gemv_wide_min_units_share"] = float(win)
+        report["min_units_share"] = {c: [round(t, 3) for t in ts] for c, ts in shares.items()}
+        say("wide GEMV, units left idle for whole codebooks: " + "; ".join(f"share {c}: " + "/".join(f"{t:.2f}" for t in ts) for c, ts in shares.items())
+            + f" us on {book_shapes} -> {win}")
+
     # 2. plain against bank-replicated table: the threshold in gathers per lane (rows per wave x runs of 2048 k)
     rows = []
     for (K, N) in [(2048, waves), (4096, waves), (4096, 2 * waves), (8192, waves)] + ([] if quick else [(2048, 2 * waves), (8192, 2 * waves)]):
