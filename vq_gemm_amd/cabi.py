@@ -121,7 +121,12 @@ def tuning() -> dict:
     return out
 
 
+tuning_generation = 0  # steps with every change of the table: what callers key cached kernel choices by
+
+
 def set_tuning(**constants) -> None:
+    global tuning_generation
+    tuning_generation += 1
     for name, value in constants.items():
         rc = lib().vqgemm_tuning_set(name.encode(), float(value))
         if rc != 0:

@@ -17,6 +17,29 @@ import torch
 from . import cabi
 
 
+# What the automatic choice wants as scratch for a shape (bytes; 0 for all but the split-K shapes), remembered per shape and
+# state of the tuning table, and one scratch buffer per device and stream, grown on demand: a layer's forward makes neither
+# a host-side cost-model pass nor an allocation per call.  (Launches on one stream run in order, so they can share the buffer.)
+_ws_need: dict = {}
+_ws_pool: dict = {}
+
+
+def _workspace_for(M, K, N, v, E, G, bits, device):
+    key = (M, K, N, v, E, G, bits, cabi.tuning_generation)
+    need = _ws_need.get(key)
+    if need is None:
+        if len(_ws_need) > 4096:
+            _ws_need.clear()
+        need = _ws_need[key] = cabi.workspace_bytes_b(M, K, N, v, E, G, bits, cabi.VARIANT_AUTO)
+    if need <= 0:
+        return None
+    slot = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _ws_pool.get(slot)
+    if ws is None or ws.numel() < need:
+        ws = _ws_pool[slot] = torch.empty(need, dtype=torch.uint8, device=device)
+    return ws
+
+
 def _out_shape(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor):
     if codes.dim() != 2 or codebook.dim() not in (2, 3) or x.dim() < 1:
         raise ValueError("vq_linear: x [..., K], codes [N, K/vec], codebook [E, vec] or [G, E, vec]")
@@ -34,9 +57,15 @@ def vq_linear(x: torch.Tensor, codes: torch.Tensor, codebook: torch.Tensor,
     if x.dtype != torch.float16 or codebook.dtype != torch.float16:
         raise ValueError("vq_linear: x and codebook must be float16")
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
-    # (the entry point with a sized workspace: allocated only for the shapes whose automatic choice wants one - split K)
-    y = cabi.e2e_gemm_b_ws(x2, codes.contiguous(), codebook.contiguous(), bias=None if bias is None else bias.contiguous())
-    return y.view(shape)
+    codes, codebook = codes.contiguous(), codebook.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    g, e, v = cabi._cb_dims(codebook)
+    ws = _workspace_for(x2.shape[0], x2.shape[1], codes.shape[0], v, e, g, 8 * codes.element_size(), x2.device)
+    if ws is None:
+        # (no kernel the automatic choice would take wants scratch for this shape: the plain entry point)
+        return cabi.e2e_gemm_b(x2, codes, codebook, bias=bias).view(shape)
+    # the entry point with a sized workspace: the automatic choice may split K
+    return cabi.e2e_gemm_b_ws(x2, codes, codebook, bias=bias, workspace=ws).view(shape)
 
 
 @vq_linear.register_fake
