@@ -482,8 +482,11 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
+            // (the row's sum goes from the scalar register straight into lane g*G + r: one v_writelane instead of a
+            // move, a compare and a select)
             const float s = wave_sum_to_uniform(acc[r]);
-            res = (int)lane == g * G + r ? s : res;
+            // (on this target the instruction takes one scalar register: the lane number goes through m0)
+            asm("s_mov_b32 m0, %2\n\tv_writelane_b32 %0, %1, m0" : "+v"(res) : "s"(s), "s"(g * G + r) : "m0");
         }
     };
     auto multiply_group = [&](int g, const uint32_t (&cur)[G][RUNS]) {
