@@ -192,6 +192,30 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
     assert np.array_equal(_np(ywp).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
 
 
+@pytest.mark.parametrize("M,K,N,v,E,bits,G", [(16, 4096, 11008, 4, 4096, 16, 1), (16, 4096, 4096, 8, 256, 8, 1),
+                                              (5, 8192, 2048, 8, 256, 8, 4), (40, 2048, 1536, 4, 256, 8, 2)])
+def test_batched_decode_kernel_gives_the_same_bits_on_every_launch(M, K, N, v, E, bits, G):
+    # The batched kernel keeps codes and gathered codewords in registers that the hardware is still writing while the
+    # wave runs on, and waits for them by count: a count that does not match the order of issue, or a register the
+    # compiler moved in that window, shows as a rare wrong element, not as a steady error.  C3 itself, one tile per
+    # workgroup, chunked K with several codebooks, and two slabs of X: 40 launches each on fixed operands, back to back
+    # and one at a time, every result equal to the first bit for bit; the first against the oracle.
+    spec = ProblemSpec("steady", GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
+    x, codes, cb = make_problem(spec, seed=91, device=DEV)
+    _say("batched decode, 40 launches", M, K, N, v, E, bits, G)
+    first = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE).clone()
+    torch.cuda.synchronize()
+    _check_gemm(first, x, codes, cb, what="first launch")
+    outs = [cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE) for _ in range(20)]
+    torch.cuda.synchronize()
+    for i, y in enumerate(outs):
+        assert torch.equal(y, first), f"launch {i} differs"
+    for i in range(20):
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
+        torch.cuda.synchronize()
+        assert torch.equal(y, first), f"synchronised launch {i} differs"
+
+
 def test_packed_codes_small_shapes_bias_and_rejections():
     for (M, K, N, v, E, G, bits) in [(1, 256, 16, 8, 256, 1, 8), (5, 512, 48, 4, 4096, 1, 16), (16, 256, 32, 2, 256, 2, 8),
                                      (33, 1024, 64, 8, 300, 4, 16), (3, 768, 32, 2, 1000, 1, 16), (16, 4096, 4096, 8, 256, 1, 8)]:
