@@ -40,6 +40,12 @@ HOST_ONLY_SOURCES = {"vq_api.hip", "vq_noalloc.hip"}
 HIP_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 
+# The decode kernels are short launches, and a wave's first instruction there is a fetch of its kernel arguments from a
+# cold scalar cache: gfx950 can hand the first arguments to a wave in scalar registers at launch (at most 14 dwords beside
+# the two of the argument pointer).  The kernels of these sources take their arguments in the order they need them.
+KERNARG_PRELOAD_SOURCES = {"vq_decode_gemv.hip"}
+KERNARG_PRELOAD_FLAGS = ["-mllvm", "-amdgpu-kernarg-preload-count=14"]
+
 # variant key -> (VQGEMM_VARIANT_* value, is the hipBLASLt baseline module)
 # The keys are the reference's strategy names: s1 is its two-pass strategy
 # (strategy_1/src.cu:323-399); s2_*/s3_* are its fused strategies, all served here by the
@@ -124,7 +130,8 @@ def build_lib(force: bool = True, jobs: int = 6) -> str:
         s = os.path.join(CSRC, src)
         o = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
         if force or not _newer(o, [s] + hdrs):
-            _run([HIPCC] + HIP_FLAGS + ["--save-temps=obj", "-c", s, "-o", o])
+            extra = KERNARG_PRELOAD_FLAGS if src in KERNARG_PRELOAD_SOURCES else []
+            _run([HIPCC] + HIP_FLAGS + extra + ["--save-temps=obj", "-c", s, "-o", o])
             if src not in HOST_ONLY_SOURCES:
                 _check_no_spills(o.replace(".o", f"-hip-amdgcn-amd-amdhsa-{ARCH}.s"))
         return o

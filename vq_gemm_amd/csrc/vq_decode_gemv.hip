@@ -285,13 +285,17 @@ __device__ __forceinline__ int small_quotient(int x, int d, float rcp)
 template <int RUNS, int G, int NBUF, int BOOKS, int COPIES>
 __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const half_t *__restrict__ x,
                                                                            const uint8_t *__restrict__ codes,
-                                                                           const half_t *__restrict__ cb,
-                                                                           half_t *__restrict__ y,
-                                                                           const half_t *__restrict__ bias, int entries,
-                                                                           int rows_q, int rows_r, int rows_per_cb,
-                                                                           float rcp_rows_per_cb, int n_books, int n_total,
-                                                                           int gated, int rotate_priority)
+                                                                           const half_t *__restrict__ cb, int entries,
+                                                                           int rows_q, int rows_r, int n_total, int gated,
+                                                                           const half_t *__restrict__ bias,
+                                                                           int rows_per_cb, float rcp_rows_per_cb,
+                                                                           int n_books, half_t *__restrict__ y,
+                                                                           int rotate_priority)
 {
+    // (The order of the arguments is the order in which the kernel needs them: the build preloads the first fourteen
+    // dwords of a kernel's arguments into scalar registers at wave launch, -amdgpu-kernarg-preload-count, and what the
+    // first loads need - x, the codes, the codebook and the numbers the wave's rows follow from - lies inside them, so
+    // that no wave waits for an argument fetch ahead of its first load.)
     // gated: the epilogue of a gate/up pair.  The rows of W are gate and up rows interleaved in groups of 16; what
     // is dealt out to the waves (rows_q, rows_r, n_total) are then the N/2 outputs, a wave's code rows are the gate
     // and the up row of each of its outputs in turn; a group of two rows is one output (G = 2), or the gate row and the
@@ -304,10 +308,6 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     constexpr int kTableSlots = (TWO ? 2 : 1) * 256 * COPIES;
     __shared__ __align__(16) uint4_t lds[kTableSlots + kXChunks];
     uint4_t *table = lds, *xs = lds + kTableSlots;
-    // All kernel arguments are fetched at once: left to first use, each pointer costs the prologue a
-    // scalar-load round trip of its own.
-    asm volatile("" ::"s"(x), "s"(codes), "s"(cb), "s"(y), "s"(bias), "s"(entries), "s"(rows_q), "s"(rows_r), "s"(rows_per_cb),
-                 "s"(rcp_rows_per_cb), "s"(n_books), "s"(n_total), "s"(gated), "s"(rotate_priority));
     const int tid = threadIdx.x;
     constexpr int J = RUNS * kRunCodes;  // codes (bytes) per row
 
@@ -594,8 +594,8 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
     // single row per wave is over before a turn would come
     const int rotate_priority = tuning().gemv_wide_rotate_priority >= 1.0 && (n_dealt + waves - 1) / waves >= 2 ? 1 : 0;
     auto launch = [&](auto kern) {
-        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.y, p.bias, p.entries, n_dealt / waves, n_dealt % waves,
-                           p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, n_dealt, p.gated ? 1 : 0,
+        hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.entries, n_dealt / waves, n_dealt % waves, n_dealt,
+                           p.gated ? 1 : 0, p.bias, p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, p.y,
                            rotate_priority);
         return hipGetLastError();
     };
