@@ -415,6 +415,13 @@ def main():
         others["decode_qkv_m1_k4096_n12288"], _ = bench_config(
             ProblemSpec("decode_qkv_m1_k4096_n12288", GEOM_B, 1, 4096, 12288, 8, 256, 3, 8),
             max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        # the down-projection behind such an MLP (K beyond what a lane's registers hold of x: rows worked through in pieces)
+        others["decode_down_m1_k14336_n4096"], _ = bench_config(
+            ProblemSpec("decode_down_m1_k14336_n4096", GEOM_B, 1, 14336, 4096, 8, 256, 1, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        others["decode_down_m1_k28672_n8192"], _ = bench_config(
+            ProblemSpec("decode_down_m1_k28672_n8192", GEOM_B, 1, 28672, 8192, 8, 256, 1, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         others["C1"], _ = bench_config("C1", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=False)
         others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
         others["C5"], _ = bench_config("C5", 10, 3, cold_pool=False)

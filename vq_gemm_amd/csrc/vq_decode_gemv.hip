@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     }
 }
 
-// ---- the wide form: long runs of rows, and every single-row launch of at least half a row per wave -------
+// ---- the wide form: long runs of rows, long rows, and every single-row launch of at least half a row per wave -------
 // One workgroup of sixteen waves per compute unit over a bank-replicated table (64 KB: 16 copies of
 // each entry in one 256-byte bank row, lane l reading copy l % 16, so the gathers never collide):
 // four waves per SIMD cover the latency of each other's gathers.  One row of X, 8-vectors, 8-bit codes.
@@ -282,15 +282,23 @@ __device__ __forceinline__ int small_quotient(int x, int d, float rcp)
 //
 // COPIES: 16 = the bank-replicated table (conflict-free gathers; 64 KB to fill), 1 = the plain 4 KB table (a wave
 // with one or two rows gathers too little for the fill of the replicated table to pay).
-template <int RUNS, int G, int NBUF, int BOOKS, int COPIES>
+//
+// XRUNS: runs of 2048 k of x that the LDS holds.  XRUNS == RUNS is the form described so far (K = RUNS * 2048, all of a
+// lane's x in registers).  XRUNS > RUNS is the form for a longer K, or one that is no multiple of 2048 (the
+// down-projection of an MLP: K = 11008, 14336, 28672): a row is cut into pieces of RUNS runs, a wave goes through
+// its rows once per piece with that piece's x in its registers (read from the LDS again at every change of piece),
+// and a row's sum so far travels in its lane of `res`: the accumulator of lane 0 starts from it.  x is padded with
+// zeros up to whole pieces, and a load that would reach past the end of a row reads the row's last dword instead: what
+// it gathers meets zeros.  One codebook, or several without a workgroup whose rows reach into two; not gated.
+template <int RUNS, int G, int NBUF, int BOOKS, int COPIES, int XRUNS = RUNS>
 __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const half_t *__restrict__ x,
                                                                            const uint8_t *__restrict__ codes,
                                                                            const half_t *__restrict__ cb, int entries,
-                                                                           int rows_q, int rows_r, int n_total, int gated,
+                                                                           int rows_q, int rows_r, int n_total,
+                                                                           int gated_row_bytes, int rows_per_cb,
+                                                                           float rcp_rows_per_cb, int n_books,
                                                                            const half_t *__restrict__ bias,
-                                                                           int rows_per_cb, float rcp_rows_per_cb,
-                                                                           int n_books, half_t *__restrict__ y,
-                                                                           int rotate_priority)
+                                                                           half_t *__restrict__ y, int rotate_priority)
 {
     // (The order of the arguments is the order in which the kernel needs them: the build preloads the first fourteen
     // dwords of a kernel's arguments into scalar registers at wave launch, -amdgpu-kernarg-preload-count, and what the
@@ -300,8 +308,13 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     // is dealt out to the waves (rows_q, rows_r, n_total) are then the N/2 outputs, a wave's code rows are the gate
     // and the up row of each of its outputs in turn; a group of two rows is one output (G = 2), or the gate row and the
     // up row are two groups in turn (G = 1).
+    // gated_row_bytes: bit 31 = gated, below it the bytes of a row of codes (K / 8; read by the long form only) - one
+    // argument, so that everything the prologue needs stays inside the preloaded fourteen dwords.
     constexpr bool TWO = BOOKS == 2;
-    constexpr int kXChunks = RUNS * kRunCodes;  // 16-byte pieces of x
+    constexpr bool LONG = XRUNS != RUNS;
+    static_assert(!LONG || (BOOKS < 2 && COPIES == kWideCopies && NBUF == 2), "the long form: one table, replicated");
+    const int gated = LONG ? 0 : (gated_row_bytes < 0 ? 1 : 0);
+    constexpr int kXChunks = XRUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
     // permute) | table of the second one (TWO) | x
     static_assert(COPIES == kWideCopies || COPIES == 1, "replicated or plain table");
@@ -309,7 +322,10 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     __shared__ __align__(16) uint4_t lds[kTableSlots + kXChunks];
     uint4_t *table = lds, *xs = lds + kTableSlots;
     const int tid = threadIdx.x;
-    constexpr int J = RUNS * kRunCodes;  // codes (bytes) per row
+    // codes (bytes) per row, and the pieces a row is worked through in
+    const int J = LONG ? (gated_row_bytes & 0xffffff) : RUNS * kRunCodes;
+    constexpr int kPieceBytes = RUNS * kRunCodes;
+    const int n_pieces = LONG ? (J + kPieceBytes - 1) / kPieceBytes : 1;
 
     // The prologue's duties are split between the waves so that each has little queued ahead of its code loads:
     // waves 0-7 fetch the table (two threads per entry), waves 8-15 fetch x (one or two pieces per thread).
@@ -344,7 +360,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         if (second_table) entry1 = reinterpret_cast<const uint4_t *>(cb + (int64_t)min(book0 + 1, n_books - 1) * entries * 8)[ec];
     } else {
 #pragma unroll
-        for (int i = 0; i < kXPerThread; i++) xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, kXChunks - 1)];
+        for (int i = 0; i < kXPerThread; i++)
+            xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, (LONG ? J : kXChunks) - 1)];
     }
 
     // the wave's share [row0, row0 + n_share) of the rows (gated: of the outputs) and its code rows: at most 64, one
@@ -371,20 +388,41 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     }
 
     uint32_t cw[NBUF][G][RUNS];
-    auto load_group = [&](int g, uint32_t (&dst)[G][RUNS]) {
+    // group g of the wave's rows, piece `piece` of them (0 outside the long form)
+    auto load_group = [&](int piece, int g, uint32_t (&dst)[G][RUNS]) {
 #pragma unroll
         for (int r = 0; r < G; r++) {
             // (a wave-uniform row pointer and the lane as a 32-bit index: one scalar base per row, no vector address arithmetic)
-            const uint32_t *row = reinterpret_cast<const uint32_t *>(codes + (int64_t)code_row(g * G + r) * J);
+            if constexpr (LONG) {
+                const uint8_t *row = codes + (int64_t)code_row(g * G + r) * J + piece * kPieceBytes;
+                const uint32_t last = (uint32_t)(J - 4 - piece * kPieceBytes);  // the row's last dword, from the piece on
 #pragma unroll
-            for (int q = 0; q < RUNS; q++)
-                // (a relaxed atomic load of wavefront scope is an ordinary load instruction that the compiler
-                // leaves where it is written: ahead of the table's stores and the barrier)
-                dst[r][q] = __hip_atomic_load(row + q * (kRunCodes / 4) + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                for (int q = 0; q < RUNS; q++)
+                    dst[r][q] = __hip_atomic_load(reinterpret_cast<const uint32_t *>(row + min(q * kRunCodes + 4u * lane, last)),
+                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            } else {
+                const uint32_t *row = reinterpret_cast<const uint32_t *>(codes + (int64_t)code_row(g * G + r) * J);
+#pragma unroll
+                for (int q = 0; q < RUNS; q++)
+                    // (a relaxed atomic load of wavefront scope is an ordinary load instruction that the compiler
+                    // leaves where it is written: ahead of the table's stores and the barrier)
+                    dst[r][q] = __hip_atomic_load(row + q * (kRunCodes / 4) + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            }
         }
     };
+    // the long form walks (piece, group) pairs, all groups of a piece before the next piece; the request runs
+    // NBUF - 1 pairs ahead of the multiply and asks for the last pair again once it is past the end
+    int req_piece = 0, req_group = 0;
+    auto request_next = [&](uint32_t (&dst)[G][RUNS]) {
+        const bool over = req_piece >= n_pieces || n_groups <= 0;
+        load_group(over ? n_pieces - 1 : req_piece, over ? max(n_groups, 1) - 1 : req_group, dst);
+        if (++req_group >= n_groups) req_group = 0, ++req_piece;
+    };
 #pragma unroll
-    for (int u = 0; u < NBUF - 1; u++) load_group(min(u, max(n_groups, 1) - 1), cw[u]);
+    for (int u = 0; u < NBUF - 1; u++) {
+        if constexpr (LONG) request_next(cw[u]);
+        else load_group(0, min(u, max(n_groups, 1) - 1), cw[u]);
+    }
 
     if (table_duty) {
         // Table: thread (e, h) writes copies 8h .. 8h+7 of entry e, in an order that sends the sixteen lanes
@@ -409,16 +447,21 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
         for (int i = 0; i < kXPerThread; i++) {
             const int xi = xt + i * kDutyThreads;
+            // (the long form: zeros behind the end of x, up to whole pieces of rows)
+            if (LONG && xi >= J) xpiece[i] = uint4_t{0u, 0u, 0u, 0u};
             if (xi < kXChunks) xs[(xi & ~255) + (xi & 3) * 64 + ((xi >> 2) & 63)] = xpiece[i];
         }
     }
     __syncthreads();
     if (n_rows <= 0) return;
     uint4_t xr[RUNS][4];
+    auto load_x_piece = [&](int piece) {
 #pragma unroll
-    for (int q = 0; q < RUNS; q++)
+        for (int q = 0; q < RUNS; q++)
 #pragma unroll
-        for (int c = 0; c < 4; c++) xr[q][c] = xs[q * kRunCodes + c * 64 + lane];
+            for (int c = 0; c < 4; c++) xr[q][c] = xs[(piece * RUNS + q) * kRunCodes + c * 64 + lane];
+    };
+    load_x_piece(0);
 
     // Gather address = table * 65536 + code * 256 + copy * 16, put together by one byte permute out of the
     // lane's dword of codes (byte 1) and a per-row base (bytes 0 and 2).
@@ -434,6 +477,9 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
         for (int r = 0; r < R; r++) {
             acc[r] = 0.f;
+            // (the long form: the row's sum over the pieces before this one, zero at the first)
+            if constexpr (LONG)
+                acc[r] = lane == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, res), g * G + r)) : 0.f;
             if constexpr (COPIES == 1) base[r] = TWO && code_row(g * G + r) >= second_book_row ? 4096u : 0u;
             else base[r] = TWO ? copy_base | (code_row(g * G + r) >= second_book_row ? 0x10000u : 0u) : copy_base;
         }
@@ -513,13 +559,29 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         default: __builtin_amdgcn_s_setprio(3); break;
         }
     };
-    for (int g = 0; g < n_groups; g += NBUF) {
+    if constexpr (LONG) {
+        int piece = 0, g = 0, turn = 0;
+        while (piece < n_pieces) {
 #pragma unroll
-        for (int u = 0; u < NBUF; u++) {
-            // (unconditional: see the header; the group requested past the end is the last one again)
-            load_group(min(g + u + NBUF - 1, n_groups - 1), cw[(u + NBUF - 1) % NBUF]);
-            if (rotate_priority) set_priority(age - (g + u));
-            if (g + u < n_groups) multiply_group(g + u, cw[u]);
+            for (int u = 0; u < NBUF; u++) {
+                request_next(cw[(u + NBUF - 1) % NBUF]);
+                if (rotate_priority) set_priority(age - turn++);
+                if (piece < n_pieces) {
+                    if (g == 0 && piece > 0) load_x_piece(piece);
+                    multiply_group(g, cw[u]);
+                    if (++g >= n_groups) g = 0, ++piece;
+                }
+            }
+        }
+    } else {
+        for (int g = 0; g < n_groups; g += NBUF) {
+#pragma unroll
+            for (int u = 0; u < NBUF; u++) {
+                // (unconditional: see the header; the group requested past the end is the last one again)
+                load_group(0, min(g + u + NBUF - 1, n_groups - 1), cw[(u + NBUF - 1) % NBUF]);
+                if (rotate_priority) set_priority(age - (g + u));
+                if (g + u < n_groups) multiply_group(g + u, cw[u]);
+            }
         }
     }
     if ((int)lane < n_share) {
@@ -545,12 +607,61 @@ static int wide_groups_in_flight(const ProblemB &p)
     return (p.K / kRunK > 2 ? tn.gemv_wide_groups_in_flight_long_k : tn.gemv_wide_groups_in_flight) >= 3.0 ? 3 : 2;
 }
 
-// One row of X, 8-vectors, 8-bit codes, K a multiple of 2048 up to 8192, and no workgroup's share of
-// the rows reaching into more than two codebooks.
+// The long form's cut of a row (see the kernel): K beyond 8192 or no multiple of 2048, up to 32768, whole dwords of
+// codes per row.  runs = runs of 2048 k per piece (3 or 4, whichever pads the row less), x_runs = what the LDS holds.
+struct LongK {
+    bool is_long;
+    int runs, x_runs;
+};
+static LongK long_k_form(const ProblemB &p)
+{
+    LongK f{false, 0, 0};
+    if (p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns) return f;
+    f.is_long = true;
+    const int runs_needed = (int)((p.K + kRunK - 1) / kRunK);
+    const int padded4 = (runs_needed + 3) / 4 * 4, padded3 = (runs_needed + 2) / 3 * 3;
+    f.runs = padded3 < padded4 ? 3 : 4;
+    f.x_runs = min(padded3, padded4) <= 8 ? 8 : 16;
+    return f;
+}
+
+// The workgroups of a launch: one per compute unit - or, with several codebooks, a few less where that makes every
+// workgroup's rows fall inside one codebook: a workgroup whose rows cross a boundary fills two tables, and the launch
+// ends with the slowest workgroup (the q, k and v projections of a layer as three codebooks of 4096 rows: 192
+// workgroups of 64 rows take 4.9 us cold where 256 workgroups of 48 rows take 5.25).  Not below
+// Tuning::gemv_wide_min_units_share of the units.
+static int wide_workgroups(const ProblemB &p)
+{
+    const int cus = device_cu_count();
+    if (p.n_codebooks > 1 && !p.gated) {
+        const int least = (int)(tuning().gemv_wide_min_units_share * cus);
+        for (int w = cus; w >= least && w >= 1; w--) {
+            const int per_wg = p.N / w;
+            if (p.N % w == 0 && per_wg % kWideWaves == 0 && per_wg / kWideWaves <= 64 && p.rows_per_cb % per_wg == 0) return w;
+        }
+    }
+    return cus;
+}
+// whether some workgroup's rows cross a codebook boundary (then every workgroup has room for two tables)
+static bool wide_straddles(const ProblemB &p, int workgroups)
+{
+    const int waves = workgroups * kWideWaves;
+    return p.n_codebooks > 1 && (p.gated || !(p.N % waves == 0 && p.rows_per_cb % (kWideWaves * (p.N / waves)) == 0));
+}
+
+// One row of X, 8-vectors, 8-bit codes, K a multiple of 2048 up to 8192 - or, not gated and with no workgroup reaching
+// into two codebooks, any multiple of 32 from 2048 up to 32768 - and no workgroup's share of the rows reaching into
+// more than two codebooks.
 bool decode_gemv_wide_supports(const ProblemB &p)
 {
     if (p.M != 1 || p.vec != 8 || p.code_bits != 8 || p.entries > 256 || p.packed) return false;
-    if (p.K < kRunK || p.K % kRunK != 0 || p.K / kRunK > kGemvMaxRuns || p.N < 1) return false;
+    if (p.K < kRunK || p.N < 1) return false;
+    if (long_k_form(p).is_long) {
+        if (p.K % 32 != 0 || p.K > 16 * kRunK || p.gated) return false;
+        const int workgroups = wide_workgroups(p);
+        if (wide_straddles(p, workgroups)) return false;
+        return (p.N + workgroups * kWideWaves - 1) / (workgroups * kWideWaves) <= 64;
+    }
     const int waves = device_cu_count() * kWideWaves;
     if (p.gated) {
         // two code rows per output: one group of two rows, or two groups of one
@@ -568,37 +679,39 @@ bool decode_gemv_wide_supports(const ProblemB &p)
 hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
 {
     if (!decode_gemv_wide_supports(p)) return hipErrorInvalidValue;
-    // One workgroup per compute unit - or, with several codebooks, a few less where that makes every workgroup's rows
-    // fall inside one codebook: a workgroup whose rows cross a boundary fills two tables, and the launch ends with the
-    // slowest workgroup (the q, k and v projections of a layer as three codebooks of 4096 rows: 192 workgroups of 64 rows
-    // take 4.9 us cold where 256 workgroups of 48 rows take 5.25).  Not below Tuning::gemv_wide_min_units_share of the units.
-    int cus = device_cu_count();
-    if (p.n_codebooks > 1 && !p.gated) {
-        const int least = (int)(tuning().gemv_wide_min_units_share * cus);
-        for (int w = cus; w >= least && w >= 1; w--) {
-            const int per_wg = p.N / w;
-            if (p.N % w == 0 && per_wg % kWideWaves == 0 && per_wg / kWideWaves <= 64 && p.rows_per_cb % per_wg == 0) {
-                cus = w;
-                break;
-            }
-        }
-    }
+    const int cus = wide_workgroups(p);
     const int waves = cus * kWideWaves;
     const dim3 grid(cus), block(kWideWaves * 64);
     const uint8_t *codes = static_cast<const uint8_t *>(p.codes);
-    // a second table only when some workgroup's rows cross a codebook boundary: then every workgroup has room for two
-    const bool straddle = p.n_codebooks > 1 && (p.gated || !(p.N % waves == 0 && p.rows_per_cb % (kWideWaves * (p.N / waves)) == 0));
-    const int books = p.n_codebooks == 1 ? 0 : (straddle ? 2 : 1);
+    const int books = p.n_codebooks == 1 ? 0 : (wide_straddles(p, cus) ? 2 : 1);
     const int n_dealt = p.gated ? p.N / 2 : p.N;  // what is dealt out to the waves: rows of W, or outputs
     // the waves of a SIMD take turns at the issue priority (see the kernel) once they have two rows or more each: a
     // single row per wave is over before a turn would come
     const int rotate_priority = tuning().gemv_wide_rotate_priority >= 1.0 && (n_dealt + waves - 1) / waves >= 2 ? 1 : 0;
     auto launch = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, block, 0, s, p.x, codes, p.cb, p.entries, n_dealt / waves, n_dealt % waves, n_dealt,
-                           p.gated ? 1 : 0, p.bias, p.rows_per_cb, 1.0f / (float)p.rows_per_cb, p.n_codebooks, p.y,
-                           rotate_priority);
+                           (int)((p.gated ? 0x80000000u : 0u) | (uint32_t)(p.K / 8)), p.rows_per_cb,
+                           1.0f / (float)p.rows_per_cb, p.n_codebooks, p.bias, p.y, rotate_priority);
         return hipGetLastError();
     };
+    using std::integral_constant;
+    const int g = wide_rows_per_group(p);
+    if (const LongK f = long_k_form(p); f.is_long) {
+        // (the replicated table, one table per workgroup, two groups in flight: three were measured and are slower,
+        // K = 11008 to 28672, N = 4096 to 16384: +3 to +6 %, one shape -3 %)
+        auto pick_long = [&](auto runs_c, auto g_c, auto x_c) {
+            constexpr int R = decltype(runs_c)::value, GG = decltype(g_c)::value, XR = decltype(x_c)::value;
+            return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, 2, 0, kWideCopies, XR>)
+                              : launch(decode_gemv_wide_kernel<R, GG, 2, 1, kWideCopies, XR>);
+        };
+        auto pick_x = [&](auto runs_c, auto g_c) {
+            return f.x_runs == 8 ? pick_long(runs_c, g_c, integral_constant<int, 8>{}) : pick_long(runs_c, g_c, integral_constant<int, 16>{});
+        };
+        auto pick_g = [&](auto runs_c) {
+            return g == 2 ? pick_x(runs_c, integral_constant<int, 2>{}) : pick_x(runs_c, integral_constant<int, 1>{});
+        };
+        return f.runs == 3 ? pick_g(integral_constant<int, 3>{}) : pick_g(integral_constant<int, 4>{});
+    }
     // The plain table while a wave gathers for at most Tuning::gemv_wide_plain_table_max_runs runs of 2048 k (8 gathers per
     // lane and run): measured cold, plain -> replicated, K = 4096: one row per wave 3.29 -> 3.43 us, two rows
     // 4.07 -> 3.89; K = 2048, one row 2.93 -> 3.12; K = 8192, one row 4.26 -> 4.02.
@@ -612,7 +725,6 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
         return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, NB, 0, kWideCopies>)
              : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1, kWideCopies>) : launch(decode_gemv_wide_kernel<R, GG, NB, 2, kWideCopies>);
     };
-    using std::integral_constant;
     auto pick_runs = [&](auto g_c, auto nbuf_c) {
         switch (p.K / kRunK) {
         case 1: return pick(integral_constant<int, 1>{}, g_c, nbuf_c);
@@ -626,7 +738,6 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
         }
         return hipErrorInvalidValue;
     };
-    const int g = wide_rows_per_group(p);
     const int nbuf = (g == 2 && p.K / kRunK > 2) ? 2 : wide_groups_in_flight(p);
     if (g == 2) return nbuf == 3 ? pick_runs(integral_constant<int, 2>{}, integral_constant<int, 3>{})
                                  : pick_runs(integral_constant<int, 2>{}, integral_constant<int, 2>{});

@@ -303,7 +303,7 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
     loop_search("K<=4096", ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight"),
                 [(4096, waves, 1), (4096, 3 * waves, 3)] + ([] if quick else [(4096, 7 * waves, 1), (2048, 4 * waves, 1)]))
     loop_search("K>4096", ("gemv_wide_rows_per_group_long_k", "gemv_wide_groups_in_flight_long_k"),
-                [(8192, 2 * waves, 1)] + ([] if quick else [(8192, 7 * waves, 1), (6144, 4 * waves, 1)]))
+                [(8192, 2 * waves, 1)] + ([] if quick else [(8192, 7 * waves, 1), (6144, 4 * waves, 1), (14336, waves, 1)]))
     loop_now = {k: out[k] for k in ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight", "gemv_wide_rows_per_group_long_k",
                                     "gemv_wide_groups_in_flight_long_k")}
 
