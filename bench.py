@@ -50,6 +50,8 @@ PROFILED_TRAFFIC = {
     "decode_m1_k4096_n28672": (14_921_700, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
     "decode_m1_k8192_n28672": (29_657_000, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
     "decode_qkv_m1_k4096_n12288": (6_578_000, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
+    "decode_down_m1_k14336_n4096": (7_692_288, "profiles/decode_gemv_wide_kernel_long_k_down_projection.md"),
+    "decode_down_m1_k28672_n8192": (29_952_000, "profiles/decode_gemv_wide_kernel_long_k_down_projection.md"),
     "C4": (85_373_000, "profiles/prefill_kernel_c4_prefill_gemm.md"),
     "C5": (489_400_000, "profiles/prefill_kernel_c5_m2048_k8192_n28672.md"),
 }
