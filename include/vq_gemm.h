@@ -40,7 +40,9 @@ extern "C" {
 #define VQGEMM_VARIANT_GENERIC 1  /* simple scalar kernel, any shape */
 #define VQGEMM_VARIANT_DECODE 2   /* small and medium M, 16 rows of X per workgroup: K-sliced waves, 16x16x32 MFMA,
                                      LDS-resident codebook; M <= 4096 when K % 256 == 0, N % 16 == 0 and
-                                     (N / n_codebooks) % 16 == 0, M <= 64 otherwise */
+                                     (N / n_codebooks) % 16 == 0, M <= 64 otherwise.  Nine to sixteen rows of X on
+                                     K >= 12288 (8-vectors, 8-bit codes, few tiles per compute unit) go through the
+                                     streaming kernel of this path: K dealt to the waves in pieces, no chunks of K */
 #define VQGEMM_VARIANT_PREFILL 3  /* large M: 256x256 tiles of 16x16x32 MFMAs, codewords gathered into operands;
                                      256x128 tiles when those put more compute units to work */
 #define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */
@@ -50,7 +52,9 @@ extern "C" {
 #define VQGEMM_VARIANT_DECODE_PACKED 7   /* VQGEMM_VARIANT_DECODE on a code matrix that vqgemm_pack_codes_b has put
                                             in the order the kernel's lanes load it (never chosen by AUTO: the
                                             layout is a property of the caller's data); the K-sliced MFMA kernel
-                                            whatever the shape, same results as on the plain matrix bit for bit */
+                                            whatever the shape, same results bit for bit as that kernel on the plain
+                                            matrix (where VQGEMM_VARIANT_DECODE takes its streaming kernel instead, the
+                                            sums are added in another order) */
 #define VQGEMM_VARIANT_DECODE_GEMV 8     /* the GEMV kernels: whole rows of W per wave, no matrix core.  One row of X,
                                             8-vectors with 8-bit codes, at most 256 entries, K a multiple of 2048 up
                                             to 8192, at most 64 rows of W per wave of a 16-wave workgroup per compute

@@ -155,8 +155,17 @@ BATCHED_B = [
 ]
 
 
+@pytest.fixture
+def batched_kernel_for_long_k():
+    """The K-sliced path with its streaming kernel switched off: long K goes through the batched kernel's chunks."""
+    before = cabi.tuning()["decode_stream_min_k"]
+    cabi.set_tuning(decode_stream_min_k=1e8)
+    yield
+    cabi.set_tuning(decode_stream_min_k=before)
+
+
 @pytest.mark.parametrize("row", BATCHED_B, ids=[r[0] for r in BATCHED_B])
-def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
+def test_batched_decode_kernel_with_many_tiles_per_workgroup(row, batched_kernel_for_long_k):
     name, M, K, N, v, E, bits = row[:7]
     G = row[7] if len(row) > 7 else 1
     spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1))
@@ -190,6 +199,66 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row):
     assert torch.equal(yp, y)
     ywp = cabi.e2e_gemm_b(eye, packed, cb, variant=cabi.VARIANT_DECODE_PACKED)
     assert np.array_equal(_np(ywp).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+
+
+# The streaming kernel of the K-sliced path (whole K per workgroup, K dealt to the waves in pieces of 128): one and two
+# tiles per group, ragged last groups, fewer groups than compute units and several per workgroup, codebooks that change
+# between a workgroup's groups, tall X in slabs, K of fewer pieces than a workgroup has waves, short codebooks.
+STREAM_B = [
+    # name, M, K, N, E, G
+    ("down_projection_m16", 16, 14336, 4096, 256, 1),
+    ("down_projection_m4_k11008", 4, 11008, 4096, 256, 1),
+    ("three_groups_per_workgroup", 16, 8192, 24576, 256, 1),
+    ("three_tiles_ragged_last_group", 3, 4096, 11008, 256, 1),
+    ("two_tiles_16_codebooks_slabs", 40, 8192, 8192, 256, 16),
+    ("few_tiles_17_pieces", 1, 2176, 256, 256, 1),
+    ("one_piece", 7, 128, 64, 77, 1),
+    ("two_groups_per_workgroup_books_change", 9, 2048, 16 * 8 * 300, 200, 50),
+    ("m64_four_slabs", 64, 5120, 2048, 256, 2),
+    ("fourteen_pieces_per_wave", 5, 28672, 8192, 256, 1),
+]
+
+
+@pytest.mark.parametrize("row", STREAM_B, ids=[r[0] for r in STREAM_B])
+def test_streaming_decode_kernel(row):
+    name, M, K, N, E, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, 8, E, G, 8, codebook_3d=(G > 1))
+    x, codes, cb = make_problem(spec, seed=23, device=DEV)
+    _say("streaming decode", spec)
+    before = cabi.tuning()
+    try:
+        for gathers in (0.0, 1e8):   # the bank-replicated table, the plain table
+            cabi.set_tuning(decode_stream_min_k=0.0, decode_stream_min_m=0.0, decode_stream_max_m=1e8, decode_stream_max_groups_per_unit=1e8,
+                            decode_stream_replicated_min_gathers=gathers)
+            y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
+            torch.cuda.synchronize()
+            w = vo.dequant_b(_np(codes), _np(cb))
+            xf = _np(x).astype(np.float64)
+            ref = np.concatenate([xf @ w[r:r + 4096].astype(np.float64).T for r in range(0, N, 4096)], axis=1)
+            e1, e2 = vo.rel_err(_np(y), ref)
+            _say(f"  {name}: rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+            assert e1 <= TOL
+            # a permuted one-hot X reads W out bit for bit
+            eye = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+            cols = [(37 * m + 11) % K for m in range(M)]
+            for m, c in enumerate(cols):
+                eye[m, c] = 1.0
+            yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_DECODE)
+            assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+            for _ in range(5):
+                assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE), y)
+            bias = torch.randn(N, device=DEV).half()
+            yb = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE, bias=bias)
+            eb, _ = vo.rel_err(_np(yb), ref + _np(bias).astype(np.float64))
+            assert eb <= TOL
+        # the batched kernel on the same inputs: the same product within the bar
+        cabi.set_tuning(decode_stream_min_k=1e8)
+        if K % 256 == 0:
+            yd = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
+            scale = yd.float().abs().max().item()
+            assert ((y.float() - yd.float()).abs().max() / scale).item() <= TOL
+    finally:
+        cabi.set_tuning(**before)
 
 
 @pytest.mark.parametrize("M,K,N,v,E,bits,G", [(16, 4096, 11008, 4, 4096, 16, 1), (16, 4096, 4096, 8, 256, 8, 1),

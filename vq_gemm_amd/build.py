@@ -30,7 +30,7 @@ ARCH = "gfx950"
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-KERNEL_SOURCES = ["vq_api.hip", "vq_dequant.hip", "vq_encode.hip", "vq_generic.hip", "vq_decode.hip", "vq_decode_gemv.hip", "vq_decode_general.hip", "vq_prefill.hip",
+KERNEL_SOURCES = ["vq_api.hip", "vq_dequant.hip", "vq_encode.hip", "vq_generic.hip", "vq_decode.hip", "vq_decode_gemv.hip", "vq_decode_stream.hip", "vq_decode_general.hip", "vq_prefill.hip",
                   "vq_prefill_small.hip", "vq_gemm_plain.hip", "vq_gemm_tiled.hip", "vq_epilogue.hip", "vq_check.hip", "vq_noalloc.hip"]
 
 # sources with no kernel of their own (argument validation and dispatch)

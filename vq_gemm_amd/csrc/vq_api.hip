@@ -75,6 +75,11 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_wide_rotate_priority", &Tuning::gemv_wide_rotate_priority},
     {"gemv_wide_min_units_share", &Tuning::gemv_wide_min_units_share},
     {"decode_replicated_table_min_tiles", &Tuning::decode_replicated_table_min_tiles},
+    {"decode_stream_min_k", &Tuning::decode_stream_min_k},
+    {"decode_stream_min_m", &Tuning::decode_stream_min_m},
+    {"decode_stream_max_m", &Tuning::decode_stream_max_m},
+    {"decode_stream_max_groups_per_unit", &Tuning::decode_stream_max_groups_per_unit},
+    {"decode_stream_replicated_min_gathers", &Tuning::decode_stream_replicated_min_gathers},
     {"splitk_fixed_us", &Tuning::splitk_fixed_us},
     {"splitk_us_per_partial_mb", &Tuning::splitk_us_per_partial_mb},
     {"splitk_force_splits", &Tuning::splitk_force_splits},

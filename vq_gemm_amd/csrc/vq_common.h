@@ -107,6 +107,11 @@ bool decode_gemv_preferred(const ProblemB &p);
 bool decode_general_supports(const ProblemB &p);
 hipError_t launch_decode_general(const ProblemB &p, hipStream_t s);
 
+// the streaming kernel behind launch_decode_b for long rows of W (vq_decode_stream.hip): 8-vectors, 8-bit codes
+bool decode_stream_supports(const ProblemB &p);
+bool decode_stream_preferred(const ProblemB &p);
+hipError_t launch_decode_stream(const ProblemB &p, hipStream_t s);
+
 // whether the batched K-sliced decode kernel takes the shape with its gated epilogue (p.gated set)
 bool decode_gated_supports(const ProblemB &p);
 // expected microseconds of the batched decode kernel for tall X (more rows than the general kernel serves); 1e30 otherwise
@@ -198,6 +203,14 @@ struct Tuning {
     double gemv_wide_rotate_priority = 1.0;
     // batched decode kernel: the bank-replicated table (64 KB to fill) from this many tiles per workgroup on
     double decode_replicated_table_min_tiles = 2.0;
+    // streaming decode kernel (whole K per workgroup, K dealt to the waves in pieces): taken by the K-sliced path from
+    // this K on (the batched kernel walks K beyond 4096 in chunks) for this range of rows of X and at most this many
+    // groups of tiles per compute unit, and its bank-replicated table from this many gathers per lane on
+    double decode_stream_min_k = 12288.0;
+    double decode_stream_min_m = 9.0;
+    double decode_stream_max_m = 16.0;
+    double decode_stream_max_groups_per_unit = 1.0;
+    double decode_stream_replicated_min_gathers = 0.0;
     // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums
     // written and read once (microseconds per MB of partial sums)
     double splitk_fixed_us = 4.5;

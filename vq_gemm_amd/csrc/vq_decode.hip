@@ -922,6 +922,8 @@ bool decode_gemv_preferred(const ProblemB &p)
 hipError_t launch_decode_b(const ProblemB &p, hipStream_t s)
 {
     if (!decode_supports(p)) return hipErrorInvalidValue;
+    // long rows of W: the streaming kernel (the batched kernel would walk K in chunks)
+    if (decode_stream_preferred(p)) return launch_decode_stream(p, s);
     const bool u8 = p.code_bits == 8;
     if (batched_supports(p)) {
         // one launch, the 16-row slabs of X on the second grid dimension
