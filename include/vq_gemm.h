@@ -40,9 +40,10 @@ extern "C" {
 #define VQGEMM_VARIANT_GENERIC 1  /* simple scalar kernel, any shape */
 #define VQGEMM_VARIANT_DECODE 2   /* small and medium M, 16 rows of X per workgroup: K-sliced waves, 16x16x32 MFMA,
                                      LDS-resident codebook; M <= 4096 when K % 256 == 0, N % 16 == 0 and
-                                     (N / n_codebooks) % 16 == 0, M <= 64 otherwise.  Nine to sixteen rows of X on
-                                     K >= 12288 (8-vectors, 8-bit codes, few tiles per compute unit) go through the
-                                     streaming kernel of this path: K dealt to the waves in pieces, no chunks of K */
+                                     (N / n_codebooks) % 16 == 0, M <= 64 otherwise.  Up to sixteen rows of X on long
+                                     rows of W (K >= 8192, 8-vectors, 8-bit codes, few tiles per compute unit) go
+                                     through the streaming kernel of this path: K dealt to the waves in pieces, no
+                                     chunks of K */
 #define VQGEMM_VARIANT_PREFILL 3  /* large M: 256x256 tiles of 16x16x32 MFMAs, codewords gathered into operands;
                                      256x128 tiles when those put more compute units to work */
 #define VQGEMM_VARIANT_TWOPASS 4  /* dequantise to HBM scratch, then the plain fp16 GEMM */

@@ -158,10 +158,10 @@ BATCHED_B = [
 @pytest.fixture
 def batched_kernel_for_long_k():
     """The K-sliced path with its streaming kernel switched off: long K goes through the batched kernel's chunks."""
-    before = cabi.tuning()["decode_stream_min_k"]
-    cabi.set_tuning(decode_stream_min_k=1e8)
+    before = {k: cabi.tuning()[k] for k in ("decode_stream_min_k", "decode_stream_min_k_few_rows")}
+    cabi.set_tuning(decode_stream_min_k=1e8, decode_stream_min_k_few_rows=1e8)
     yield
-    cabi.set_tuning(decode_stream_min_k=before)
+    cabi.set_tuning(**before)
 
 
 @pytest.mark.parametrize("row", BATCHED_B, ids=[r[0] for r in BATCHED_B])
@@ -228,7 +228,7 @@ def test_streaming_decode_kernel(row):
     before = cabi.tuning()
     try:
         for gathers in (0.0, 1e8):   # the bank-replicated table, the plain table
-            cabi.set_tuning(decode_stream_min_k=0.0, decode_stream_min_m=0.0, decode_stream_max_m=1e8, decode_stream_max_groups_per_unit=1e8,
+            cabi.set_tuning(decode_stream_min_k=0.0, decode_stream_min_k_few_rows=0.0, decode_stream_min_m=0.0, decode_stream_max_m=1e8, decode_stream_max_groups_per_unit=1e8,
                             decode_stream_replicated_min_gathers=gathers)
             y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
             torch.cuda.synchronize()
@@ -252,7 +252,7 @@ def test_streaming_decode_kernel(row):
             eb, _ = vo.rel_err(_np(yb), ref + _np(bias).astype(np.float64))
             assert eb <= TOL
         # the batched kernel on the same inputs: the same product within the bar
-        cabi.set_tuning(decode_stream_min_k=1e8)
+        cabi.set_tuning(decode_stream_min_k=1e8, decode_stream_min_k_few_rows=1e8)
         if K % 256 == 0:
             yd = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE)
             scale = yd.float().abs().max().item()

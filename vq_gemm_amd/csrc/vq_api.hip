@@ -76,6 +76,7 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_wide_min_units_share", &Tuning::gemv_wide_min_units_share},
     {"decode_replicated_table_min_tiles", &Tuning::decode_replicated_table_min_tiles},
     {"decode_stream_min_k", &Tuning::decode_stream_min_k},
+    {"decode_stream_min_k_few_rows", &Tuning::decode_stream_min_k_few_rows},
     {"decode_stream_min_m", &Tuning::decode_stream_min_m},
     {"decode_stream_max_m", &Tuning::decode_stream_max_m},
     {"decode_stream_max_groups_per_unit", &Tuning::decode_stream_max_groups_per_unit},

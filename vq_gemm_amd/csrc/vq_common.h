@@ -206,8 +206,9 @@ struct Tuning {
     // streaming decode kernel (whole K per workgroup, K dealt to the waves in pieces): taken by the K-sliced path from
     // this K on (the batched kernel walks K beyond 4096 in chunks) for this range of rows of X and at most this many
     // groups of tiles per compute unit, and its bank-replicated table from this many gathers per lane on
-    double decode_stream_min_k = 12288.0;
-    double decode_stream_min_m = 9.0;
+    double decode_stream_min_k = 8192.0;
+    double decode_stream_min_k_few_rows = 14336.0;  // with eight rows of X or fewer
+    double decode_stream_min_m = 1.0;
     double decode_stream_max_m = 16.0;
     double decode_stream_max_groups_per_unit = 1.0;
     double decode_stream_replicated_min_gathers = 0.0;

@@ -97,7 +97,11 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
         const half_t *cbg = cb + (int64_t)(tile0 * kTile / rows_per_cb) * entries * 8;
         const int e = (tid >> 1) & 255, h = tid & 1;
         uint4_t entry = reinterpret_cast<const uint4_t *>(cbg)[min(e, entries - 1)];
-        const int last_piece = min(w + kStreamWaves * (max(n_mine, 1) - 1), n_pieces - 1);
+        // (the count of the wave's pieces goes through an empty asm once per group, so that the fourteen comparisons
+        // with it are not all made ahead of the loop over the groups and kept in scalar registers)
+        int n_mine_g = n_mine;
+        asm volatile("" : "+s"(n_mine_g));
+        const int last_piece = min(w + kStreamWaves * (max(n_mine_g, 1) - 1), n_pieces - 1);
         auto piece_of = [&](int i) { return min(w + kStreamWaves * i, last_piece); };
         // (the lane offsets go through an empty asm once per group: what does not change from group to group - X
         // altogether, the lane's part of every address - would otherwise be computed, or loaded, ahead of the loop over
@@ -114,20 +118,24 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
         // has to cover the latency of the L2 at the rate the unit's L1 delivers: 16 waves x 2 pieces x 4 KB), one in
         // the block, one in operand registers
         // (with many code registers one piece less: its iterations are longer, and the registers are needed)
-        constexpr int kXRing = NP * T >= 16 ? 2 : 3;
+        constexpr int kXRing = (NP * T >= 16 || NP > 8) ? 2 : 3;
         uint4_t xs[kXRing][4];
         auto load_x = [&](int i, uint4_t (&xd)[4]) {
             const uint32_t piece_off = (uint32_t)(piece_of(i) * (kPieceK * 2));
 #pragma unroll
             for (int j = 0; j < 4; j++) xd[j] = *reinterpret_cast<const uint4_t *>(x_slab + (uint32_t)(x_off[j] + piece_off));
         };
+        // (only the rows of X that exist go through the LDS: the traffic of a piece is what the stream waits for)
         auto stage_x = [&](const uint4_t (&xd)[4]) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) x_block[j * 64 + lane] = xd[j];
+            for (int j = 0; j < 4; j++)
+                if (4 * j < M) x_block[j * 64 + lane] = xd[j];
         };
         auto pick_x = [&](uint4_t (&xo)[kPieceSteps]) {
+            if (r16 < M) {
 #pragma unroll
-            for (int s2 = 0; s2 < kPieceSteps; s2++) xo[s2] = x_block[x_read_slot + (((kq * 4 + s2) ^ r16) & 15)];
+                for (int s2 = 0; s2 < kPieceSteps; s2++) xo[s2] = x_block[x_read_slot + (((kq * 4 + s2) ^ r16) & 15)];
+            }
         };
         // (the first pieces of X go out ahead of the codes: they come out of the L2 and are in the block and in operand
         // registers by the time the codes arrive from HBM)
@@ -189,23 +197,24 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
         // piece 0 into the block and out of it into operand registers; then per piece: the next piece into the block and
         // out of it into the other set of operand registers (the wave's own LDS operations complete in order), the piece
         // after the ring requested, the multiply
-        // (with the most code registers a single set of operand registers, picked up in front of the multiply)
-        constexpr int kXO = NP * T > 24 ? 1 : 2;
+        // (with two tiles a single set of operand registers, picked up in front of the multiply)
+        constexpr int kXO = T > 1 ? 1 : 2;
         uint4_t xo[kXO][kPieceSteps];
         stage_x(xs[0]);
         if (kXO == 2) pick_x(xo[0]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < NP; i++) {
-            if (kXO == 1) pick_x(xo[0]);
-            if (i + 1 < NP) {
+            if (kXO == 1 && i < n_mine_g) pick_x(xo[0]);
+            // (pieces past the wave's last are requested - clamped - but not put through the LDS)
+            if (i + 1 < NP && i + 1 < n_mine_g) {
                 stage_x(xs[(i + 1) % kXRing]);
                 if (kXO == 2) pick_x(xo[(i + 1) % kXO]);
             }
             __builtin_amdgcn_sched_barrier(0);
             if (i + kXRing < NP) load_x(i + kXRing, xs[i % kXRing]);  // (the slot of piece i, which went into the block one piece ago)
             __builtin_amdgcn_sched_barrier(0);
-            if (i < n_mine) multiply_piece(xo[i % kXO], cw[i]);
+            if (i < n_mine_g) multiply_piece(xo[i % kXO], cw[i]);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (T > 0) __syncthreads();  // every wave is done with its block of X: the partial tiles lie over the blocks
@@ -274,14 +283,14 @@ bool decode_stream_supports(const ProblemB &p)
 }
 
 // Where it was measured ahead of the batched kernel's chunks (cold, 256 units, batched -> this): 9 to 16 rows of X on
-// K from 12288 on with at most one group of tiles per unit - M = 16: K = 14336 / N = 4096 17.4 -> 14.0 us, 28672 / 8192
-// 37.1 -> 29.0; M = 8 is a tie (14.4 / 13.6), fewer rows, K = 8192 and 11008, more tiles per unit and taller X lose.
-// What a piece costs does not depend on M: every piece of X goes through the LDS as 16 rows (write, read, and the
-// gathers beside them), and that traffic is what the stream waits for.
+// K from 8192 on, fewer rows from 14336 on (at K = 12288 two rows lose 4 to 12 %), with at most one group of tiles per unit.  M = 16: K = 14336 / N = 4096 17.3 -> 13.1 us, 28672 / 8192
+// 37.2 -> 28.3, 8192 / 8192 13.3 -> 11.8, 11008 / 4096 13.9 -> 12.4; M = 4: 13.0 -> 10.9, 25.6 -> 23.6, 9.9 -> 9.8,
+// 10.6 -> 10.6; M = 2: 12.5 -> 10.9, 24.8 -> 23.4, 9.7 -> 9.8, 10.2 -> 10.5.  More groups per unit (N = 28672) and
+// taller X (one workgroup per 16-row slab, the codes read again by each) stay with the batched kernel: 0.5 - 0.9x.
 bool decode_stream_preferred(const ProblemB &p)
 {
     const Tuning &tn = tuning();
-    if (!decode_stream_supports(p) || (double)p.K < tn.decode_stream_min_k) return false;
+    if (!decode_stream_supports(p) || (double)p.K < (p.M <= 8 ? tn.decode_stream_min_k_few_rows : tn.decode_stream_min_k)) return false;
     if ((double)p.M < tn.decode_stream_min_m || (double)p.M > tn.decode_stream_max_m) return false;
     const int t = stream_tiles_per_group(p);
     const int n_groups = (p.N / kTile + t - 1) / t;

@@ -185,8 +185,14 @@ def fit(device: str = "cuda:0", verbose: bool = True) -> dict:
         out["decode_tile_us"] = tile
         out["decode_prologue_us"] = max(t1 - tile, 0.5)
         say(f"decode, K=4096: {t1:.2f} us at one tile per unit, {t8:.2f} us at eight: {tile:.3f} us per tile")
-    t1c = _t(16, 8192, 16 * cus, cabi.VARIANT_DECODE)
-    t8c = _t(16, 8192, 128 * cus, cabi.VARIANT_DECODE)
+    # (the batched kernel's chunks of K: its streaming sibling, which would take the first of these shapes, is switched off)
+    stream_was = {k: cabi.tuning()[k] for k in ("decode_stream_min_k", "decode_stream_min_k_few_rows")}
+    cabi.set_tuning(decode_stream_min_k=1e8, decode_stream_min_k_few_rows=1e8)
+    try:
+        t1c = _t(16, 8192, 16 * cus, cabi.VARIANT_DECODE)
+        t8c = _t(16, 8192, 128 * cus, cabi.VARIANT_DECODE)
+    finally:
+        cabi.set_tuning(**stream_was)
     if t1c and t8c:
         out["decode_tile_chunked_us"] = (t8c - t1c) / 7.0 / 2.0   # per 4096 k
         say(f"decode, K=8192 (two chunks): {(t8c - t1c) / 7.0:.3f} us per tile")
