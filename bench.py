@@ -52,6 +52,7 @@ PROFILED_TRAFFIC = {
     "decode_qkv_m1_k4096_n12288": (6_578_000, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
     "decode_down_m1_k14336_n4096": (7_692_288, "profiles/decode_gemv_wide_kernel_long_k_down_projection.md"),
     "decode_down_m1_k28672_n8192": (29_952_000, "profiles/decode_gemv_wide_kernel_long_k_down_projection.md"),
+    "decode_down_m16_k14336_n4096": (11_270_000, "profiles/decode_stream_kernel_m16_k14336_n4096.md"),
     "C4": (85_373_000, "profiles/prefill_kernel_c4_prefill_gemm.md"),
     "C5": (489_400_000, "profiles/prefill_kernel_c5_m2048_k8192_n28672.md"),
 }
@@ -423,6 +424,10 @@ def main():
             max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         others["decode_down_m1_k28672_n8192"], _ = bench_config(
             ProblemSpec("decode_down_m1_k28672_n8192", GEOM_B, 1, 28672, 8192, 8, 256, 1, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        # the same down-projection at a batch of sixteen: the streaming kernel of the K-sliced path
+        others["decode_down_m16_k14336_n4096"], _ = bench_config(
+            ProblemSpec("decode_down_m16_k14336_n4096", GEOM_B, 16, 14336, 4096, 8, 256, 1, 8),
             max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         others["C1"], _ = bench_config("C1", max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=False)
         others["C4"], _ = bench_config("C4", 40, 10, cold_pool=False)
