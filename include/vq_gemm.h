@@ -102,9 +102,11 @@ int vqgemm_e2e_gemm_b_bias(const void *x, const void *codes, const void *codeboo
 
 /*
  * vqgemm_e2e_gemm_b_bias with a workspace whose size the library is told, so that the automatic choice may use
- * kernels that need scratch memory: today split K (VQGEMM_VARIANT_PREFILL_SPLITK), which VQGEMM_VARIANT_AUTO takes
- * where its cost model expects at least 10 % over what it would launch otherwise and `workspace_bytes` suffices
- * (a workspace that is too small, or NULL, is no error for AUTO: it does without).  vqgemm_workspace_bytes_b says
+ * kernels that need scratch memory: split K over every 128x128 tile (VQGEMM_VARIANT_PREFILL_SPLITK), which
+ * VQGEMM_VARIANT_AUTO takes where its cost model expects at least 10 % over what it would launch otherwise, and -
+ * where the large tiles of a shape are a few more than whole rounds over the compute units - those whole rounds as
+ * one launch and the columns of W that are left over as a second one, in 128x128 tiles with K split there; either
+ * only when `workspace_bytes` suffices (a workspace that is too small, or NULL, is no error for AUTO: it does without).  vqgemm_workspace_bytes_b says
  * how many bytes the given variant (AUTO, PREFILL_SPLITK, TWOPASS) wants for a shape: 0 when it uses none, a
  * negative error for an invalid shape.  `workspace` must be 256-byte aligned device memory; its contents before the
  * call do not matter and are undefined after it; two calls that overlap in time need a workspace each.  An explicit

@@ -1593,6 +1593,56 @@ def test_split_k_against_the_oracle_and_from_run_to_run(row):
     assert vo.rel_err(_np(ya), want)[0] <= TOL
 
 
+# Whole rounds of large tiles over the first columns of W, the left-over columns in 128x128 tiles with K split: shapes
+# whose large tiles are a few more than a round on a 256-unit device (K kept short: the oracle multiplies all of it).
+TAIL_SPLIT_B = [
+    # name, M, K, N, vec, E, bits, G
+    ("wide_head_258_tiles", 1536, 512, 11008, 8, 256, 8, 1),
+    ("narrow_head_258_tiles_86_books", 768, 1024, 11008, 8, 256, 8, 86),
+    ("ragged_m_and_last_column", 1500, 512, 11008 + 72, 8, 256, 8, 1),
+    ("u16_v4", 1536, 512, 11008, 4, 1024, 16, 2),
+]
+
+
+@pytest.mark.parametrize("row", TAIL_SPLIT_B, ids=[r[0] for r in TAIL_SPLIT_B])
+def test_whole_rounds_of_large_tiles_then_the_left_over_columns_with_k_split(row):
+    name, M, K, N, v, E, bits, G = row
+    spec = ProblemSpec(name, GEOM_B, M, K, N, v, E, G, bits, codebook_3d=(G > 1), codebook_std=0.05)
+    x, codes, cb = make_problem(spec, seed=71, device=DEV)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(72)) * 0.5).half().to(DEV)
+    w = vo.dequant_b(_np(codes), _np(cb)).astype(np.float64)
+    xf = _np(x).astype(np.float64)
+    want = np.concatenate([xf @ w[r:r + 2048].T for r in range(0, N, 2048)], axis=1)
+    before = cabi.tuning()
+    try:
+        cabi.set_tuning(tail_split_margin=0.0)
+        y_single = cabi.e2e_gemm_b_ws(x, codes, cb).clone()           # the best single plan
+        cabi.set_tuning(tail_split_margin=1e6, splitk_force_splits=2) # the two-launch plan wherever it exists, K in two slices
+        need = cabi.workspace_bytes_b(M, K, N, v, E, G, bits)
+        assert need > 0, "every shape of this list leaves columns over, and K can be split there"
+        ws = torch.empty(need, dtype=torch.uint8, device=DEV).random_()
+        for b, ref in ((None, want), (bias, want + _np(bias).astype(np.float64)[None, :])):
+            _say("tail split", name, "bias" if b is not None else "")
+            y = cabi.e2e_gemm_b_ws(x, codes, cb, workspace=ws, bias=b).clone()
+            torch.cuda.synchronize()
+            e1, e2 = vo.rel_err(_np(y), ref)
+            _say(f"    rel_err(floor)={e1:.3e} max/max={e2:.3e}")
+            assert e1 <= TOL, (name, e1, e2)
+            for _ in range(3):   # the same bits whoever finishes last, whatever the workspace held
+                ws.random_()
+                assert torch.equal(cabi.e2e_gemm_b_ws(x, codes, cb, workspace=ws, bias=b), y)
+        # the columns of the first launch are the single plan's bits where that plan used the same tiles; all of Y is close
+        y2 = cabi.e2e_gemm_b_ws(x, codes, cb, workspace=ws)
+        assert vo.rel_err(_np(y2), _np(y_single).astype(np.float64))[0] <= 2e-3
+        # (it is this plan that ran: K split over every tile would need a slot per tile and slice)
+        assert need < cabi.workspace_bytes_b(M, K, N, v, E, G, bits, cabi.VARIANT_PREFILL_SPLITK) // 4
+        # a workspace that is too small is no obstacle: the automatic choice does without
+        ya = cabi.e2e_gemm_b_ws(x, codes, cb, workspace=torch.empty(256, dtype=torch.uint8, device=DEV))
+        assert vo.rel_err(_np(ya), want)[0] <= TOL
+    finally:
+        cabi.set_tuning(**before)
+
+
 def test_split_k_scoped_accesses_equal_the_textbook_fences_bit_for_bit():
     # The exchange moves partial sums with device-scope loads and stores and hand-written waits; the library also
     # carries the release / acquire fences the memory model asks for, behind a switch of the tuning table.  Same

@@ -81,6 +81,7 @@ const TuningEntry kTuningEntries[] = {
     {"decode_stream_max_m", &Tuning::decode_stream_max_m},
     {"decode_stream_max_groups_per_unit", &Tuning::decode_stream_max_groups_per_unit},
     {"decode_stream_replicated_min_gathers", &Tuning::decode_stream_replicated_min_gathers},
+    {"tail_split_margin", &Tuning::tail_split_margin},
     {"splitk_fixed_us", &Tuning::splitk_fixed_us},
     {"splitk_us_per_partial_mb", &Tuning::splitk_us_per_partial_mb},
     {"splitk_force_splits", &Tuning::splitk_force_splits},
@@ -344,10 +345,12 @@ namespace {
 
 // Split K with the cost model's number of slices when that is expected to beat what the automatic choice would
 // launch otherwise by a margin (and then at least two slices); 0: do not split.
-int splitk_auto(const ProblemB &p, bool all_aligned16)
+int splitk_auto(const ProblemB &p, bool all_aligned16, double *t_best = nullptr, int *plain_variant = nullptr)
 {
+    if (t_best) *t_best = 1e30;
     if (p.K == 0 || !all_aligned16 || p.gated) return 0;
     const int plain = select_b(p, all_aligned16);
+    if (plain_variant) *plain_variant = plain;
     double t_plain;
     if (plain == VQGEMM_VARIANT_PREFILL) t_plain = prefill_cost_us(p);
     else if (plain == VQGEMM_VARIANT_DECODE) t_plain = decode_cost_us(p);
@@ -355,7 +358,37 @@ int splitk_auto(const ProblemB &p, bool all_aligned16)
     if (t_plain >= 1e29) return 0;  // (short X: the decode path is taken without a comparison, and stays)
     double t_split = 1e30;
     const int sp = prefill_splitk_choice(p, &t_split, 2);
-    return sp >= 2 && t_split < 0.9 * t_plain ? sp : 0;
+    const bool take = sp >= 2 && t_split < 0.9 * t_plain;
+    if (t_best) *t_best = take ? t_split : t_plain;
+    return take ? sp : 0;
+}
+
+// What the automatic choice does with a workspace: nothing, K split over every 128x128 tile (sp slices), or whole rounds
+// of large tiles with the left-over columns in 128x128 tiles and K split there (tail) - whichever the cost models
+// expect to be fastest by a margin.
+struct WorkspaceChoice {
+    int sp;
+    TailSplitPlan tail;
+    size_t bytes;
+};
+WorkspaceChoice workspace_auto(const ProblemB &p, bool all_aligned16)
+{
+    WorkspaceChoice c = {0, {false, 0, 0, 0, 1e30, 0}, 0};
+    double t_best = 1e30;
+    int plain = 0;
+    c.sp = splitk_auto(p, all_aligned16, &t_best, &plain);
+    if (c.sp >= 2) c.bytes = prefill_splitk_workspace_bytes(p, c.sp);
+    if (plain == VQGEMM_VARIANT_PREFILL && t_best < 1e29) {
+        const TailSplitPlan tail = prefill_tail_split_plan(p);
+        // (a margin of 1000 and more: wherever the plan exists - for measurements and tests)
+        const double margin = tuning().tail_split_margin;
+        if (tail.ok && (margin >= 1e3 || tail.cost_us < margin * t_best)) {
+            c.sp = 0;
+            c.tail = tail;
+            c.bytes = tail.workspace_bytes;
+        }
+    }
+    return c;
 }
 
 }  // namespace
@@ -368,9 +401,9 @@ int64_t vqgemm_workspace_bytes_b(int64_t M, int64_t K, int64_t N, int32_t vec, i
     if (M == 0 || N == 0 || K == 0) return 0;
     const ProblemB p = make_b(nullptr, nullptr, nullptr, nullptr, M, K, N, vec, entries, n_codebooks, code_bits);
     if (variant == VQGEMM_VARIANT_TWOPASS) return N * K * 2;
+    if (variant == VQGEMM_VARIANT_AUTO) return (int64_t)workspace_auto(p, true).bytes;
     int sp = 0;
-    if (variant == VQGEMM_VARIANT_AUTO) sp = splitk_auto(p, true);
-    else if (variant == VQGEMM_VARIANT_PREFILL_SPLITK) sp = prefill_splitk_choice(p, nullptr, 2);
+    if (variant == VQGEMM_VARIANT_PREFILL_SPLITK) sp = prefill_splitk_choice(p, nullptr, 2);
     return sp >= 2 ? (int64_t)prefill_splitk_workspace_bytes(p, sp) : 0;
 }
 
@@ -400,7 +433,10 @@ int vqgemm_e2e_gemm_b_ws(const void *x, const void *codes, const void *codebook,
         if (sp < 2) return VQGEMM_E_VARIANT;
         if ((int64_t)prefill_splitk_workspace_bytes(p, sp) > workspace_bytes) return VQGEMM_E_SCRATCH;
     } else {
-        sp = splitk_auto(p, a16);
+        const WorkspaceChoice c = workspace_auto(p, a16);
+        if (c.tail.ok && (int64_t)c.bytes <= workspace_bytes)
+            return static_cast<int>(launch_prefill_tail_split(p, c.tail, static_cast<hipStream_t>(stream), workspace));
+        sp = c.tail.ok ? splitk_auto(p, a16) : c.sp;
         // (a workspace that is too small is not an error for the automatic choice: it does without)
         if (sp < 2 || (int64_t)prefill_splitk_workspace_bytes(p, sp) > workspace_bytes)
             return vqgemm_e2e_gemm_b_bias(x, codes, codebook, bias, y, M, K, N, vec, entries, n_codebooks, code_bits, VQGEMM_VARIANT_AUTO,

@@ -126,11 +126,25 @@ double prefill_cost_us(const ProblemB &p);
 // 1 = 256x256, 2 = 256x128
 hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile = 0);
 
+// Whole rounds of large tiles over the first columns of W, the columns that are left in 128x128 tiles with K split
+// (needs a workspace when splits > 1): the plan with its expected time, and its two launches.
+struct TailSplitPlan {
+    bool ok;
+    int head_tile;   // 1: 256x256 tiles, 2: 256x128 tiles over the W rows [0, n_split)
+    int n_split;     // the 128x128 kernel takes the W rows [n_split, N)
+    int splits;      // slices of K there (1: none)
+    double cost_us;
+    size_t workspace_bytes;
+};
+TailSplitPlan prefill_tail_split_plan(const ProblemB &p);
+hipError_t launch_prefill_tail_split(const ProblemB &p, const TailSplitPlan &plan, hipStream_t s, void *workspace);
+
 // the prefill kernel with 128x128 tiles (vq_prefill_small.hip), for medium M
 bool prefill_small_supports(const ProblemB &p);
 double prefill_small_cost_us(const ProblemB &p);  // expected time, microseconds (1e30: not supported)
 // splits > 1: split K, `splits` workgroups per tile (workspace of prefill_splitk_workspace_bytes, device memory)
-hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s, int splits = 1, void *workspace = nullptr);
+// n_begin > 0: the W rows [n_begin, N) only (a multiple of 128; the workspace is then sized for those columns)
+hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s, int splits = 1, void *workspace = nullptr, int n_begin = 0);
 bool prefill_splitk_supports(const ProblemB &p, int splits);
 size_t prefill_splitk_counter_bytes(int64_t tiles);
 size_t prefill_splitk_workspace_bytes(const ProblemB &p, int splits);
@@ -212,6 +226,9 @@ struct Tuning {
     double decode_stream_max_m = 16.0;
     double decode_stream_max_groups_per_unit = 1.0;
     double decode_stream_replicated_min_gathers = 0.0;
+    // whole rounds of large tiles plus the left-over columns in 128x128 tiles with K split: taken with a workspace when
+    // expected below this share of the best single plan (0: never; 1000 and more: wherever the plan exists)
+    double tail_split_margin = 0.93;
     // split K over 128x128 tiles: the clearing launch and the last workgroup's extra pass, and the partial sums
     // written and read once (microseconds per MB of partial sums)
     double splitk_fixed_us = 4.5;

@@ -876,15 +876,17 @@ TilePlan plan_tiles(const ProblemB &p)
     return best;
 }
 
-// tile: 0 = as planned, 1 = 256x256 only, 2 = 256x128 only
+// tile: 0 = as planned, 1 = 256x256 only, 2 = 256x128 only.  n_end > 0: only the W rows [0, n_end) (a multiple of 256;
+// the rest of the columns is another launch's)
 template <int VEC, typename CodeT>
-hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
+hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile, int n_end = 0)
 {
     const bool tail = (p.K % kStageK) != 0;
     const int tiles_m = (p.M + BM - 1) / BM;
-    int n_split = p.N;
+    if (n_end <= 0 || n_end > p.N) n_end = p.N;
+    int n_split = n_end;
     if (tile == 2) n_split = 0;
-    else if (tile == 0) n_split = plan_tiles<VEC, CodeT>(p).n_split;
+    else if (tile == 0) n_split = min(plan_tiles<VEC, CodeT>(p).n_split, n_end);
     if (n_split > 0) {
         const int tiles_n = (n_split + BN - 1) / BN;
         const int n_cb = codebooks_per_tile(p, BN);
@@ -910,9 +912,9 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (n_split < p.N) {
+    if (n_split < n_end) {
         if (lds_bytes_narrow<VEC, CodeT>(p) > kLdsLimit) return hipErrorInvalidValue;
-        const int tiles_n = (p.N - n_split + BNN - 1) / BNN;
+        const int tiles_n = (n_end - n_split + BNN - 1) / BNN;
         const size_t smem = lds_bytes_narrow<VEC, CodeT>(p);
         constexpr bool can_split = VEC == 8 && sizeof(CodeT) == 1;
         const bool split = can_split && split_layout_applies(p, codebooks_per_tile(p, BNN), kStageBytes);
@@ -921,7 +923,7 @@ hipError_t launch_prefill_typed(const ProblemB &p, hipStream_t s, int tile)
         hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(kThreads), smem, s, p.x,
-                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, n_split, p.N, p.entries,
+                           static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, n_end, n_split, p.N, p.entries,
                            p.rows_per_cb, tiles_m, tiles_n, codebooks_per_tile(p, BNN), p.gated ? 1 : 0);
         return hipGetLastError();
     }
@@ -993,6 +995,55 @@ double prefill_cost_us(const ProblemB &p)
     if (!what.wide) return what.cost_us;
     const double small = prefill_small_cost_us(p);
     return small < kSmallTileMargin * what.cost_us ? small : what.cost_us;
+}
+
+// ---- whole rounds of large tiles, then the columns that are left in 128x128 tiles with K split ------------------
+// A launch whose large tiles are a few more than a multiple of the compute units pays a whole further round for them.
+// With a workspace the left-over columns go to the 128x128 kernel instead, K split over as many workgroups as fill
+// the device: the second launch then takes a fraction of a round (M = 1536, K = 4096, N = 11008: 6 x 43 = 258 tiles of
+// 256x256 on 256 units; 42 columns make one round, the 43rd is 48 small tiles with K in 8 slices).
+TailSplitPlan prefill_tail_split_plan(const ProblemB &p)
+{
+    TailSplitPlan best = {false, 0, 0, 0, 1e30, 0};
+    if (p.gated || !prefill_supports(p) || !prefill_small_supports(p)) return best;
+    const int cus = device_cu_count(), tiles_m = (p.M + BM - 1) / BM;
+    const bool narrow_ok = prefill_narrow_supports(p);
+    for (int head_tile = 1; head_tile <= 2; head_tile++) {
+        if (head_tile == 2 && !narrow_ok) break;
+        const int bn = head_tile == 1 ? BN : BNN;
+        const int cols = (p.N + bn - 1) / bn;
+        const int64_t rounds = (int64_t)tiles_m * cols / cus;
+        // as many columns as whole rounds hold (in whole 256-row steps, so that either tile can serve them)
+        int cols_head = (int)(rounds * cus / tiles_m);
+        if (head_tile == 2) cols_head &= ~1;
+        if (rounds < 1 || cols_head < 1 || cols_head >= cols) continue;
+        const int n_split = cols_head * bn;
+        ProblemB tail = p;  // the left-over columns as the 128x128 kernel's cost model sees them
+        tail.N = p.N - n_split;
+        double t_tail = 1e30;
+        int sp = prefill_splitk_choice(tail, &t_tail, 1);
+        if (sp < 1 || t_tail >= 1e29) continue;
+        // (Tuning::splitk_force_splits, for measurements and tests: that many slices where the shape allows)
+        const int forced = (int)tuning().splitk_force_splits;
+        if (forced >= 2 && prefill_splitk_supports(tail, forced)) sp = forced;
+        const double t = tile_cost_us(p, bn, cols_head) + t_tail + 3.0;
+        if (t < best.cost_us) best = {true, head_tile, n_split, sp, t, sp > 1 ? prefill_splitk_workspace_bytes(tail, sp) : 0};
+    }
+    return best;
+}
+
+hipError_t launch_prefill_tail_split(const ProblemB &p, const TailSplitPlan &plan, hipStream_t s, void *workspace)
+{
+    if (!plan.ok || plan.n_split <= 0 || plan.n_split >= p.N || plan.n_split % BN != 0) return hipErrorInvalidValue;
+    const bool u8 = p.code_bits == 8;
+    hipError_t e;
+    switch (p.vec) {
+    case 8: e = u8 ? launch_prefill_typed<8, uint8_t>(p, s, plan.head_tile, plan.n_split) : launch_prefill_typed<8, uint16_t>(p, s, plan.head_tile, plan.n_split); break;
+    case 4: e = u8 ? launch_prefill_typed<4, uint8_t>(p, s, plan.head_tile, plan.n_split) : launch_prefill_typed<4, uint16_t>(p, s, plan.head_tile, plan.n_split); break;
+    default: e = u8 ? launch_prefill_typed<2, uint8_t>(p, s, plan.head_tile, plan.n_split) : hipErrorInvalidValue;
+    }
+    if (e != hipSuccess) return e;
+    return launch_prefill_small_b(p, s, plan.splits, workspace, plan.n_split);
 }
 
 hipError_t launch_prefill_b(const ProblemB &p, hipStream_t s, int tile)

@@ -51,7 +51,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                                                                     const half_t *__restrict__ cb,
                                                                     half_t *__restrict__ y,
                                                                     const half_t *__restrict__ bias, int M, int K,
-                                                                    int N, int entries, int rows_per_cb, int tiles_m,
+                                                                    int N, int n_begin, int ldn, int entries,
+                                                                    int rows_per_cb, int tiles_m,
                                                                     int tiles_n, int cb_lds_count, int gated, int k_len,
                                                                     int splits, float4_t *__restrict__ partials,
                                                                     unsigned int *__restrict__ counters, int fenced)
@@ -79,7 +80,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
     int wg = (int)blockIdx.x - split * n_wg;
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
     const int tm = wg / tiles_n, tn = wg % tiles_n;
-    const int m0 = tm * SBM, n0 = tn * SBN;
+    // The launch covers the W rows (columns of Y) [n_begin, N) of a problem with ldn rows in all.
+    const int m0 = tm * SBM, n0 = n_begin + tn * SBN;
     const int n_stage = k_len / kStageK;
     const int n_super = n_stage / C::STAGES;
 
@@ -362,7 +364,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                 const int n = n0 + wn * SWN + j * 16 + 4 * kg + e;
                 bj[j][e] = HB && n < N ? (float)bias[n] : 0.f;
             }
-        if ((N & 7) == 0) {
+        if ((ldn & 7) == 0) {
             constexpr int kPitch = 144;  // 64 fp16 + 16 bytes: rows land in different banks
             uint8_t *stage_out = smem + wave * (SWM * kPitch);
 #pragma unroll
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
                 const uint4_t v = *reinterpret_cast<const uint4_t *>(stage_out + row * kPitch + c * 16);
                 const int m = m0 + wm * SWM + row;
                 const int n = n0 + wn * SWN + c * 8;
-                if (m < M && n < N) st_global_16_streaming(y + (int64_t)m * N + n, v);
+                if (m < M && n < N) st_global_16_streaming(y + (int64_t)m * ldn + n, v);
             }
         } else {
 #pragma unroll
@@ -387,9 +389,9 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
 #pragma unroll
                 for (int j = 0; j < SNP; j++) {
                     const int n = n0 + wn * SWN + j * 16 + 4 * kg;
-                    half_t *dst = y + (int64_t)m * N + n;
+                    half_t *dst = y + (int64_t)m * ldn + n;
                     const half4_t hv = round4<HB>(acc[j][i], bj[j]);
-                    if ((N & 3) == 0 && n + 3 < N) {
+                    if ((ldn & 3) == 0 && n + 3 < N) {
                         *reinterpret_cast<half4_t *>(dst) = hv;
                     } else {
 #pragma unroll
@@ -402,8 +404,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_small_kernel(const half_t
     };
     if (gated) {
         // gate and up rows of W interleaved in groups of 16: a lane holds both factors of its outputs
-        if (bias) store_gated<SNP, SMP, true>(acc, y, bias, M, N, N, m0 + wm * SWM, n0 + wn * SWN, r16, kg);
-        else store_gated<SNP, SMP, false>(acc, y, bias, M, N, N, m0 + wm * SWM, n0 + wn * SWN, r16, kg);
+        if (bias) store_gated<SNP, SMP, true>(acc, y, bias, M, N, ldn, m0 + wm * SWM, n0 + wn * SWN, r16, kg);
+        else store_gated<SNP, SMP, false>(acc, y, bias, M, N, ldn, m0 + wm * SWM, n0 + wn * SWN, r16, kg);
         return;
     }
     if (bias) epilogue(std::true_type{});
@@ -430,13 +432,15 @@ bool small_cfg_supports(const ProblemB &p)
 // float4 slots of partial sums per tile and slice, and where the tiles' counters start inside the workspace
 constexpr size_t kPartialBytes = (size_t)SNP * SMP * kThreads * 16;  // 64 KB
 
+// n_begin: the launch covers the W rows [n_begin, N) only (a multiple of the tile's 128 rows)
 template <int VEC, typename CodeT>
-hipError_t launch_small_typed(const ProblemB &p, hipStream_t s, int splits, void *workspace)
+hipError_t launch_small_typed(const ProblemB &p, hipStream_t s, int splits, void *workspace, int n_begin)
 {
     typedef PrefillCfg<VEC, CodeT> C;
     if (!small_cfg_supports<VEC, CodeT>(p)) return hipErrorInvalidValue;
     if (splits < 1 || p.K % splits != 0 || (p.K / splits) % C::K_SUPER != 0 || (splits > 1 && !workspace)) return hipErrorInvalidValue;
-    const int tiles_m = (p.M + SBM - 1) / SBM, tiles_n = (p.N + SBN - 1) / SBN;
+    if (n_begin < 0 || n_begin >= p.N || n_begin % SBN != 0) return hipErrorInvalidValue;
+    const int tiles_m = (p.M + SBM - 1) / SBM, tiles_n = (p.N - n_begin + SBN - 1) / SBN;
     // workspace: the tiles' counters (cleared here, by a kernel: the launch may be captured), then the partial sums
     unsigned int *counters = static_cast<unsigned int *>(workspace);
     float4_t *partials = nullptr;
@@ -454,8 +458,8 @@ hipError_t launch_small_typed(const ProblemB &p, hipStream_t s, int splits, void
     const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(kThreads), smem, s, p.x,
-                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, p.entries, p.rows_per_cb,
-                       tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0, p.K / splits, splits, partials, counters,
+                       static_cast<const CodeT *>(p.codes), p.cb, p.y, p.bias, p.M, p.K, p.N, n_begin, p.N, p.entries,
+                       p.rows_per_cb, tiles_m, tiles_n, codebooks_per_tile(p, SBN), p.gated ? 1 : 0, p.K / splits, splits, partials, counters,
                        tuning().splitk_validate_fences >= 1.0 ? 1 : 0);
     return hipGetLastError();
 }
@@ -492,14 +496,14 @@ double prefill_small_cost_us(const ProblemB &p)
            (double)rounds * (p.K / 64.0 * (tn.prefill_small_stage_us_idle + (tn.prefill_small_stage_us_busy - tn.prefill_small_stage_us_idle) * busy));
 }
 
-hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s, int splits, void *workspace)
+hipError_t launch_prefill_small_b(const ProblemB &p, hipStream_t s, int splits, void *workspace, int n_begin)
 {
     if (!prefill_small_supports(p)) return hipErrorInvalidValue;
     const bool u8 = p.code_bits == 8;
     switch (p.vec) {
-    case 8: return u8 ? launch_small_typed<8, uint8_t>(p, s, splits, workspace) : launch_small_typed<8, uint16_t>(p, s, splits, workspace);
-    case 4: return u8 ? launch_small_typed<4, uint8_t>(p, s, splits, workspace) : launch_small_typed<4, uint16_t>(p, s, splits, workspace);
-    default: return launch_small_typed<2, uint8_t>(p, s, splits, workspace);
+    case 8: return u8 ? launch_small_typed<8, uint8_t>(p, s, splits, workspace, n_begin) : launch_small_typed<8, uint16_t>(p, s, splits, workspace, n_begin);
+    case 4: return u8 ? launch_small_typed<4, uint8_t>(p, s, splits, workspace, n_begin) : launch_small_typed<4, uint16_t>(p, s, splits, workspace, n_begin);
+    default: return launch_small_typed<2, uint8_t>(p, s, splits, workspace, n_begin);
     }
 }
 
