@@ -1015,6 +1015,7 @@ def test_tune_search_tries_the_kernel_parameter_candidates_cold_and_the_library_
     # candidates stay inside what the kernels are built for
     assert found["gemv_wide_rows_per_group"] in (1.0, 2.0) and found["gemv_wide_groups_in_flight"] in (2.0, 3.0)
     assert found["gemv_wide_rows_per_group_long_k"] in (1.0, 2.0) and found["gemv_wide_groups_in_flight_long_k"] in (2.0, 3.0)
+    assert found["decode_stream_min_k"] in (8192.0, 14336.0, 1e8) and found["decode_stream_min_k_few_rows"] in (8192.0, 14336.0, 1e8)
     assert cabi.tuning() == before, "the search leaves the table as it found it"
     # every candidate of the wide form's loop gives the same bits as the default (same sums in the same order per row)
     spec = ProblemSpec("cand", GEOM_B, 1, 4096, 12288, 8, 256, 3, 8, codebook_3d=True)

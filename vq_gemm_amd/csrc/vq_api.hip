@@ -68,6 +68,7 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_max_k", &Tuning::gemv_max_k},
     {"gemv_wide_min_rows_per_wave", &Tuning::gemv_wide_min_rows_per_wave},
     {"gemv_wide_plain_table_max_runs", &Tuning::gemv_wide_plain_table_max_runs},
+    {"gemv_wide_single_rows_max", &Tuning::gemv_wide_single_rows_max},
     {"gemv_wide_rows_per_group", &Tuning::gemv_wide_rows_per_group},
     {"gemv_wide_groups_in_flight", &Tuning::gemv_wide_groups_in_flight},
     {"gemv_wide_rows_per_group_long_k", &Tuning::gemv_wide_rows_per_group_long_k},

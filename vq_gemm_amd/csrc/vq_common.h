@@ -206,6 +206,7 @@ struct Tuning {
     double gemv_wide_plain_table_max_runs = 2.0;
     // the wide form's loop: rows of W per group (1 or 2) and groups of codes in flight (2 or 3), for K up to 4096
     // and beyond
+    double gemv_wide_single_rows_max = 2.0;  // up to this many rows per wave: groups of one row, two in flight
     double gemv_wide_rows_per_group = 2.0;
     double gemv_wide_groups_in_flight = 2.0;
     double gemv_wide_rows_per_group_long_k = 1.0;

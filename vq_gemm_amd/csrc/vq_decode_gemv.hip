@@ -596,14 +596,27 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 // Rows per group (1 or 2) and groups of codes in flight (2 or 3) of the wide form are runtime choices out of the
 // tuning table, separately for K up to 4096 and beyond: `python -m vq_gemm_amd.tune --search` times the four
 // combinations on the box at hand, on codes that come from HBM.
+// A wave with one or two rows (Tuning::gemv_wide_single_rows_max) takes them one by one with two groups in flight
+// whatever the table says: a group of two would request a row that is not there ahead of the one that is (cold, K = 4096,
+// groups of two -> groups of one: one row per wave 3.36 -> 3.13 us, two rows 4.00 -> 3.75; from three rows on the two
+// are level, from seven on groups of two are ahead).  Not for gated launches, where the group size says how a gate/up
+// pair is dealt.
+static bool wide_few_rows(const ProblemB &p)
+{
+    if (p.gated) return false;
+    const int waves = device_cu_count() * kWideWaves;
+    return (double)((p.N + waves - 1) / waves) <= tuning().gemv_wide_single_rows_max;
+}
 static int wide_rows_per_group(const ProblemB &p)
 {
     const Tuning &tn = tuning();
+    if (wide_few_rows(p)) return 1;
     return (p.K / kRunK > 2 ? tn.gemv_wide_rows_per_group_long_k : tn.gemv_wide_rows_per_group) >= 2.0 ? 2 : 1;
 }
 static int wide_groups_in_flight(const ProblemB &p)
 {
     const Tuning &tn = tuning();
+    if (wide_few_rows(p)) return 2;
     return (p.K / kRunK > 2 ? tn.gemv_wide_groups_in_flight_long_k : tn.gemv_wide_groups_in_flight) >= 3.0 ? 3 : 2;
 }
 

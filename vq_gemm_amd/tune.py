@@ -306,10 +306,11 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
         report[tag] = {f"g{c[0]}_nbuf{c[1]}": [round(t, 3) for t in ts] for c, ts in totals.items()}
         say(f"wide GEMV loop, {tag}: " + "; ".join(f"G={c[0]} NBUF={c[1]}: " + "/".join(f"{t:.2f}" for t in ts) for c, ts in totals.items())
             + f" us on {shapes} -> G={win[0]} NBUF={win[1]}")
+    # (a wave with one or two rows takes them one by one whatever these say: shapes of three rows per wave and more)
     loop_search("K<=4096", ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight"),
-                [(4096, waves, 1), (4096, 3 * waves, 3)] + ([] if quick else [(4096, 7 * waves, 1), (2048, 4 * waves, 1)]))
+                [(4096, 4 * waves, 1), (4096, 3 * waves, 3)] + ([] if quick else [(4096, 7 * waves, 1), (2048, 4 * waves, 1)]))
     loop_search("K>4096", ("gemv_wide_rows_per_group_long_k", "gemv_wide_groups_in_flight_long_k"),
-                [(8192, 2 * waves, 1)] + ([] if quick else [(8192, 7 * waves, 1), (6144, 4 * waves, 1), (14336, waves, 1)]))
+                [(8192, 3 * waves, 1)] + ([] if quick else [(8192, 7 * waves, 1), (6144, 4 * waves, 1), (14336, waves, 1)]))
     loop_now = {k: out[k] for k in ("gemv_wide_rows_per_group", "gemv_wide_groups_in_flight", "gemv_wide_rows_per_group_long_k",
                                     "gemv_wide_groups_in_flight_long_k")}
 
@@ -425,6 +426,25 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
         cost = {c: sum(tr if tiles >= c else tp for tiles, tp, tr in rows) for c in cands}
         out["decode_replicated_table_min_tiles"] = min(cost, key=cost.get)
         report["decode_table"] = [(t, round(a, 3), round(b, 3)) for t, a, b in rows]
+
+    # 6. the streaming kernel of the K-sliced path against the batched kernel's chunks of K: from which K on it is ahead,
+    #    for sixteen and for four rows of X (one tile per unit)
+    stream_on = dict(decode_stream_min_k=0.0, decode_stream_min_k_few_rows=0.0, decode_stream_min_m=0.0, decode_stream_max_m=16.0)
+    stream_off = dict(decode_stream_min_k=1e8, decode_stream_min_k_few_rows=1e8)
+    for rows_x, name in ((16, "decode_stream_min_k"), (4, "decode_stream_min_k_few_rows")):
+        first = None
+        ks = (8192, 14336) if quick else (8192, 12288, 14336, 16384)
+        for K in reversed(ks):
+            ts = _cold_us(rows_x, K, 16 * cus, DEC, device=device, **stream_on)
+            tb = _cold_us(rows_x, K, 16 * cus, DEC, device=device, **stream_off)
+            if ts is None or tb is None:
+                break
+            say(f"{rows_x} rows of X, K={K}, one tile per unit: streaming {ts:.2f} us, batched {tb:.2f} us")
+            report.setdefault("decode_stream", []).append((rows_x, K, round(ts, 3), round(tb, 3)))
+            if ts > tb * (1.0 - margin):
+                break
+            first = K
+        out[name] = float(first) if first else 1e8
 
     if verbose:
         print("constant                          current -> searched")
