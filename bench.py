@@ -41,7 +41,7 @@ from vq_gemm_amd.timing import MIN_TIMED_LAUNCHES, POOL_BYTES  # the cold-HBM pr
 # HBM bytes one cold decode launch moves: NOT measured by this program.  From rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE of `bench.py --probe C2`, scaled by a 256 MiB copy in the same run
 # (1104.1 KiB x 2.0 read + 8 KiB written); the summary and its command are in the file named here.
-PROFILED_C2_HBM_BYTES_PER_LAUNCH = 2_260_992
+PROFILED_C2_HBM_BYTES_PER_LAUNCH = 2_228_224
 PROFILED_C2_TRAFFIC_SOURCE = "profiles/decode_gemv_wide_kernel_c2_decode_gemv.md"
 # The same for the other configurations (name in `other_configs` -> bytes per launch, summary file): what the
 # per-configuration `roofline` objects carry as `traffic`.  None where no counter run exists.

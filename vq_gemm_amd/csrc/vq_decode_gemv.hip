@@ -313,6 +313,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     constexpr bool TWO = BOOKS == 2;
     constexpr bool LONG = XRUNS != RUNS;
     static_assert(!LONG || (BOOKS < 2 && COPIES == kWideCopies && NBUF == 2), "the long form: one table, replicated");
+    static_assert(NBUF > 1 || G == 1, "a single group per wave: of one row");
     const int gated = LONG ? 0 : (gated_row_bytes < 0 ? 1 : 0);
     constexpr int kXChunks = XRUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
@@ -423,6 +424,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         if constexpr (LONG) request_next(cw[u]);
         else load_group(0, min(u, max(n_groups, 1) - 1), cw[u]);
     }
+    // (NBUF == 1: no wave has more than one group - its codes are all the loads there are, and there is no loop)
+    if constexpr (NBUF == 1) load_group(0, 0, cw[0]);
 
     if (table_duty) {
         // Table: thread (e, h) writes copies 8h .. 8h+7 of entry e, in an order that sends the sixteen lanes
@@ -559,7 +562,9 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         default: __builtin_amdgcn_s_setprio(3); break;
         }
     };
-    if constexpr (LONG) {
+    if constexpr (NBUF == 1) {
+        multiply_group(0, cw[0]);
+    } else if constexpr (LONG) {
         int piece = 0, g = 0, turn = 0;
         while (piece < n_pieces) {
 #pragma unroll
@@ -751,6 +756,9 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
         }
         return hipErrorInvalidValue;
     };
+    // (a launch in which no wave has more than one row: no second group to request)
+    const bool single = !p.gated && tuning().gemv_wide_single_rows_max >= 1.0 && (n_dealt + waves - 1) / waves <= 1;
+    if (single) return pick_runs(integral_constant<int, 1>{}, integral_constant<int, 1>{});
     const int nbuf = (g == 2 && p.K / kRunK > 2) ? 2 : wide_groups_in_flight(p);
     if (g == 2) return nbuf == 3 ? pick_runs(integral_constant<int, 2>{}, integral_constant<int, 3>{})
                                  : pick_runs(integral_constant<int, 2>{}, integral_constant<int, 2>{});
