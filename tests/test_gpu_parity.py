@@ -350,6 +350,10 @@ GEMV_B = [
     ("wide_plain_table_books_straddled", 2048, 3 * 2000, 256, 3, 1),
     ("wide_plain_table_short_books", 4096, 4096, 77, 4, 1),
     ("wide_plain_table_ragged", 2048, 7001, 256, 1, 1),
+    # no wave with more than one row: the single-group instance (codebooks that workgroups straddle, waves without a row,
+    # the replicated table at three runs)
+    ("wide_single_group_three_books_straddled", 4096, 3 * 1008, 200, 3, 1),
+    ("wide_single_group_three_runs", 6144, 4096 - 7, 256, 1, 1),
     ("many_tiles_three_runs_ragged_walk", 6144, 16 * 1500, 256, 1, 1),
     ("many_tiles_one_run", 2048, 65536, 77, 1, 1),
     # the wide form's long rows (K beyond 8192, or no multiple of 2048), worked through in pieces of three or four runs:
