@@ -201,14 +201,15 @@ def test_batched_decode_kernel_with_many_tiles_per_workgroup(row, batched_kernel
     assert np.array_equal(_np(ywp).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
 
 
-# The streaming kernel of the K-sliced path (whole K per workgroup, K dealt to the waves in pieces of 128): one and two
+# The streaming kernel of the K-sliced path (whole K per workgroup, K dealt to the waves in pieces of 128): one to seven
 # tiles per group, ragged last groups, fewer groups than compute units and several per workgroup, codebooks that change
 # between a workgroup's groups, tall X in slabs, K of fewer pieces than a workgroup has waves, short codebooks.
 STREAM_B = [
     # name, M, K, N, E, G
     ("down_projection_m16", 16, 14336, 4096, 256, 1),
     ("down_projection_m4_k11008", 4, 11008, 4096, 256, 1),
-    ("three_groups_per_workgroup", 16, 8192, 24576, 256, 1),
+    ("six_tiles_per_group", 16, 8192, 24576, 256, 1),
+    ("seven_tiles_per_group", 12, 4096, 28672, 256, 1),
     ("three_tiles_ragged_last_group", 3, 4096, 11008, 256, 1),
     ("two_tiles_16_codebooks_slabs", 40, 8192, 8192, 256, 16),
     ("few_tiles_17_pieces", 1, 2176, 256, 256, 1),

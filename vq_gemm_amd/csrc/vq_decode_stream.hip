@@ -3,7 +3,7 @@
 // of its first codes).  8-vectors, 8-bit codes, up to 16 rows of X per workgroup (taller X: one 16-row slab per
 // index of the second grid dimension).
 //
-// One workgroup of sixteen waves per compute unit owns a group of one or two tiles of 16 rows of W over the whole of
+// One workgroup of sixteen waves per compute unit owns a group of one to seven tiles of 16 rows of W over the whole of
 // K.  K is cut into pieces of 128 k and the pieces are dealt to the waves in turn (wave w takes pieces w, w + 16, ...):
 // every wave streams its own pieces with no barrier and nothing shared inside the stream.
 //   * The codes of all of a wave's pieces (one dword per piece and tile, from HBM) are requested at once, behind the
@@ -35,7 +35,7 @@ constexpr int kPieceSteps = kPieceK / 32;
 constexpr int kTile = 16;                         // rows of W per tile
 constexpr int kReduceTiles = 4;                   // tiles summed per barrier
 constexpr int kCopies = 16;                       // replicated table: copies per entry (one 256-byte bank row)
-constexpr int kMaxTiles = 2;                      // tiles per group
+constexpr int kMaxTiles = 7;                      // tiles per group
 
 // T: tiles per group; NP: pieces per wave at most (the loop over a wave's pieces is unrolled NP times: code registers
 // and ring slots are then compile-time indices); REPL: the bank-replicated table (64 KB, conflict-free gathers) or the
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
         // has to cover the latency of the L2 at the rate the unit's L1 delivers: 16 waves x 2 pieces x 4 KB), one in
         // the block, one in operand registers
         // (with many code registers one piece less: its iterations are longer, and the registers are needed)
-        constexpr int kXRing = (NP * T >= 16 || NP > 8) ? 2 : 3;
+        constexpr int kXRing = (NP * T >= 16 || NP > 8 || T > 2) ? 2 : 3;
         uint4_t xs[kXRing][4];
         auto load_x = [&](int i, uint4_t (&xd)[4]) {
             const uint32_t piece_off = (uint32_t)(piece_of(i) * (kPieceK * 2));
@@ -173,10 +173,14 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
         __syncthreads();
 
         // ---- the stream ---------------------------------------------------------------------------
-        // (two accumulators per tile: a chain of dependent MFMAs is half as long)
-        float4_t acc[T][2];
+        // (two accumulators per tile while there are one or two tiles: a chain of dependent MFMAs is half as long; with
+        // more tiles the tiles' chains interleave)
+        constexpr int kAcc = T > 2 ? 1 : 2;
+        float4_t acc[T][kAcc];
 #pragma unroll
-        for (int t = 0; t < T; t++) acc[t][0] = acc[t][1] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < T; t++)
+#pragma unroll
+            for (int a = 0; a < kAcc; a++) acc[t][a] = float4_t{0.f, 0.f, 0.f, 0.f};
         auto multiply_piece = [&](const uint4_t (&xd)[kPieceSteps], const uint32_t (&cd)[T]) {
 #pragma unroll
             for (int t = 0; t < T; t++) {
@@ -191,7 +195,7 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
                 }
 #pragma unroll
                 for (int s = 0; s < kPieceSteps; s++)
-                    acc[t][s & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(wv[s]), as_half8(xd[s]), acc[t][s & 1], 0, 0, 0);
+                    acc[t][s % kAcc] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(wv[s]), as_half8(xd[s]), acc[t][s % kAcc], 0, 0, 0);
             }
         };
         // piece 0 into the block and out of it into operand registers; then per piece: the next piece into the block and
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(kStreamWaves * 64) void decode_stream_kernel(const 
         for (int r0 = 0; r0 < T; r0 += kRT) {
             if (r0 > 0) __syncthreads();  // the round before has been read
 #pragma unroll
-            for (int t = r0; t < r0 + kRT && t < T; t++) partial[((t - r0) * kStreamWaves + w) * 64 + lane] = acc[t][0] + acc[t][1];
+            for (int t = r0; t < r0 + kRT && t < T; t++) partial[((t - r0) * kStreamWaves + w) * 64 + lane] = kAcc == 2 ? acc[t][0] + acc[t][kAcc - 1] : acc[t][0];
             __syncthreads();
             // thread (t, l) of the first kRT * 64 sums lane l's entries of tile r0 + t in the order of the waves:
             // D[4 * (l / 16) + e][l % 16], rows of W by rows of X
@@ -282,10 +286,12 @@ bool decode_stream_supports(const ProblemB &p)
     return (p.M + kTile - 1) / kTile <= 65535;
 }
 
-// Where it was measured ahead of the batched kernel's chunks (cold, 256 units, batched -> this): 9 to 16 rows of X on
-// K from 8192 on, fewer rows from 14336 on (at K = 12288 two rows lose 4 to 12 %), with at most one group of tiles per unit.  M = 16: K = 14336 / N = 4096 17.3 -> 13.1 us, 28672 / 8192
-// 37.2 -> 28.3, 8192 / 8192 13.3 -> 11.8, 11008 / 4096 13.9 -> 12.4; M = 4: 13.0 -> 10.9, 25.6 -> 23.6, 9.9 -> 9.8,
-// 10.6 -> 10.6; M = 2: 12.5 -> 10.9, 24.8 -> 23.4, 9.7 -> 9.8, 10.2 -> 10.5.  More groups per unit (N = 28672) and
+// Where it was measured ahead of the batched kernel's chunks (cold, 256 units, batched -> this), always with at most
+// one group of tiles per unit.  9 to 16 rows of X from K = 8192 on, one to seven tiles per group: M = 16, K = 14336 /
+// N = 4096 17.3 -> 13.1 us, 28672 / 8192 37.2 -> 28.3, 16384 / 8192 22.8 -> 18.0, 8192 / 8192 13.3 -> 11.8, 8192 / 12288
+// 15.9 -> 13.7, 8192 / 28672 25.8 -> 23.9; M = 12: 1.02 to 1.24x on the same shapes.  Eight rows and fewer from
+// K = 14336 on with one or two tiles per group: M = 4, 14336 / 4096 13.0 -> 10.9, 14336 / 8192 15.7 -> 14.8, 28672 /
+// 8192 25.6 -> 23.6 (three tiles per group: 0.97 - 0.99x; K = 8192 and 12288: 0.84 - 1.0x).  More groups per unit and
 // taller X (one workgroup per 16-row slab, the codes read again by each) stay with the batched kernel: 0.5 - 0.9x.
 bool decode_stream_preferred(const ProblemB &p)
 {
@@ -293,6 +299,7 @@ bool decode_stream_preferred(const ProblemB &p)
     if (!decode_stream_supports(p) || (double)p.K < (p.M <= 8 ? tn.decode_stream_min_k_few_rows : tn.decode_stream_min_k)) return false;
     if ((double)p.M < tn.decode_stream_min_m || (double)p.M > tn.decode_stream_max_m) return false;
     const int t = stream_tiles_per_group(p);
+    if (p.M <= 8 && t > 2) return false;  // (few rows of X on three tiles and more per group: 1 to 15 % behind)
     const int n_groups = (p.N / kTile + t - 1) / t;
     return (double)n_groups <= tn.decode_stream_max_groups_per_unit * device_cu_count();
 }
@@ -318,13 +325,27 @@ hipError_t launch_decode_stream(const ProblemB &p, hipStream_t s)
         constexpr int TT = decltype(t_c)::value, NPP = decltype(np_c)::value;
         return repl ? launch(decode_stream_kernel<TT, NPP, true>) : launch(decode_stream_kernel<TT, NPP, false>);
     };
-    // (pieces per wave in steps of 4, 8 and 14; one or two tiles per group)
-    auto pick_np = [&](auto t_c) {
-        if (pieces <= 4) return pick(t_c, integral_constant<int, 4>{});
-        if (pieces <= 8) return pick(t_c, integral_constant<int, 8>{});
-        return pick(t_c, integral_constant<int, 14>{});
-    };
-    return t == 1 ? pick_np(integral_constant<int, 1>{}) : pick_np(integral_constant<int, 2>{});
+    // (pieces per wave in steps of 4, 8 and 14; tiles per group within what the code registers hold)
+    if (pieces <= 4) {
+        switch (t) {
+        case 1: return pick(integral_constant<int, 1>{}, integral_constant<int, 4>{});
+        case 2: return pick(integral_constant<int, 2>{}, integral_constant<int, 4>{});
+        case 3: return pick(integral_constant<int, 3>{}, integral_constant<int, 4>{});
+        case 4: return pick(integral_constant<int, 4>{}, integral_constant<int, 4>{});
+        case 5: return pick(integral_constant<int, 5>{}, integral_constant<int, 4>{});
+        case 6: return pick(integral_constant<int, 6>{}, integral_constant<int, 4>{});
+        default: return pick(integral_constant<int, 7>{}, integral_constant<int, 4>{});
+        }
+    }
+    if (pieces <= 8) {
+        switch (t) {
+        case 1: return pick(integral_constant<int, 1>{}, integral_constant<int, 8>{});
+        case 2: return pick(integral_constant<int, 2>{}, integral_constant<int, 8>{});
+        default: return pick(integral_constant<int, 3>{}, integral_constant<int, 8>{});
+        }
+    }
+    return t == 1 ? pick(integral_constant<int, 1>{}, integral_constant<int, 14>{})
+                  : pick(integral_constant<int, 2>{}, integral_constant<int, 14>{});
 }
 
 }  // namespace vq
