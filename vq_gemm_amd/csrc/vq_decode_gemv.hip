@@ -578,6 +578,30 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
                 }
             }
         }
+    } else if constexpr (NBUF == 2) {
+        // Two groups in flight: the loop runs while both of its requests are for groups that exist, and the last one or
+        // two groups are multiplied behind it in straight-line code, so that no group is requested twice (a wave's
+        // last request would otherwise be its last group again, and the wave ends only when that load has landed).
+        // Inside either branch of the tail the order of loads and uses is fixed: the wait counts stay exact.
+        int g = 0;
+        for (; g + 2 < n_groups; g += 2) {
+            load_group(0, g + 1, cw[1]);
+            if (rotate_priority) set_priority(age - g);
+            multiply_group(g, cw[0]);
+            load_group(0, g + 2, cw[0]);
+            if (rotate_priority) set_priority(age - (g + 1));
+            multiply_group(g + 1, cw[1]);
+        }
+        if (n_groups - g == 2) {
+            load_group(0, g + 1, cw[1]);
+            if (rotate_priority) set_priority(age - g);
+            multiply_group(g, cw[0]);
+            if (rotate_priority) set_priority(age - (g + 1));
+            multiply_group(g + 1, cw[1]);
+        } else {
+            if (rotate_priority) set_priority(age - g);
+            multiply_group(g, cw[0]);
+        }
     } else {
         for (int g = 0; g < n_groups; g += NBUF) {
 #pragma unroll
