@@ -399,6 +399,17 @@ def test_gemv_kernel_few_rows_of_x(row):
     assert e1 <= TOL
     for _ in range(4):
         assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), y)
+    # one row of X goes to the wide form at any N; the four-wave kernel takes the same launch when the wide form is
+    # switched off: same product within the bar, a column of W bit for bit
+    if M == 1 and K % 2048 == 0 and K <= 8192 and N % 16 == 0 and N <= 4096:
+        before = cabi.tuning()["gemv_wide_min_rows_per_wave"]
+        cabi.set_tuning(gemv_wide_min_rows_per_wave=1e6)
+        try:
+            _check_gemm(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), x, codes, cb, what=name + " (four-wave)")
+            yw = cabi.e2e_gemm_b(eye, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+            assert np.array_equal(_np(yw).view(np.uint16), w[:, cols].T.copy().view(np.uint16))
+        finally:
+            cabi.set_tuning(gemv_wide_min_rows_per_wave=before)
     # the K-sliced MFMA kernel and the automatic choice on the same inputs: same product within the bar
     if K % 64 == 0:   # (the K-sliced kernels take K in whole matrix-core steps)
         _check_gemm(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE), x, codes, cb, what=name + " (decode)")
@@ -468,7 +479,7 @@ def test_gemv_kernel_code_formats(row):
 
 def test_gemv_kernel_refuses_other_shapes():
     cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
-    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 10240, 64, 8, 8), (1, 2048, 24, 8, 8),
+    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 2056, 64, 8, 8), (1, 34816, 64, 8, 8), (2, 2048, 24, 8, 8),
                                (1, 2048, 64, 2, 16), (3, 2048, 64, 4, 8)]:
         x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
         codes = torch.zeros(N, K // v, dtype=torch.uint8 if bits == 8 else torch.uint16, device=DEV)
@@ -476,6 +487,19 @@ def test_gemv_kernel_refuses_other_shapes():
         with pytest.raises(cabi.VqGemmError) as ei:
             cabi.e2e_gemm_b(x, codes, c, variant=cabi.VARIANT_DECODE_GEMV)
         assert ei.value.code == -4
+
+
+def test_gemv_kernel_one_row_of_x_small_launches_in_the_long_form():
+    """One row of X with a K or an N that the four-wave kernel does not take goes to the wide form at any size: K no whole
+    number of runs, K beyond 8192, N no multiple of 16, on launches far smaller than the device."""
+    for (K, N, E, G) in [(2080, 64, 256, 1), (10240, 64, 256, 1), (2048, 24, 100, 1), (6144, 8, 256, 1), (4096, 40, 256, 2)]:
+        spec = ProblemSpec(f"small_k{K}_n{N}", GEOM_B, 1, K, N, 8, E, G, 8, codebook_3d=(G > 1))
+        x, codes, cb = make_problem(spec, seed=77, device=DEV)
+        _say("gemv small", spec)
+        y = cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV)
+        torch.cuda.synchronize()
+        _check_gemm(y, x, codes, cb, what=spec.name)
+        _check_gemm(cabi.e2e_gemm_b(x, codes, cb), x, codes, cb, what=spec.name + " (auto)")
 
 
 # Shapes that walk the prefill kernel through each of its instantiations: both super-stage

@@ -200,7 +200,7 @@ struct Tuning {
     // many rows per wave on
     double gemv_max_tiles_per_cu = 4.0;
     double gemv_max_k = 8192.0;
-    double gemv_wide_min_rows_per_wave = 0.5;
+    double gemv_wide_min_rows_per_wave = 0.0;
     // the wide form gathers from the plain 4 KB table while a wave's rows are at most this many runs of 2048 k, from the
     // bank-replicated one (64 KB to fill) beyond
     double gemv_wide_plain_table_max_runs = 2.0;

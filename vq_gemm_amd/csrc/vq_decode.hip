@@ -896,7 +896,7 @@ double decode_cost_us(const ProblemB &p)
 
 // The GEMV kernels have no work shared between their waves.  One row of X in the first format
 // (8-vectors, 8-bit codes, at most two codebooks per workgroup's share of the rows) goes to the wide
-// form from half a row per wave on (2048 rows on a 256-CU device; Tuning::gemv_wide_min_rows_per_wave): measured against the batched kernel
+// form at any N (Tuning::gemv_wide_min_rows_per_wave rows per wave, 0 by default): measured against the batched kernel
 // on a 256-CU MI355X, cold HBM, K = 4096: N = 4096 4.96 -> 3.4 us, N = 16384 7.5 -> 5.1, N = 28672
 // 9.9 -> 7.1, N = 65536 15.6 -> 12.4; K = 8192: N = 8192 8.3 -> 5.6, N = 28672 18.3 -> 10.8.
 // The four-wave kernel takes what is left where it was measured faster than the batched kernel

@@ -366,7 +366,7 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
 
     # 3. wide form against the four-wave form: from how many rows per wave on the wide form wins
     limit = None
-    fracs = (0.25, 0.5, 0.75, 1.0)
+    fracs = (0.0625, 0.125, 0.25, 0.5, 0.75, 1.0)
     wins = []
     for f in fracs:
         N = int(waves * f) // 16 * 16
@@ -381,6 +381,8 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
         if not won:
             break
         limit = f
+    if wins and all(won for _, won in wins):
+        limit = 0.0   # ahead down to the smallest launch tried: every launch the wide form supports
     if limit is not None:
         out["gemv_wide_min_rows_per_wave"] = limit
     report["wide_vs_four_wave"] = wins
