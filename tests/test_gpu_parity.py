@@ -322,6 +322,9 @@ def test_packed_codes_small_shapes_bias_and_rejections():
     assert cabi.select_variant_b(16, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.select_variant_b(2, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(3, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
+    assert cabi.select_variant_b(2, 4096, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV   # two rows of X: the wide form ...
+    assert cabi.select_variant_b(2, 4096, 65536, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... up to eleven rows per wave at K = 4096
+    assert cabi.select_variant_b(2, 8192, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... and K up to 4096
     assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(1, 4096, 131072, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 2, 8) == cabi.VARIANT_DECODE_GEMV
@@ -368,6 +371,13 @@ GEMV_B = [
     ("long_k_10240_three_rows_per_wave_ragged", 10240, 9001, 256, 1, 1),
     ("long_k_12288_two_books", 12288, 8192, 256, 2, 1),
     ("two_rows_of_x", 4096, 4096, 256, 1, 2),
+    # two rows of X in the wide form (K up to 4096): ragged N, codebooks that workgroups straddle, the single-group
+    # instance with waves without a row, seven rows per wave in groups of two, one run
+    ("wide_two_rows_of_x_ragged", 4096, 5003, 256, 1, 2),
+    ("wide_two_rows_three_books_straddled", 2048, 12288, 256, 3, 2),
+    ("wide_two_rows_single_group", 4096, 4096 - 7, 200, 1, 2),
+    ("wide_two_rows_many_tiles", 4096, 28672, 256, 1, 2),
+    ("wide_two_rows_one_run_two_books", 2048, 2 * 9008, 77, 2, 2),
     ("two_rows_four_runs", 8192, 512, 256, 2, 2),
     ("three_rows", 2048, 1024, 256, 1, 3),
     ("four_rows_two_runs", 4096, 1024, 200, 4, 4),
@@ -399,9 +409,9 @@ def test_gemv_kernel_few_rows_of_x(row):
     assert e1 <= TOL
     for _ in range(4):
         assert torch.equal(cabi.e2e_gemm_b(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV), y)
-    # one row of X goes to the wide form at any N; the four-wave kernel takes the same launch when the wide form is
+    # one or two rows of X go to the wide form at any N; the four-wave kernel takes the same launch when the wide form is
     # switched off: same product within the bar, a column of W bit for bit
-    if M == 1 and K % 2048 == 0 and K <= 8192 and N % 16 == 0 and N <= 4096:
+    if M <= 2 and K % 2048 == 0 and K <= 8192 and N % 16 == 0 and N <= 4096:
         before = cabi.tuning()["gemv_wide_min_rows_per_wave"]
         cabi.set_tuning(gemv_wide_min_rows_per_wave=1e6)
         try:
@@ -479,7 +489,7 @@ def test_gemv_kernel_code_formats(row):
 
 def test_gemv_kernel_refuses_other_shapes():
     cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
-    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 2056, 64, 8, 8), (1, 34816, 64, 8, 8), (2, 2048, 24, 8, 8),
+    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 2056, 64, 8, 8), (1, 34816, 64, 8, 8), (3, 2048, 24, 8, 8), (2, 8192, 24, 8, 8),
                                (1, 2048, 64, 2, 16), (3, 2048, 64, 4, 8)]:
         x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
         codes = torch.zeros(N, K // v, dtype=torch.uint8 if bits == 8 else torch.uint16, device=DEV)
@@ -1045,6 +1055,7 @@ def test_tune_search_tries_the_kernel_parameter_candidates_cold_and_the_library_
     assert found["gemv_wide_rows_per_group"] in (1.0, 2.0) and found["gemv_wide_groups_in_flight"] in (2.0, 3.0)
     assert found["gemv_wide_rows_per_group_long_k"] in (1.0, 2.0) and found["gemv_wide_groups_in_flight_long_k"] in (2.0, 3.0)
     assert found["decode_stream_min_k"] in (8192.0, 14336.0, 1e8) and found["decode_stream_min_k_few_rows"] in (8192.0, 14336.0, 1e8)
+    assert found["gemv_wide_two_rows_max_runs"] in (before["gemv_wide_two_rows_max_runs"], 16.0, 22.0, 28.0)
     assert cabi.tuning() == before, "the search leaves the table as it found it"
     # every candidate of the wide form's loop gives the same bits as the default (same sums in the same order per row)
     spec = ProblemSpec("cand", GEOM_B, 1, 4096, 12288, 8, 256, 3, 8, codebook_3d=True)
@@ -1464,6 +1475,8 @@ GATED_B = [
     ("gemv_wide_many_books", 1, 4096, 16384, 8, 256, 8, 16),
     ("gemv_wide_k8192", 1, 8192, 16384, 8, 256, 8, 1),           # gate row and up row as two groups of one row in turn
     ("gemv_wide_k6144_books", 1, 6144, 3 * 2752, 8, 256, 8, 3),
+    ("gemv_wide_two_rows_of_x", 2, 4096, 8192, 8, 256, 8, 1),     # two rows of X: two outputs per pair of code rows
+    ("gemv_wide_two_rows_of_x_k2048_books", 2, 2048, 8192 + 64, 8, 200, 8, 2),
     ("decode_shape", 16, 1024, 2048, 4, 4096, 16, 1),           # batched K-sliced kernel: gate and up tiles summed in pairs
     ("decode_shape_m2", 2, 4096, 4096, 8, 256, 8, 1),
     ("decode_books_ragged_units", 16, 4096, 4 * 1056, 8, 256, 8, 4),   # 33 pairs per codebook: short last batches
@@ -1477,7 +1490,7 @@ GATED_B = [
     ("gemv4_c3_weights_m2", 2, 4096, 1376, 4, 4096, 16, 1),
     ("gemv4_v4_u8_m1", 1, 2048, 2048, 4, 256, 8, 4),
     ("gemv4_v4_u8_m2", 2, 4096, 1024, 4, 256, 8, 1),
-    ("gemv4_v8_u8_few_rows_m2", 2, 4096, 2048, 8, 256, 8, 2),    # fewer rows than the wide form takes
+    ("gemv4_v8_u8_few_rows_m2", 2, 4096, 2048, 8, 256, 8, 2),    # a quarter of a row per wave
     ("gemv4_v2_u8_m1", 1, 2048, 512, 2, 256, 8, 1),
     ("odd_k_scalar_only", 5, 72, 64, 8, 256, 8, 1),
 ]

@@ -67,6 +67,8 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_max_tiles_per_cu", &Tuning::gemv_max_tiles_per_cu},
     {"gemv_max_k", &Tuning::gemv_max_k},
     {"gemv_wide_min_rows_per_wave", &Tuning::gemv_wide_min_rows_per_wave},
+    {"gemv_wide_max_m", &Tuning::gemv_wide_max_m},
+    {"gemv_wide_two_rows_max_runs", &Tuning::gemv_wide_two_rows_max_runs},
     {"gemv_wide_plain_table_max_runs", &Tuning::gemv_wide_plain_table_max_runs},
     {"gemv_wide_single_rows_max", &Tuning::gemv_wide_single_rows_max},
     {"gemv_wide_rows_per_group", &Tuning::gemv_wide_rows_per_group},

@@ -20,7 +20,8 @@
 // serves two to four rows of X and the other code formats; one row of X in the first format goes to
 // the wide form below (decode_gemv_wide_kernel) at any N (Tuning::gemv_wide_min_rows_per_wave = 0:
 // with its single-group instance the wide form is ahead from N = 256 on, cold, K = 4096: 2.55
-// against 2.76 us; N = 2048: 2.71 against 2.98; K = 8192, N = 1024: 3.29 against 3.93).
+// against 2.76 us; N = 2048: 2.71 against 2.98; K = 8192, N = 1024: 3.29 against 3.93), and so do
+// two rows of X with K up to 4096 while a wave has few enough rows.
 #include "vq_common.h"
 
 #include <limits.h>
@@ -284,6 +285,10 @@ __device__ __forceinline__ int small_quotient(int x, int d, float rcp)
 // COPIES: 16 = the bank-replicated table (conflict-free gathers; 64 KB to fill), 1 = the plain 4 KB table (a wave
 // with one or two rows gathers too little for the fill of the replicated table to pay).
 //
+// XM: rows of X (1 or 2).  With two, a lane keeps its shares of both rows in registers (RUNS <= 2), every gathered
+// codeword is multiplied with both, and a wave folds and keeps two sums per row of W (cold, M = 2, K = 4096, the
+// K-sliced matrix-core kernel -> this: N = 11008 7.2 -> 5.3 us, N = 28672 10.5 -> 8.7).
+//
 // XRUNS: runs of 2048 k of x that the LDS holds.  XRUNS == RUNS is the form described so far (K = RUNS * 2048, all of a
 // lane's x in registers).  XRUNS > RUNS is the form for a longer K, or one that is no multiple of 2048 (the
 // down-projection of an MLP: K = 11008, 14336, 28672): a row is cut into pieces of RUNS runs, a wave goes through
@@ -291,7 +296,7 @@ __device__ __forceinline__ int small_quotient(int x, int d, float rcp)
 // and a row's sum so far travels in its lane of `res`: the accumulator of lane 0 starts from it.  x is padded with
 // zeros up to whole pieces, and a load that would reach past the end of a row reads the row's last dword instead: what
 // it gathers meets zeros.  One codebook, or several without a workgroup whose rows reach into two; not gated.
-template <int RUNS, int G, int NBUF, int BOOKS, int COPIES, int XRUNS = RUNS>
+template <int RUNS, int G, int NBUF, int BOOKS, int COPIES, int XRUNS = RUNS, int XM = 1>
 __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const half_t *__restrict__ x,
                                                                            const uint8_t *__restrict__ codes,
                                                                            const half_t *__restrict__ cb, int entries,
@@ -315,13 +320,14 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     constexpr bool LONG = XRUNS != RUNS;
     static_assert(!LONG || (BOOKS < 2 && COPIES == kWideCopies && NBUF == 2), "the long form: one table, replicated");
     static_assert(NBUF > 1 || G == 1, "a single group per wave: of one row");
+    static_assert(XM == 1 || (XM == 2 && !LONG && RUNS <= 2), "two rows of X: both in the lane's registers, K up to 4096");
     const int gated = LONG ? 0 : (gated_row_bytes < 0 ? 1 : 0);
     constexpr int kXChunks = XRUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
     // permute) | table of the second one (TWO) | x
     static_assert(COPIES == kWideCopies || COPIES == 1, "replicated or plain table");
     constexpr int kTableSlots = (TWO ? 2 : 1) * 256 * COPIES;
-    __shared__ __align__(16) uint4_t lds[kTableSlots + kXChunks];
+    __shared__ __align__(16) uint4_t lds[kTableSlots + XM * kXChunks];
     uint4_t *table = lds, *xs = lds + kTableSlots;
     const int tid = threadIdx.x;
     // codes (bytes) per row, and the pieces a row is worked through in
@@ -349,7 +355,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         second_table = TWO && second_book_row <= wg_row_last;
     }
     constexpr int kDutyThreads = kWideWaves * 64 / 2;
-    constexpr int kXPerThread = (kXChunks + kDutyThreads - 1) / kDutyThreads;
+    constexpr int kXPerThread = (XM * kXChunks + kDutyThreads - 1) / kDutyThreads;   // (the rows of X lie one behind the other)
     const bool table_duty = tid < kDutyThreads;
     const int e = tid >> 1, half_of_copies = tid & 1;   // table duty: entry and which eight of its sixteen copies
     const int xt = tid - kDutyThreads;                  // x duty: pieces xt, xt + 512
@@ -363,7 +369,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     } else {
 #pragma unroll
         for (int i = 0; i < kXPerThread; i++)
-            xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, (LONG ? J : kXChunks) - 1)];
+            xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, (LONG ? J : XM * kXChunks) - 1)];
     }
 
     // the wave's share [row0, row0 + n_share) of the rows (gated: of the outputs) and its code rows: at most 64, one
@@ -453,17 +459,19 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
             const int xi = xt + i * kDutyThreads;
             // (the long form: zeros behind the end of x, up to whole pieces of rows)
             if (LONG && xi >= J) xpiece[i] = uint4_t{0u, 0u, 0u, 0u};
-            if (xi < kXChunks) xs[(xi & ~255) + (xi & 3) * 64 + ((xi >> 2) & 63)] = xpiece[i];
+            if (xi < XM * kXChunks) xs[(xi & ~255) + (xi & 3) * 64 + ((xi >> 2) & 63)] = xpiece[i];
         }
     }
     __syncthreads();
     if (n_rows <= 0) return;
-    uint4_t xr[RUNS][4];
+    uint4_t xr[XM][RUNS][4];
     auto load_x_piece = [&](int piece) {
 #pragma unroll
-        for (int q = 0; q < RUNS; q++)
+        for (int m = 0; m < XM; m++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) xr[q][c] = xs[(piece * RUNS + q) * kRunCodes + c * 64 + lane];
+            for (int q = 0; q < RUNS; q++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) xr[m][q][c] = xs[m * kXChunks + (piece * RUNS + q) * kRunCodes + c * 64 + lane];
     };
     load_x_piece(0);
 
@@ -471,19 +479,22 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     // lane's dword of codes (byte 1) and a per-row base (bytes 0 and 2).
     const uint32_t copy_base = (lane & (kWideCopies - 1)) * 16u;
     const uint8_t *tbl = reinterpret_cast<const uint8_t *>(table);
-    float res = 0.f;  // lane i: the sum of the wave's row i
-    float gate_sum = 0.f;  // gated, G = 1: the gate row's sum (wave-uniform) until the up row's group has run
+    float res[XM];       // lane i: the sum of the wave's row i (for each row of X)
+    float gate_sum[XM];  // gated, G = 1: the gate row's sum (wave-uniform) until the up row's group has run
+#pragma unroll
+    for (int m = 0; m < XM; m++) res[m] = gate_sum[m] = 0.f;
     // rows [g*G, g*G + R) of the wave, R <= G (a compile-time count: the last group may be short)
     auto multiply_rows = [&](int g, const uint32_t (&cur)[G][RUNS], auto r_const) {
         constexpr int R = decltype(r_const)::value;
-        float acc[R];
+        float acc[XM][R];
         uint32_t base[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            acc[r] = 0.f;
+#pragma unroll
+            for (int m = 0; m < XM; m++) acc[m][r] = 0.f;
             // (the long form: the row's sum over the pieces before this one, zero at the first)
             if constexpr (LONG)
-                acc[r] = lane == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, res), g * G + r)) : 0.f;
+                acc[0][r] = lane == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, res[0]), g * G + r)) : 0.f;
             if constexpr (COPIES == 1) base[r] = TWO && code_row(g * G + r) >= second_book_row ? 4096u : 0u;
             else base[r] = TWO ? copy_base | (code_row(g * G + r) >= second_book_row ? 0x10000u : 0u) : copy_base;
         }
@@ -506,38 +517,48 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
                 for (int r = 0; r < R; r++)
 #pragma unroll
-                    for (int d = 0; d < 4; d++) {
-                        const uint32_t wd = w[r][c][d], xd = xr[q][c][d];
-                        acc[r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[r], false);
-                    }
+                    for (int d = 0; d < 4; d++)
+#pragma unroll
+                        for (int m = 0; m < XM; m++) {
+                            const uint32_t wd = w[r][c][d], xd = xr[m][q][c][d];
+                            acc[m][r] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, wd), __builtin_bit_cast(half2_t, xd), acc[m][r], false);
+                        }
         }
         if (G == 2 && R == 2 && gated) {
             // one output: gate and up sums, the bias of the output's lane, silu(gate) * up
-            const float sg = wave_sum_to_uniform(acc[0]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), g));
-            const float su = wave_sum_to_uniform(acc[R - 1]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), g));
-            res = (int)lane == g ? silu_f32(sg) * su : res;
+#pragma unroll
+            for (int m = 0; m < XM; m++) {
+                const float sg = wave_sum_to_uniform(acc[m][0]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), g));
+                const float su = wave_sum_to_uniform(acc[m][R - 1]) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), g));
+                res[m] = (int)lane == g ? silu_f32(sg) * su : res[m];
+            }
             return;
         }
         if (G == 1 && gated) {
             // even groups are gate rows, odd groups the up rows of the same output
             const int o = g >> 1;
-            const float s = wave_sum_to_uniform(acc[0]);
-            if ((g & 1) == 0) {
-                gate_sum = s + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), o));
-            } else {
-                const float su = s + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), o));
-                res = (int)lane == o ? silu_f32(gate_sum) * su : res;
+#pragma unroll
+            for (int m = 0; m < XM; m++) {
+                const float s = wave_sum_to_uniform(acc[m][0]);
+                if ((g & 1) == 0) {
+                    gate_sum[m] = s + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_gate), o));
+                } else {
+                    const float su = s + __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_up), o));
+                    res[m] = (int)lane == o ? silu_f32(gate_sum[m]) * su : res[m];
+                }
             }
             return;
         }
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            // (the row's sum goes from the scalar register straight into lane g*G + r: one v_writelane instead of a
-            // move, a compare and a select)
-            const float s = wave_sum_to_uniform(acc[r]);
-            // (on this target the instruction takes one scalar register: the lane number goes through m0)
-            asm("s_mov_b32 m0, %2\n\tv_writelane_b32 %0, %1, m0" : "+v"(res) : "s"(s), "s"(g * G + r) : "m0");
-        }
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int m = 0; m < XM; m++) {
+                // (the row's sum goes from the scalar register straight into lane g*G + r: one v_writelane instead of a
+                // move, a compare and a select)
+                const float s = wave_sum_to_uniform(acc[m][r]);
+                // (on this target the instruction takes one scalar register: the lane number goes through m0)
+                asm("s_mov_b32 m0, %2\n\tv_writelane_b32 %0, %1, m0" : "+v"(res[m]) : "s"(s), "s"(g * G + r) : "m0");
+            }
     };
     auto multiply_group = [&](int g, const uint32_t (&cur)[G][RUNS]) {
         const int left = n_rows - g * G;  // wave-uniform
@@ -615,9 +636,9 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         }
     }
     if ((int)lane < n_share) {
-        float s = res;
-        if (bias && !gated) s += (float)bias[row0 + lane];
-        y[row0 + lane] = (half_t)s;
+        const float b = bias && !gated ? (float)bias[row0 + lane] : 0.f;
+#pragma unroll
+        for (int m = 0; m < XM; m++) y[(int64_t)m * n_total + row0 + lane] = (half_t)(res[m] + b);   // (a row of y: what was dealt out)
     }
 }
 
@@ -697,8 +718,10 @@ static bool wide_straddles(const ProblemB &p, int workgroups)
 // more than two codebooks.
 bool decode_gemv_wide_supports(const ProblemB &p)
 {
-    if (p.M != 1 || p.vec != 8 || p.code_bits != 8 || p.entries > 256 || p.packed) return false;
+    if (p.M < 1 || p.M > 2 || p.vec != 8 || p.code_bits != 8 || p.entries > 256 || p.packed) return false;
     if (p.K < kRunK || p.N < 1) return false;
+    // two rows of X: both in the lane's registers, K = 2048 or 4096
+    if (p.M == 2 && (long_k_form(p).is_long || p.K / kRunK > 2)) return false;
     if (long_k_form(p).is_long) {
         if (p.K % 32 != 0 || p.K > 16 * kRunK || p.gated) return false;
         const int workgroups = wide_workgroups(p);
@@ -739,6 +762,21 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
     };
     using std::integral_constant;
     const int g = wide_rows_per_group(p);
+    if (p.M == 2) {
+        // two rows of X against every gathered codeword: the replicated table, one or two groups
+        auto pick2 = [&](auto runs_c, auto g_c, auto nbuf_c) {
+            constexpr int R = decltype(runs_c)::value, GG = decltype(g_c)::value, NB = decltype(nbuf_c)::value;
+            return books == 0 ? launch(decode_gemv_wide_kernel<R, GG, NB, 0, kWideCopies, R, 2>)
+                 : books == 1 ? launch(decode_gemv_wide_kernel<R, GG, NB, 1, kWideCopies, R, 2>)
+                              : launch(decode_gemv_wide_kernel<R, GG, NB, 2, kWideCopies, R, 2>);
+        };
+        auto pick2_runs = [&](auto g_c, auto nbuf_c) {
+            return p.K / kRunK == 1 ? pick2(integral_constant<int, 1>{}, g_c, nbuf_c) : pick2(integral_constant<int, 2>{}, g_c, nbuf_c);
+        };
+        if (!p.gated && (n_dealt + waves - 1) / waves <= 1) return pick2_runs(integral_constant<int, 1>{}, integral_constant<int, 1>{});
+        return g == 2 ? pick2_runs(integral_constant<int, 2>{}, integral_constant<int, 2>{})
+                      : pick2_runs(integral_constant<int, 1>{}, integral_constant<int, 2>{});
+    }
     if (const LongK f = long_k_form(p); f.is_long) {
         // (the replicated table, one table per workgroup, two groups in flight: three were measured and are slower,
         // K = 11008 to 28672, N = 4096 to 16384: +3 to +6 %, one shape -3 %)
@@ -819,7 +857,15 @@ bool decode_gemv_supports(const ProblemB &p) { return decode_gemv_wide_preferred
 
 bool decode_gemv_wide_preferred(const ProblemB &p)
 {
-    return decode_gemv_wide_supports(p) &&
+    // two rows of X: while a wave's rows are at most Tuning::gemv_wide_two_rows_max_runs runs of 2048 k (measured cold
+    // against the K-sliced kernel, K = 4096: 8 rows per wave 9.8 against 11.2 us, 11 rows 12.6 against 13.1, 12 rows 13.8
+    // against 13.7, 14 rows 16.5 against 14.9; K = 2048: 14 rows 10.3 against 11.1)
+    if (p.M == 2) {
+        const int waves = device_cu_count() * kWideWaves;
+        const double runs = (double)(((p.gated ? p.N / 2 : p.N) + waves - 1) / waves) * (p.gated ? 2 : 1) * (double)(p.K / kRunK);
+        if (runs > tuning().gemv_wide_two_rows_max_runs) return false;
+    }
+    return decode_gemv_wide_supports(p) && (double)p.M <= tuning().gemv_wide_max_m &&
            (double)(p.gated ? p.N / 2 : p.N) >= tuning().gemv_wide_min_rows_per_wave * kWideWaves * device_cu_count();
 }
 

@@ -387,6 +387,23 @@ def search(device: str = "cuda:0", verbose: bool = True, quick: bool = False, ma
         out["gemv_wide_min_rows_per_wave"] = limit
     report["wide_vs_four_wave"] = wins
 
+    # 3b. two rows of X: the wide form against the K-sliced kernel, by the runs of 2048 k a wave's rows make (K = 4096)
+    best_runs = None
+    for rows in ((8, 11, 14) if quick else (6, 8, 10, 11, 12, 14)):
+        N = rows * waves
+        tw = _cold_us(2, 4096, N, GEMV, device=device, gemv_wide_two_rows_max_runs=1e6, gemv_wide_max_m=2.0)
+        td = _cold_us(2, 4096, N, DEC, device=device)
+        if tw is None or td is None:
+            continue
+        say(f"two rows of X, K=4096, {rows} rows per wave: wide {tw:.2f} us, K-sliced {td:.2f} us")
+        if tw <= td:
+            best_runs = 2.0 * rows
+        else:
+            break
+    if best_runs is not None:
+        out["gemv_wide_two_rows_max_runs"] = best_runs
+    report["wide_two_rows"] = best_runs
+
     # 4. four-wave GEMV against the batched K-sliced kernel in a format the wide form does not take: tiles per unit, K
     best_tiles = 0.0
     for tiles in (1, 2, 4, 8) if not quick else (1, 2):
