@@ -418,6 +418,10 @@ def main():
         others["decode_qkv_m1_k4096_n12288"], _ = bench_config(
             ProblemSpec("decode_qkv_m1_k4096_n12288", GEOM_B, 1, 4096, 12288, 8, 256, 3, 8),
             max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
+        # two tokens through the same up-projection: the wide GEMV form with two rows of X
+        others["decode_m2_k4096_n28672"], _ = bench_config(
+            ProblemSpec("decode_m2_k4096_n28672", GEOM_B, 2, 4096, 28672, 8, 256, 1, 8),
+            max(200, args.steps // 5), max(20, args.warmup // 5), cold_pool=True)
         # the down-projection behind such an MLP (K beyond what a lane's registers hold of x: rows worked through in pieces)
         others["decode_down_m1_k14336_n4096"], _ = bench_config(
             ProblemSpec("decode_down_m1_k14336_n4096", GEOM_B, 1, 14336, 4096, 8, 256, 1, 8),
