@@ -324,7 +324,9 @@ def test_packed_codes_small_shapes_bias_and_rejections():
     assert cabi.select_variant_b(3, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.select_variant_b(2, 4096, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV   # two rows of X: the wide form ...
     assert cabi.select_variant_b(2, 4096, 65536, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... up to eleven rows per wave at K = 4096
-    assert cabi.select_variant_b(2, 8192, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... and K up to 4096
+    assert cabi.select_variant_b(2, 8192, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... five at K = 8192
+    assert cabi.select_variant_b(2, 8192, 8192, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
+    assert cabi.select_variant_b(2, 14336, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(1, 4096, 131072, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 2, 8) == cabi.VARIANT_DECODE_GEMV
@@ -378,6 +380,12 @@ GEMV_B = [
     ("wide_two_rows_single_group", 4096, 4096 - 7, 200, 1, 2),
     ("wide_two_rows_many_tiles", 4096, 28672, 256, 1, 2),
     ("wide_two_rows_one_run_two_books", 2048, 2 * 9008, 77, 2, 2),
+    # ... and beyond K = 4096 in pieces of two runs: a last piece that is partly padding, several codebooks, the longest K
+    ("wide_two_rows_long_k_8192_ragged", 8192, 5003, 200, 1, 2),
+    ("wide_two_rows_long_k_14336_down_projection", 14336, 4096, 256, 1, 2),
+    ("wide_two_rows_long_k_4128_padded_piece", 4128, 3000, 256, 1, 2),
+    ("wide_two_rows_long_k_12288_two_books", 12288, 8192, 256, 2, 2),
+    ("wide_two_rows_long_k_16384_longest", 16384, 2048 + 16, 77, 1, 2),
     ("two_rows_four_runs", 8192, 512, 256, 2, 2),
     ("three_rows", 2048, 1024, 256, 1, 3),
     ("four_rows_two_runs", 4096, 1024, 200, 4, 4),
@@ -489,7 +497,7 @@ def test_gemv_kernel_code_formats(row):
 
 def test_gemv_kernel_refuses_other_shapes():
     cb = torch.zeros(256, 8, dtype=torch.float16, device=DEV)
-    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 2056, 64, 8, 8), (1, 34816, 64, 8, 8), (3, 2048, 24, 8, 8), (2, 8192, 24, 8, 8),
+    for (M, K, N, v, bits) in [(5, 2048, 64, 8, 8), (4, 6144, 64, 8, 8), (1, 1024, 64, 8, 8), (1, 2056, 64, 8, 8), (1, 34816, 64, 8, 8), (3, 2048, 24, 8, 8), (2, 18432, 24, 8, 8),
                                (1, 2048, 64, 2, 16), (3, 2048, 64, 4, 8)]:
         x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
         codes = torch.zeros(N, K // v, dtype=torch.uint8 if bits == 8 else torch.uint16, device=DEV)

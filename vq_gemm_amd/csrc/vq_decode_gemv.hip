@@ -21,7 +21,7 @@
 // the wide form below (decode_gemv_wide_kernel) at any N (Tuning::gemv_wide_min_rows_per_wave = 0:
 // with its single-group instance the wide form is ahead from N = 256 on, cold, K = 4096: 2.55
 // against 2.76 us; N = 2048: 2.71 against 2.98; K = 8192, N = 1024: 3.29 against 3.93), and so do
-// two rows of X with K up to 4096 while a wave has few enough rows.
+// two rows of X (K up to 16384) while a wave has few enough rows.
 #include "vq_common.h"
 
 #include <limits.h>
@@ -287,7 +287,8 @@ __device__ __forceinline__ int small_quotient(int x, int d, float rcp)
 //
 // XM: rows of X (1 or 2).  With two, a lane keeps its shares of both rows in registers (RUNS <= 2), every gathered
 // codeword is multiplied with both, and a wave folds and keeps two sums per row of W (cold, M = 2, K = 4096, the
-// K-sliced matrix-core kernel -> this: N = 11008 7.2 -> 5.3 us, N = 28672 10.5 -> 8.7).
+// K-sliced matrix-core kernel -> this: N = 11008 7.2 -> 5.3 us, N = 28672 10.5 -> 8.7).  K beyond 4096 is the long
+// form in pieces of two runs, both rows of x in the LDS (K = 14336, N = 4096: 10.9 -> 8.5 us).
 //
 // XRUNS: runs of 2048 k of x that the LDS holds.  XRUNS == RUNS is the form described so far (K = RUNS * 2048, all of a
 // lane's x in registers).  XRUNS > RUNS is the form for a longer K, or one that is no multiple of 2048 (the
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
     constexpr bool LONG = XRUNS != RUNS;
     static_assert(!LONG || (BOOKS < 2 && COPIES == kWideCopies && NBUF == 2), "the long form: one table, replicated");
     static_assert(NBUF > 1 || G == 1, "a single group per wave: of one row");
-    static_assert(XM == 1 || (XM == 2 && !LONG && RUNS <= 2), "two rows of X: both in the lane's registers, K up to 4096");
+    static_assert(XM == 1 || (XM == 2 && RUNS <= 2), "two rows of X: both in the lane's registers, 4096 k of each at a time");
     const int gated = LONG ? 0 : (gated_row_bytes < 0 ? 1 : 0);
     constexpr int kXChunks = XRUNS * kRunCodes;  // 16-byte pieces of x
     // table of the first codebook (at LDS address 0: a gather address is used as it comes out of the byte
@@ -368,8 +369,11 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         if (second_table) entry1 = reinterpret_cast<const uint4_t *>(cb + (int64_t)min(book0 + 1, n_books - 1) * entries * 8)[ec];
     } else {
 #pragma unroll
-        for (int i = 0; i < kXPerThread; i++)
-            xpiece[i] = reinterpret_cast<const uint4_t *>(x)[min(xt + i * kDutyThreads, (LONG ? J : XM * kXChunks) - 1)];
+        for (int i = 0; i < kXPerThread; i++) {
+            // (the long form: a row of x is J pieces in memory and kXChunks in the LDS)
+            const int xi = xt + i * kDutyThreads, m = XM > 1 && xi >= kXChunks ? 1 : 0;
+            xpiece[i] = reinterpret_cast<const uint4_t *>(x)[LONG ? m * J + min(xi - m * kXChunks, J - 1) : min(xi, XM * kXChunks - 1)];
+        }
     }
 
     // the wave's share [row0, row0 + n_share) of the rows (gated: of the outputs) and its code rows: at most 64, one
@@ -458,7 +462,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
         for (int i = 0; i < kXPerThread; i++) {
             const int xi = xt + i * kDutyThreads;
             // (the long form: zeros behind the end of x, up to whole pieces of rows)
-            if (LONG && xi >= J) xpiece[i] = uint4_t{0u, 0u, 0u, 0u};
+            if (LONG && xi - (XM > 1 && xi >= kXChunks ? kXChunks : 0) >= J) xpiece[i] = uint4_t{0u, 0u, 0u, 0u};
             if (xi < XM * kXChunks) xs[(xi & ~255) + (xi & 3) * 64 + ((xi >> 2) & 63)] = xpiece[i];
         }
     }
@@ -493,8 +497,11 @@ __global__ __launch_bounds__(kWideWaves * 64) void decode_gemv_wide_kernel(const
 #pragma unroll
             for (int m = 0; m < XM; m++) acc[m][r] = 0.f;
             // (the long form: the row's sum over the pieces before this one, zero at the first)
-            if constexpr (LONG)
-                acc[0][r] = lane == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, res[0]), g * G + r)) : 0.f;
+            if constexpr (LONG) {
+#pragma unroll
+                for (int m = 0; m < XM; m++)
+                    acc[m][r] = lane == 0 ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, res[m]), g * G + r)) : 0.f;
+            }
             if constexpr (COPIES == 1) base[r] = TWO && code_row(g * G + r) >= second_book_row ? 4096u : 0u;
             else base[r] = TWO ? copy_base | (code_row(g * G + r) >= second_book_row ? 0x10000u : 0u) : copy_base;
         }
@@ -680,9 +687,18 @@ struct LongK {
 static LongK long_k_form(const ProblemB &p)
 {
     LongK f{false, 0, 0};
+    const int runs_needed = (int)((p.K + kRunK - 1) / kRunK);
+    if (p.M == 2) {
+        // two rows of X: a lane's registers hold two runs of each, so K beyond 4096 goes in pieces of two runs, and
+        // the LDS has room for eight runs of each row beside the table
+        if (p.K % kRunK == 0 && p.K / kRunK <= 2) return f;
+        f.is_long = true;
+        f.runs = 2;
+        f.x_runs = (runs_needed + 1) / 2 * 2 <= 4 ? 4 : 8;
+        return f;
+    }
     if (p.K % kRunK == 0 && p.K / kRunK <= kGemvMaxRuns) return f;
     f.is_long = true;
-    const int runs_needed = (int)((p.K + kRunK - 1) / kRunK);
     const int padded4 = (runs_needed + 3) / 4 * 4, padded3 = (runs_needed + 2) / 3 * 3;
     f.runs = padded3 < padded4 ? 3 : 4;
     f.x_runs = min(padded3, padded4) <= 8 ? 8 : 16;
@@ -720,10 +736,9 @@ bool decode_gemv_wide_supports(const ProblemB &p)
 {
     if (p.M < 1 || p.M > 2 || p.vec != 8 || p.code_bits != 8 || p.entries > 256 || p.packed) return false;
     if (p.K < kRunK || p.N < 1) return false;
-    // two rows of X: both in the lane's registers, K = 2048 or 4096
-    if (p.M == 2 && (long_k_form(p).is_long || p.K / kRunK > 2)) return false;
     if (long_k_form(p).is_long) {
-        if (p.K % 32 != 0 || p.K > 16 * kRunK || p.gated) return false;
+        // (two rows of X: K up to 16384)
+        if (p.K % 32 != 0 || p.K > (p.M == 2 ? 8 : 16) * kRunK || p.gated) return false;
         const int workgroups = wide_workgroups(p);
         if (wide_straddles(p, workgroups)) return false;
         return (p.N + workgroups * kWideWaves - 1) / (workgroups * kWideWaves) <= 64;
@@ -762,6 +777,17 @@ hipError_t launch_decode_gemv_wide(const ProblemB &p, hipStream_t s)
     };
     using std::integral_constant;
     const int g = wide_rows_per_group(p);
+    if (const LongK f = long_k_form(p); p.M == 2 && f.is_long) {
+        auto pick_long2 = [&](auto g_c, auto x_c) {
+            constexpr int GG = decltype(g_c)::value, XR = decltype(x_c)::value;
+            return books == 0 ? launch(decode_gemv_wide_kernel<2, GG, 2, 0, kWideCopies, XR, 2>)
+                              : launch(decode_gemv_wide_kernel<2, GG, 2, 1, kWideCopies, XR, 2>);
+        };
+        auto pick_x2 = [&](auto g_c) {
+            return f.x_runs == 4 ? pick_long2(g_c, integral_constant<int, 4>{}) : pick_long2(g_c, integral_constant<int, 8>{});
+        };
+        return g == 2 ? pick_x2(integral_constant<int, 2>{}) : pick_x2(integral_constant<int, 1>{});
+    }
     if (p.M == 2) {
         // two rows of X against every gathered codeword: the replicated table, one or two groups
         auto pick2 = [&](auto runs_c, auto g_c, auto nbuf_c) {
