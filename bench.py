@@ -50,6 +50,7 @@ PROFILED_TRAFFIC = {
     "decode_m1_k4096_n28672": (14_921_700, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
     "decode_m1_k8192_n28672": (29_657_000, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
     "decode_qkv_m1_k4096_n12288": (6_578_000, "profiles/decode_gemv_wide_kernel_m1_n28672.md"),
+    "decode_m2_k4096_n28672": (15_187_968, "profiles/decode_gemv_wide_kernel_m2_two_rows_of_x.md"),
     "decode_down_m1_k14336_n4096": (7_692_288, "profiles/decode_gemv_wide_kernel_long_k_down_projection.md"),
     "decode_down_m1_k28672_n8192": (29_952_000, "profiles/decode_gemv_wide_kernel_long_k_down_projection.md"),
     "decode_down_m16_k14336_n4096": (11_270_000, "profiles/decode_stream_kernel_m16_k14336_n4096.md"),
