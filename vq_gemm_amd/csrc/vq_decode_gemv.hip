@@ -210,10 +210,10 @@ __global__ __launch_bounds__(kGemvWaves * 64) void decode_gemv_kernel(const half
     }
 }
 
-// ---- the wide form: long runs of rows, long rows, and every single-row launch of the first format -------------------
+// ---- the wide form: long runs of rows, long rows, and every launch of one or two rows of X in the first format -------
 // One workgroup of sixteen waves per compute unit over a bank-replicated table (64 KB: 16 copies of
 // each entry in one 256-byte bank row, lane l reading copy l % 16, so the gathers never collide):
-// four waves per SIMD cover the latency of each other's gathers.  One row of X, 8-vectors, 8-bit codes.
+// four waves per SIMD cover the latency of each other's gathers.  One or two rows of X, 8-vectors, 8-bit codes.
 //   * The rows of W are dealt out to the waves of the whole grid in contiguous runs of equal length
 //     (one more for the first N % waves), so no unit idles while another finishes a longer share.
 //     A workgroup's rows may reach into a second codebook: it then holds two tables (128 KB) and a
