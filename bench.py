@@ -1,6 +1,6 @@
 """Benchmark of the VQ-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only-main]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-traffic] [--only-main]
     python bench.py --launch-floor | --mfma-ceiling | --probe CONFIG     (measurement aids, no JSON)
 
 One "step" is one fused VQ-GEMM launch over one weight matrix.  The headline workload is the
@@ -16,7 +16,9 @@ caches runs between the untimed replay that uploads the graphs and the timed one
 Printed: ONE JSON line (rank 0).  `value` is the decode configuration's effective bandwidth:
 the bytes an uncompressed fp16 GEMV would have had to stream (fp16 weights + X + Y) per
 second.  `roofline` prices the same kernel against HBM peak on its *algorithmic* bytes (codes
-+ codebook + X + Y).  Next to it: the hipBLASLt fp16 GEMM on the dequantised weights timed by
++ codebook + X + Y); its `traffic` is what two `rocprofv3 --pmc` child runs of `--probe C2` count
+after the timed region (FETCH_SIZE and WRITE_SIZE, scaled by a 256 MiB copy; `--skip-traffic`
+leaves them out and reports the committed summary's figure).  Next to it: the hipBLASLt fp16 GEMM on the dequantised weights timed by
 the same loop, the other measured configurations, and the reference math on the host CPU
 (torch gather + fp32 matmul, all cores) on a bounded sample.
 
@@ -59,6 +61,48 @@ PROFILED_TRAFFIC = {
 }
 
 
+def measured_traffic_bytes(probe: str = "C2", kernel: str = "decode_gemv", steps: int = 200):
+    """HBM bytes per launch of `kernel` from two counter runs in child processes (FETCH_SIZE, WRITE_SIZE: KiB per dispatch),
+    each scaled by what the same counter reads for the 256 MiB device copy at the end of the probe.  None when a run fails."""
+    import csv, glob, shutil, statistics, subprocess, tempfile
+    # (not under a profiler: its preloaded library would be inherited by the children)
+    if any("rocprof" in v.lower() for k, v in os.environ.items() if k in ("LD_PRELOAD", "HSA_TOOLS_LIB", "ROCP_TOOL_LIBRARIES")) or \
+            any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ):
+        return None
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    here = os.path.abspath(__file__)
+    total = 0.0
+    detail = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        out = tempfile.mkdtemp(prefix="vq_traffic_", dir="/tmp")
+        try:
+            cmd = [rocprof, "--pmc", counter, "--output-format", "csv", "-d", out, "-o", "p", "--", sys.executable, here,
+                   "--probe", probe, "--steps", str(steps)]
+            res = subprocess.run(cmd, cwd="/tmp", env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.PIPE,
+                                 stderr=subprocess.STDOUT, timeout=90)
+            files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
+            if res.returncode != 0 or not files:
+                return None
+            kern, copy = [], []
+            with open(files[0]) as f:
+                for row in csv.DictReader(f):
+                    if row["Counter_Name"] != counter:
+                        continue
+                    (kern if kernel in row["Kernel_Name"] else copy if "copyBuffer" in row["Kernel_Name"] else []).append(
+                        float(row["Counter_Value"]))
+            if not kern or not copy or max(copy) <= 0:
+                return None
+            factor = 262144.0 / max(copy)     # the copy moves 256 MiB each way: what one counted KiB stands for
+            kib = statistics.median(kern)
+            detail[counter] = {"kib_per_dispatch": kib, "copy_256MiB_reads": max(copy), "factor": factor, "dispatches": len(kern)}
+            total += kib * factor * 1024.0
+        except (OSError, subprocess.SubprocessError):
+            return None
+        finally:
+            shutil.rmtree(out, ignore_errors=True)
+    return int(total), detail
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,6 +110,11 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
+    ap.add_argument("--skip-traffic", action="store_true",
+                    help="do not measure roofline.traffic in this run (two child runs of `rocprofv3 --pmc`, FETCH_SIZE and then "
+                         "WRITE_SIZE, on `bench.py --probe C2`, each scaled by the 256 MiB copy of the same run: about ten "
+                         "seconds); the figure of the committed counter summary is reported instead, as it is when a child "
+                         "run fails or this command itself runs under a profiler")
     ap.add_argument("--probe", metavar="CONFIG", default=None,
                     help="profiling aid (BLAS,C4 = hipBLASLt on the dequantised weights of C4): launch CONFIG (C1..C5, REF = the reference's own shape in its native layout, "
                          "a geometry-B shape M,K,N,vec,entries,code_bits, or GEMM,M,K,N = the plain fp16 GEMM) "
@@ -544,6 +593,11 @@ def main():
     # Every configuration carries the same evidence as the headline: which roofline bounds it, what it achieves against
     # the published peak on its algorithmic bytes or flops (the launch time is this run's, HIP events around replayed
     # graphs), and the HBM traffic a counter run measured (not this run: the summary file is named).
+    if not args.skip_traffic:
+        measured = measured_traffic_bytes()
+        if measured:
+            out["roofline"].update({"traffic": measured[0], "traffic_from": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, child runs of this command",
+                                    "traffic_measured_in_this_run": True, "traffic_counters": measured[1]})
     for name, res in others.items():
         mfma_bound = res["variant"].startswith("prefill")
         traffic = PROFILED_TRAFFIC.get(name)
