@@ -63,7 +63,9 @@ PROFILED_TRAFFIC = {
 
 def measured_traffic_bytes(probe: str = "C2", kernel: str = "decode_gemv", steps: int = 200):
     """HBM bytes per launch of `kernel` from two counter runs in child processes (FETCH_SIZE, WRITE_SIZE: KiB per dispatch),
-    each scaled by what the same counter reads for the 256 MiB device copy at the end of the probe.  None when a run fails."""
+    each scaled by what the same counter reads for the 256 MiB device copy at the end of the probe.  `kernel` = a piece of
+    the kernel's name, or "vq" for every kernel of this library that the probe launches (a launch of several kernels:
+    their sum per launch).  None when a run fails."""
     import csv, glob, shutil, statistics, subprocess, tempfile
     # (not under a profiler: its preloaded library would be inherited by the children)
     if any("rocprof" in v.lower() for k, v in os.environ.items() if k in ("LD_PRELOAD", "HSA_TOOLS_LIB", "ROCP_TOOL_LIBRARIES")) or \
@@ -83,17 +85,22 @@ def measured_traffic_bytes(probe: str = "C2", kernel: str = "decode_gemv", steps
             files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
             if res.returncode != 0 or not files:
                 return None
-            kern, copy = [], []
+            kern, copy, by_name = [], [], {}
             with open(files[0]) as f:
                 for row in csv.DictReader(f):
                     if row["Counter_Name"] != counter:
                         continue
-                    (kern if kernel in row["Kernel_Name"] else copy if "copyBuffer" in row["Kernel_Name"] else []).append(
-                        float(row["Counter_Value"]))
+                    name = row["Kernel_Name"]
+                    if "copyBuffer" in name:
+                        copy.append(float(row["Counter_Value"]))
+                    elif kernel in name and "pack_codes" not in name:
+                        kern.append(float(row["Counter_Value"]))
+                        by_name.setdefault(name, []).append(float(row["Counter_Value"]))
             if not kern or not copy or max(copy) <= 0:
                 return None
             factor = 262144.0 / max(copy)     # the copy moves 256 MiB each way: what one counted KiB stands for
-            kib = statistics.median(kern)
+            # one kernel per launch: the median dispatch; several: each kernel's median times its dispatches per launch
+            kib = sum(statistics.median(v) * max(1, round(len(v) / steps)) for v in by_name.values())
             detail[counter] = {"kib_per_dispatch": kib, "copy_256MiB_reads": max(copy), "factor": factor, "dispatches": len(kern)}
             total += kib * factor * 1024.0
         except (OSError, subprocess.SubprocessError):
@@ -111,10 +118,11 @@ def parse_args():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-main", action="store_true", help="time only the headline decode configuration")
     ap.add_argument("--skip-traffic", action="store_true",
-                    help="do not measure roofline.traffic in this run (two child runs of `rocprofv3 --pmc`, FETCH_SIZE and then "
-                         "WRITE_SIZE, on `bench.py --probe C2`, each scaled by the 256 MiB copy of the same run: about ten "
-                         "seconds); the figure of the committed counter summary is reported instead, as it is when a child "
-                         "run fails or this command itself runs under a profiler")
+                    help="do not measure the roofline objects' traffic in this run (per configuration two child runs of "
+                         "`rocprofv3 --pmc`, FETCH_SIZE and then WRITE_SIZE, on `bench.py --probe <configuration>`, each scaled by "
+                         "the 256 MiB copy of the same run: about half a minute in all); the figures of the committed counter "
+                         "summaries are reported instead, as they are when a child run fails or this command itself runs "
+                         "under a profiler")
     ap.add_argument("--probe", metavar="CONFIG", default=None,
                     help="profiling aid (BLAS,C4 = hipBLASLt on the dequantised weights of C4): launch CONFIG (C1..C5, REF = the reference's own shape in its native layout, "
                          "a geometry-B shape M,K,N,vec,entries,code_bits, or GEMM,M,K,N = the plain fp16 GEMM) "
@@ -610,6 +618,13 @@ def main():
             "traffic": traffic[0] if traffic else None, "traffic_from": traffic[1] if traffic else None,
             "traffic_measured_in_this_run": False, "kernel_us": res["us"],
         }
+        if not args.skip_traffic:
+            probe = name if name in CONFIGS else ",".join(str(v) for v in (res["M"], res["K"], res["N"], res["vec"], res["entries"],
+                                                                            res["code_bits"], res["n_codebooks"]))
+            measured = measured_traffic_bytes(probe, "vq", 20 if mfma_bound else 100)
+            if measured:
+                res["roofline"].update({"traffic": measured[0], "traffic_measured_in_this_run": True, "traffic_counters": measured[1],
+                                        "traffic_from": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, child runs of this command"})
     if others:
         # what the matrix cores sustain on this device with random operands (register-only MFMA loop):
         # the ceiling the MFMA-bound configurations are to be read against, next to the nominal peak
