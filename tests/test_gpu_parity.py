@@ -837,6 +837,45 @@ def test_random_shapes_agree_across_kernels():
     assert done >= 40
 
 
+def test_random_shapes_gemv_forms_against_the_scalar_kernel():
+    """Seeded random launches of one and two rows of X through the GEMV kernels (K in whole runs, in long rows and in
+    rows with a padded last piece; one to many codebooks, workgroups that straddle them, short codebooks; plain, with a
+    bias and gated) against the scalar kernel of the same library, which the tests above pin to the oracle."""
+    import random
+    rnd = random.Random(77)
+    ran = refused = 0
+    for case in range(240):
+        M = rnd.choice([1, 1, 2])
+        K = rnd.choice([2048, 4096, 4096, 6144, 8192, 10240, 14336, 2208, 4128, 11008, 16384, 28672])
+        G = rnd.choice([1, 1, 2, 3, 4, 7, 8, 16, 56])
+        gated = rnd.random() < 0.35
+        unit = 32 if gated else rnd.choice([1, 16, 16, 64])
+        rows_per_cb = unit * rnd.randint(1, max(1, rnd.choice([3000, 9000, 30000]) // (unit * G)))
+        N = G * rows_per_cb
+        if N * K > 150_000_000:
+            continue
+        E = rnd.choice([256, 256, 200, 16])
+        spec = ProblemSpec("rnd_gemv", GEOM_B, M, K, N, 8, E, G, 8, codebook_3d=(G > 1))
+        x, codes, cb = make_problem(spec, seed=1000 + case, device=DEV)
+        bias = (torch.randn(N, generator=torch.Generator().manual_seed(case)) * 0.5).half().to(DEV) if case % 2 else None
+        _say("random gemv", case, spec, "gated" if gated else "", "bias" if bias is not None else "")
+        call = cabi.e2e_gemm_b_gated if gated else cabi.e2e_gemm_b
+        try:
+            y = call(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV, bias=bias)
+        except cabi.VqGemmError as e:
+            assert e.code == -4, e
+            refused += 1
+            continue
+        ref = call(x, codes, cb, variant=cabi.VARIANT_GENERIC, bias=bias).float()
+        torch.cuda.synchronize()
+        err = ((y.float() - ref).abs().max() / max(ref.abs().max().item(), 1e-3)).item()
+        assert err <= TOL, (case, spec, gated, err)
+        assert torch.equal(call(x, codes, cb, variant=cabi.VARIANT_DECODE_GEMV, bias=bias), y)
+        ran += 1
+    _say(f"  {ran} launches compared, {refused} shapes refused")
+    assert ran >= 80
+
+
 def test_every_m_from_1_to_16_on_the_decode_kernel():
     K, N = 1024, 80
     for M in range(1, 17):
