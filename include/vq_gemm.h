@@ -62,8 +62,9 @@ extern "C" {
                                             unit and at most two codebooks per workgroup: the wide form (AUTO takes it
                                             at any N).  Two rows of X in the same form with K = 2048 or 4096, and with
                                             any other multiple of 32 up to 16384 in pieces like the long rows below (AUTO
-                                            takes two rows while a wave's rows of W make at most 22 runs of 2048 k, the
-                                            tuning table's gemv_wide_two_rows_max_runs).  The wide form also takes any other K from
+                                            takes two rows while a wave's rows of W make at most 22 runs of 2048 k, 36
+                                            from K = 8192 on: the tuning table's gemv_wide_two_rows_max_runs and
+                                            ..._long_k).  The wide form also takes any other K from
                                             2048 to 32768 that is a multiple of 32 (a row worked through in pieces of
                                             6144 or 8192 k: the down-projection of an MLP), then not gated and with
                                             every workgroup's rows inside one codebook.  Otherwise the four-wave form: M <= 4 for that

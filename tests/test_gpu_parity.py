@@ -324,7 +324,8 @@ def test_packed_codes_small_shapes_bias_and_rejections():
     assert cabi.select_variant_b(3, 4096, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.select_variant_b(2, 4096, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV   # two rows of X: the wide form ...
     assert cabi.select_variant_b(2, 4096, 65536, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... up to eleven rows per wave at K = 4096
-    assert cabi.select_variant_b(2, 8192, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE        # ... five at K = 8192
+    assert cabi.select_variant_b(2, 8192, 28672, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV   # ... nine at K = 8192
+    assert cabi.select_variant_b(2, 8192, 49152, 8, 256, 1, 8) == cabi.VARIANT_DECODE
     assert cabi.select_variant_b(2, 8192, 8192, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(2, 14336, 4096, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV
     assert cabi.select_variant_b(1, 4096, 32768, 8, 256, 1, 8) == cabi.VARIANT_DECODE_GEMV

@@ -69,6 +69,7 @@ const TuningEntry kTuningEntries[] = {
     {"gemv_wide_min_rows_per_wave", &Tuning::gemv_wide_min_rows_per_wave},
     {"gemv_wide_max_m", &Tuning::gemv_wide_max_m},
     {"gemv_wide_two_rows_max_runs", &Tuning::gemv_wide_two_rows_max_runs},
+    {"gemv_wide_two_rows_max_runs_long_k", &Tuning::gemv_wide_two_rows_max_runs_long_k},
     {"gemv_wide_plain_table_max_runs", &Tuning::gemv_wide_plain_table_max_runs},
     {"gemv_wide_single_rows_max", &Tuning::gemv_wide_single_rows_max},
     {"gemv_wide_rows_per_group", &Tuning::gemv_wide_rows_per_group},

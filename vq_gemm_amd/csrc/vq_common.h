@@ -203,6 +203,7 @@ struct Tuning {
     double gemv_wide_min_rows_per_wave = 0.0;
     double gemv_wide_max_m = 2.0;   // rows of X the automatic choice gives the wide form (it takes one or two)
     double gemv_wide_two_rows_max_runs = 22.0;   // ... two rows of X while a wave's rows are at most this many runs of 2048 k
+    double gemv_wide_two_rows_max_runs_long_k = 36.0;   // ... the same from K = 8192 on
     // the wide form gathers from the plain 4 KB table while a wave's rows are at most this many runs of 2048 k, from the
     // bank-replicated one (64 KB to fill) beyond
     double gemv_wide_plain_table_max_runs = 2.0;

@@ -889,7 +889,9 @@ bool decode_gemv_wide_preferred(const ProblemB &p)
     if (p.M == 2) {
         const int waves = device_cu_count() * kWideWaves;
         const double runs = (double)(((p.gated ? p.N / 2 : p.N) + waves - 1) / waves) * (p.gated ? 2 : 1) * (double)(p.K / kRunK);
-        if (runs > tuning().gemv_wide_two_rows_max_runs) return false;
+        // (K from 8192 on the K-sliced kernels walk K in chunks and fall behind later: K = 8192, 28 runs per wave 17.3
+        // against 18.9 us, 32 runs 19.8 against 20.6, 40 runs 23.0 against 23.2; K = 14336, 35 runs 23.3 against 27.6)
+        if (runs > (p.K >= 4 * kRunK ? tuning().gemv_wide_two_rows_max_runs_long_k : tuning().gemv_wide_two_rows_max_runs)) return false;
     }
     return decode_gemv_wide_supports(p) && (double)p.M <= tuning().gemv_wide_max_m &&
            (double)(p.gated ? p.N / 2 : p.N) >= tuning().gemv_wide_min_rows_per_wave * kWideWaves * device_cu_count();
